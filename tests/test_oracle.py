@@ -1,0 +1,424 @@
+"""Pins the CPU oracle against independent routines (torch CPU, numpy closed
+forms, hand-computed values from the reference's own tests) so that a dropped
+term, a wrong sign/index or a transposed operand fails here."""
+import numpy as np
+import pytest
+import torch
+import torch.nn.functional as F
+
+import oracle
+
+rng = np.random.default_rng(1234)
+
+
+def small_ints(shape, lo=-3, hi=4):
+    return rng.integers(lo, hi, size=shape).astype(np.float32)
+
+
+CONV_CASES = [
+    # n, c, h, w, f, cpg, r, s, ph, pw, sh, sw, dh, dw
+    (1, 4, 9, 9, 6, 4, 3, 3, 1, 1, 1, 1, 1, 1),
+    (2, 3, 12, 10, 5, 3, 3, 3, 0, 0, 1, 1, 1, 1),
+    (1, 4, 11, 13, 8, 4, 3, 3, 1, 1, 2, 2, 1, 1),
+    (1, 8, 12, 12, 8, 8, 3, 3, 2, 2, 1, 1, 2, 2),      # dilated, CSRNet-style
+    (1, 8, 10, 10, 12, 2, 3, 3, 1, 1, 1, 1, 1, 1),     # groups = 4
+    (2, 6, 8, 8, 6, 1, 3, 3, 1, 1, 1, 1, 1, 1),        # depthwise
+    (1, 5, 14, 14, 7, 5, 1, 1, 0, 0, 2, 2, 1, 1),      # 1x1 / s2 downsample
+    (1, 3, 20, 20, 4, 3, 7, 7, 3, 3, 2, 2, 1, 1),      # 7x7 / s2 stem
+    (1, 2, 9, 15, 3, 2, 1, 3, 0, 1, 1, 1, 1, 1),       # 1xk kernel
+    (1, 2, 9, 15, 3, 2, 3, 1, 2, 0, 1, 2, 1, 1),       # asymmetric pads / strides
+    (1, 2, 16, 16, 2, 2, 5, 5, 2, 2, 1, 1, 1, 1),
+]
+
+
+@pytest.mark.parametrize("case", CONV_CASES)
+def test_conv2d_vs_torch(case):
+    n, c, h, w, f, cpg, r, s, ph, pw, sh, sw, dh, dw = case
+    x = small_ints((n, c, h, w))
+    wt = small_ints((f, cpg, r, s))
+    ref = F.conv2d(torch.from_numpy(x).double(), torch.from_numpy(wt).double(),
+                   padding=(ph, pw), stride=(sh, sw), dilation=(dh, dw),
+                   groups=c // cpg).numpy()
+    got = oracle.conv2d(x, wt, ph, pw, sh, sw, dh, dw)
+    assert got.shape == ref.shape
+    np.testing.assert_array_equal(got.astype(np.float64), ref)
+    # uint32 tier: two's-complement view of the same integers
+    gu = oracle.conv2d(x.astype(np.int64).astype(np.uint32),
+                       wt.astype(np.int64).astype(np.uint32), ph, pw, sh, sw,
+                       dh, dw)
+    np.testing.assert_array_equal(gu.view(np.int32).astype(np.float64), ref)
+
+
+def test_conv2d_hand_values_no_kernel_flip():
+    x = np.array([1, 2, 3, 4], np.float32).reshape(1, 1, 1, 4)
+    w = np.array([1, 10, 100], np.float32).reshape(1, 1, 1, 3)
+    y = oracle.conv2d(x, w, 0, 1)
+    np.testing.assert_array_equal(y.ravel(), [210, 321, 432, 43])
+
+
+def test_conv2d_float_tier_vs_torch_double():
+    x = rng.uniform(-1, 1, (1, 16, 14, 14)).astype(np.float32)
+    w = rng.uniform(-1, 1, (8, 16, 3, 3)).astype(np.float32)
+    ref = F.conv2d(torch.from_numpy(x).double(), torch.from_numpy(w).double(),
+                   padding=1).numpy()
+    got = oracle.conv2d(x, w, 1, 1)
+    np.testing.assert_allclose(got, ref, rtol=1e-6, atol=1e-6)
+
+
+def test_conv2d_u32_wraps_like_uint32():
+    x = oracle.fastrand(2 * 5 * 5, seed=3, mod=0).reshape(1, 2, 5, 5) * np.uint32(70001)
+    w = oracle.fastrand(3 * 2 * 3 * 3, seed=5, mod=0).reshape(3, 2, 3, 3) * np.uint32(90001)
+    got = oracle.conv2d(x, w, 1, 1)
+    xp = np.pad(x.astype(object), ((0, 0), (0, 0), (1, 1), (1, 1)))
+    for f in range(3):
+        for i in range(5):
+            for j in range(5):
+                acc = 0
+                for c in range(2):
+                    for r in range(3):
+                        for s in range(3):
+                            acc += int(w[f, c, r, s]) * int(xp[0, c, i + r, j + s])
+                assert int(got[0, f, i, j]) == acc % (1 << 32)
+
+
+def test_conv_out_dim_rule():
+    # textbook cases
+    assert oracle.conv_out_dim(224, 7, 3, 2, 1) == 112
+    assert oracle.conv_out_dim(56, 1, 0, 2, 1) == 28
+    assert oracle.conv_out_dim(56, 3, 1, 2, 1) == 28
+    assert oracle.conv_out_dim(64, 3, 2, 1, 2) == 64
+    # the reference's formula differs from the textbook one when d>1 and s>1:
+    # (i - (k - s) d + 2p) / s = (17 - 2 + 0) / 2 = 7, textbook gives 7 too for
+    # i=17 but 6 for i=16 -> reference (16 - 2)/2 = 7.
+    assert oracle.conv_out_dim(16, 3, 0, 2, 2) == 7
+    assert (16 + 0 - 2 * (3 - 1) - 1) // 2 + 1 == 6
+
+
+def test_conv_reference_shape_quirk_reads_zero_outside():
+    x = small_ints((1, 1, 16, 16))
+    w = small_ints((1, 1, 3, 3))
+    y = oracle.conv2d(x, w, 0, 0, 2, 2, 2, 2)
+    assert y.shape == (1, 1, 7, 7)
+    xp = np.pad(x, ((0, 0), (0, 0), (0, 4), (0, 4)))
+    ref = F.conv2d(torch.from_numpy(xp).double(), torch.from_numpy(w).double(),
+                   stride=2, dilation=2).numpy()[:, :, :7, :7]
+    np.testing.assert_array_equal(y.astype(np.float64), ref)
+
+
+def test_conv2d_invalid_groups_returns_none():
+    # f % g != 0 -> nullptr (src/Graph/operator.cc:108-109)
+    x = small_ints((1, 4, 5, 5))
+    w = small_ints((3, 2, 3, 3))
+    assert oracle.conv2d(x, w, 1, 1) is None
+
+
+def test_conv2d_full_equals_pointwise():
+    # src/Test/conv_test_3.cc: iota inputs, every output point
+    n, c, h, w, f, r, s = 2, 4, 6, 6, 5, 3, 3
+    x = np.arange(n * c * h * w, dtype=np.uint32).reshape(n, c, h, w)
+    wt = np.arange(f * c * r * s, dtype=np.uint32).reshape(f, c, r, s)
+    full = oracle.conv2d(x, wt, 1, 1)
+    for pos in np.ndindex(*full.shape):
+        assert oracle.conv2d_point(x, wt, 1, 1, 1, 1, 1, 1, pos) == full[pos]
+
+
+def test_conv3d_reduces_to_conv2d_and_matches_torch():
+    x = small_ints((1, 3, 1, 8, 8))
+    w = small_ints((4, 3, 1, 3, 3))
+    y3 = oracle.conv3d(x, w, (0, 1, 1))
+    y2 = oracle.conv2d(x[:, :, 0], w[:, :, 0], 1, 1)
+    np.testing.assert_array_equal(y3[:, :, 0], y2)
+    for (pad, st, dl, g) in [((1, 1, 1), (1, 1, 1), (1, 1, 1), 1),
+                             ((1, 3, 3), (1, 2, 2), (1, 1, 1), 1),
+                             ((1, 1, 1), (2, 2, 2), (1, 1, 1), 1),
+                             ((2, 2, 2), (1, 1, 1), (2, 2, 2), 2)]:
+        x = small_ints((2, 4, 6, 9, 10))
+        kt = 3
+        kh = 7 if pad[1] == 3 else 3
+        w = small_ints((6, 4 // g, kt, kh, kh))
+        ref = F.conv3d(torch.from_numpy(x).double(), torch.from_numpy(w).double(),
+                       padding=pad, stride=st, dilation=dl, groups=g).numpy()
+        got = oracle.conv3d(x, w, pad, st, dl)
+        np.testing.assert_array_equal(got.astype(np.float64), ref)
+
+
+@pytest.mark.parametrize("tA", [False, True])
+@pytest.mark.parametrize("tB", [False, True])
+def test_matmul_vs_numpy(tA, tB):
+    b, m, n, k = 3, 5, 7, 4
+    A = small_ints((b, k, m) if tA else (b, m, k))
+    B = small_ints((b, n, k) if tB else (b, k, n))
+    ref = np.matmul(A.transpose(0, 2, 1) if tA else A,
+                    B.transpose(0, 2, 1) if tB else B)
+    np.testing.assert_array_equal(oracle.matmul(A, B, tA, tB), ref)
+    Au = A.astype(np.int64).astype(np.uint32)
+    Bu = B.astype(np.int64).astype(np.uint32)
+    np.testing.assert_array_equal(
+        oracle.matmul(Au, Bu, tA, tB).view(np.int32), ref.astype(np.int32))
+
+
+def test_matmul_batch_gemm_test_values():
+    # src/Test/batch_gemm_test.cc:10,45-50: m=n=8, k=4, A=iota, W0=3*iota, W1=7*iota
+    m, n, k = 8, 8, 4
+    A = np.arange(m * k, dtype=np.uint32).reshape(1, m, k)
+    W0 = (3 * np.arange(k * n, dtype=np.uint32)).reshape(1, k, n)
+    W1 = (7 * np.arange(k * n, dtype=np.uint32)).reshape(1, k, n)
+    o0 = oracle.matmul(A, W0)
+    o1 = oracle.matmul(A, W1)
+    # o0[0,0,0] = sum_k k * 3 * 8k = 24 * (0+1+4+9)
+    assert o0[0, 0, 0] == 336
+    # o1[0,1,3] = sum_k (4+k) * 7 * (8k+3)
+    assert o1[0, 1, 3] == sum((4 + kk) * 7 * (8 * kk + 3) for kk in range(4))
+    # the merged program: concat lhs twice, concat rhs, bmm, split on dim 0
+    l2 = oracle.concat([A, A], 0)
+    r2 = oracle.concat([W0, W1], 0)
+    a0, a1 = oracle.split(oracle.matmul(l2, r2), 0, sizes=[1, 1])
+    np.testing.assert_array_equal(a0, o0)
+    np.testing.assert_array_equal(a1, o1)
+
+
+def test_transpose_closed_forms_from_reference_tests():
+    # src/Test/transpose_test_2.py:4-31
+    i0 = np.arange(64, dtype=np.uint32).reshape(1, 1, 8, 8)
+    d2h = i0.reshape(1, 1, 4, 2, 8).transpose(0, 1, 3, 2, 4).reshape(1, 1, 8, 8)
+    got = oracle.transpose(i0, 2, [0, 1, [-1, 2], 3], 2)      # D2H, factor 2
+    np.testing.assert_array_equal(got, d2h)
+    back = d2h.reshape(1, 1, 2, 4, 8).transpose(0, 1, 3, 2, 4).reshape(1, 1, 8, 8)
+    got_back = oracle.transpose(d2h, 2, [0, 1, [-1, 2], 3], -2)
+    np.testing.assert_array_equal(got_back, back)
+    np.testing.assert_array_equal(got_back, i0)
+
+    i0 = np.arange(32, dtype=np.uint32).reshape(2, 1, 4, 4)
+    n2h = i0.reshape(1, 2, 1, 4, 4).transpose(0, 2, 1, 3, 4).reshape(1, 1, 8, 4)
+    got = oracle.transpose(i0, 0, [0, 1, [-1, 2], 3], 2)      # N2H
+    np.testing.assert_array_equal(got, n2h)
+    h2n = n2h.reshape(1, 1, 2, 4, 4).transpose(0, 2, 1, 3, 4).reshape(2, 1, 4, 4)
+    got = oracle.transpose(n2h, 2, [[0, 2], 1, -1, 3], -2)    # H2N
+    np.testing.assert_array_equal(got, h2n)
+    np.testing.assert_array_equal(got, i0)
+
+
+def test_transpose_ops_file_case():
+    # src/Test/dat/transpose_test/transpose_ops.op with transpose_test_1.cc:11-27
+    n, c, h, w = 16, 16, 32, 32
+    x = rng.integers(0, 10, (n, c, h, w)).astype(np.uint32)
+    ref = x.reshape(-1, 2, 16, 32, 32).transpose(0, 2, 1, 3, 4).reshape(8, 16, -1, 32)
+    got = oracle.transpose(x, 0, [0, 1, [-1, 2], 3], 2)
+    np.testing.assert_array_equal(got, ref)
+
+
+def test_transpose_other_catalogue_entries():
+    x = rng.integers(0, 100, (4, 6, 8, 10)).astype(np.uint32)
+    # N2W / W2N (src/Mutant/generator.cc:1033-1036)
+    n2w = oracle.transpose(x, 0, [0, 1, 2, [-1, 3]], 2)
+    ref = x.reshape(2, 2, 6, 8, 10).transpose(0, 2, 3, 1, 4).reshape(2, 6, 8, 20)
+    np.testing.assert_array_equal(n2w, ref)
+    w2n = oracle.transpose(n2w, 3, [[0, 3], 1, 2, -1], -2)
+    np.testing.assert_array_equal(w2n, x)
+    # C2H (:1039-1040)
+    c2h = oracle.transpose(x, 1, [0, 1, [2, -1], 3], 2)
+    ref = x.reshape(4, 3, 2, 8, 10).transpose(0, 1, 3, 2, 4).reshape(4, 3, 16, 10)
+    np.testing.assert_array_equal(c2h, ref)
+    # plain permutes (:1101, :1153)
+    np.testing.assert_array_equal(oracle.transpose(x, -1, [0, 1, 3, 2]),
+                                  x.transpose(0, 1, 3, 2))
+    y = rng.integers(0, 100, (3, 5, 7)).astype(np.uint32)
+    np.testing.assert_array_equal(oracle.transpose(y, -1, [0, 2, 1]),
+                                  y.transpose(0, 2, 1))
+    # not divisible -> nullptr
+    assert oracle.transpose(x[:3], 0, [0, 1, [-1, 2], 3], 2) is None
+
+
+def test_transpose_float_tier_is_a_copy():
+    x = rng.standard_normal((2, 3, 4, 6)).astype(np.float32)
+    got = oracle.transpose(x, 2, [[0, 2], 1, -1, 3], -2)
+    ref = x.reshape(2, 3, 2, 2, 6).transpose(0, 2, 1, 3, 4).reshape(4, 3, 2, 6)
+    assert got.tobytes() == np.ascontiguousarray(ref).tobytes()
+
+
+def test_split_concat_pad_slice_extend_vs_numpy():
+    x = rng.integers(0, 1000, (2, 6, 4, 5)).astype(np.uint32)
+    for dim in range(4):
+        if x.shape[dim] % 2 == 0:
+            outs = oracle.split(x, dim, num=2)
+            for a, b in zip(outs, np.split(x, 2, axis=dim)):
+                np.testing.assert_array_equal(a, b)
+            np.testing.assert_array_equal(oracle.concat(outs, dim), x)
+    # ratio rule: sizes are proportions of the dim (operator.cc:2085-2094)
+    o = oracle.split(x, 1, sizes=[1, 2])
+    assert [t.shape[1] for t in o] == [2, 4]
+    np.testing.assert_array_equal(o[0], x[:, :2])
+    np.testing.assert_array_equal(o[1], x[:, 2:])
+    assert oracle.split(x, 1, sizes=[1, 3]) is None
+    # concat of unequal parts and repeated inputs
+    y = oracle.concat([x[:, :1], x[:, :4], x[:, :1]], 1)
+    np.testing.assert_array_equal(y, np.concatenate([x[:, :1], x[:, :4], x[:, :1]], 1))
+    b, e = [0, 1, 2, 0], [1, 0, 1, 3]
+    np.testing.assert_array_equal(oracle.pad(x, b, e),
+                                  np.pad(x, list(zip(b, e))))
+    xs = oracle.slice_(x, [0, 1, 1, 2], [1, 2, 0, 1])
+    np.testing.assert_array_equal(xs, x[0:1, 1:4, 1:4, 2:4])
+    assert oracle.slice_(x, [2, 0, 0, 0], [1, 0, 0, 0]) is None
+    for dim in range(4):
+        reps = [1, 1, 1, 1]
+        reps[dim] = 3
+        np.testing.assert_array_equal(oracle.extend(x, dim, 2), np.tile(x, reps))
+
+
+def test_pad_conv_slice_identity():
+    # src/Test/pad_slice_test.cc idea: pad -> conv -> slice == conv on odd sizes
+    x = small_ints((1, 3, 7, 7))
+    w = small_ints((4, 3, 3, 3))
+    ref = oracle.conv2d(x, w, 1, 1)
+    xp = oracle.pad(x, [0, 0, 0, 0], [0, 0, 1, 1])
+    y = oracle.slice_(oracle.conv2d(xp, w, 1, 1), [0, 0, 0, 0], [0, 0, 1, 1])
+    np.testing.assert_array_equal(y, ref)
+
+
+def test_eltwise_flat_modulo_broadcast():
+    a = np.arange(24, dtype=np.uint32).reshape(2, 3, 4)
+    b = np.array([10, 20, 30, 40], dtype=np.uint32)
+    c = np.arange(12, dtype=np.uint32).reshape(3, 4) * 100
+    idx = np.arange(24)
+    ref = (a.ravel() + b[idx % 4] + c.ravel()[idx % 12]).reshape(2, 3, 4)
+    np.testing.assert_array_equal(oracle.eltwise("add", [a, b, c], (2, 3, 4)), ref)
+    ref = (a.ravel() * b[idx % 4]).reshape(2, 3, 4)
+    np.testing.assert_array_equal(oracle.eltwise("mul", [a, b], (2, 3, 4)), ref)
+    ref = (a.ravel() - b[idx % 4]).reshape(2, 3, 4)       # wraps below zero
+    np.testing.assert_array_equal(oracle.eltwise("sub", [a, b], (2, 3, 4)), ref)
+    # a size that does not divide: still i % size (include/tensor.h:257-260)
+    d = np.array([1, 2, 3, 4, 5], dtype=np.uint32)
+    ref = (a.ravel() + d[idx % 5]).reshape(2, 3, 4)
+    np.testing.assert_array_equal(oracle.eltwise("add", [a, d], (2, 3, 4)), ref)
+
+
+def test_trans_chain_plain_equals_transpose():
+    x = rng.integers(0, 1000, (2, 3, 8, 5)).astype(np.uint32)
+    # H2N as micro-ops (TransposeOp::getTTParam, operator.cc:2436-2455)
+    got = oracle.trans_chain(x, [("split", 2, 4, 0, 0),
+                                 ("reorder", [0, 2, 1, 3, 4]),
+                                 ("fuse", 0, 0, 0)])
+    np.testing.assert_array_equal(
+        got, oracle.transpose(x, 2, [[0, 2], 1, -1, 3], -2))
+
+
+def test_trans_chain_halo_split_and_drop_fuse():
+    n, c, h, w, p = 1, 2, 8, 5, 1
+    x = np.arange(n * c * h * w, dtype=np.uint32).reshape(n, c, h, w) + 1
+    half = h // 2
+    # split with copys: rows a*in + b - a*copys (transpose.cc:33-40)
+    halo = oracle.trans_chain(x, [("split", 2, half, 0, p),
+                                  ("reorder", [0, 2, 1, 3, 4]),
+                                  ("fuse", 0, 0, 0)])
+    assert halo.shape == (2, c, half + p, w)
+    np.testing.assert_array_equal(halo[0], x[0, :, :half + p])
+    np.testing.assert_array_equal(halo[1], x[0, :, half - p:])
+    # inverse with dels: (a // (in-dels), a % (in-dels) + (a // (in-dels)) * dels)
+    # (transpose.cc:75-88)
+    back = oracle.trans_chain(halo, [("split", 0, 2, 0, 0),
+                                     ("reorder", [0, 2, 1, 3, 4]),
+                                     ("fuse", 2, 0, p)])
+    np.testing.assert_array_equal(back, x)
+
+
+def test_trans_chain_corrected_h2n_conv_equals_conv():
+    # config-1 shape family, small: conv == halo-split -> conv -> drop-fuse
+    x = small_ints((1, 3, 12, 7))
+    w = small_ints((4, 3, 3, 3))
+    ref = oracle.conv2d(x, w, 1, 1)
+    halo = oracle.trans_chain(x, [("split", 2, 6, 0, 1),
+                                  ("reorder", [0, 2, 1, 3, 4]),
+                                  ("fuse", 0, 0, 0)])
+    y = oracle.conv2d(halo, w, 1, 1)
+    out = oracle.trans_chain(y, [("split", 0, 2, 0, 0),
+                                 ("reorder", [0, 2, 1, 3, 4]),
+                                 ("fuse", 2, 0, 1)])
+    np.testing.assert_array_equal(out, ref)
+    # without correction the seam rows differ (why PET calls it partially equivalent)
+    plain = oracle.transpose(
+        oracle.conv2d(oracle.transpose(x, 2, [[0, 2], 1, -1, 3], -2), w, 1, 1),
+        0, [0, 1, [-1, 2], 3], 2)
+    assert plain.shape == ref.shape
+    assert not np.array_equal(plain, ref)
+    np.testing.assert_array_equal(plain[:, :, :5], ref[:, :, :5])
+
+
+def test_trans_chain_pad_fuse_and_extr_split():
+    # N2H with zero rows between merged images (transpose.cc:89-105) and the
+    # inverse split with stride in+extr (transpose.cc:27-32)
+    x = np.arange(2 * 2 * 3 * 4, dtype=np.uint32).reshape(2, 2, 3, 4) + 1
+    pad = 1
+    y = oracle.trans_chain(x, [("split", 0, 2, 0, 0),
+                               ("reorder", [0, 2, 1, 3, 4]),
+                               ("fuse", 2, pad, 0)])
+    assert y.shape == (1, 2, 2 * (3 + pad) - pad, 4)
+    np.testing.assert_array_equal(y[0, :, 0:3], x[0])
+    np.testing.assert_array_equal(y[0, :, 3], 0)
+    np.testing.assert_array_equal(y[0, :, 4:7], x[1])
+    back = oracle.trans_chain(y, [("split", 2, 3, pad, 0),
+                                  ("reorder", [0, 2, 1, 3, 4]),
+                                  ("fuse", 0, 0, 0)])
+    np.testing.assert_array_equal(back, x)
+
+
+def test_space_to_batch_dilated_conv_equivalence():
+    # dilation == padding, stride 1 (src/nnet/nmutator.cc:529-567): the dilated
+    # conv equals a dense conv on the d*d phase images
+    d = 2
+    x = small_ints((1, 3, 8, 8))
+    w = small_ints((4, 3, 3, 3))
+    ref = oracle.conv2d(x, w, d, d, 1, 1, d, d)
+    s2b = oracle.permute_flat(x, [1, 3, 4, d, 4, d], [3, 5, 0, 1, 2, 4])
+    s2b = s2b.reshape(d * d, 3, 4, 4)
+    y = oracle.conv2d(s2b, w, 1, 1)
+    b2s = oracle.permute_flat(y, [d, d, 1, 4, 4, 4], [2, 3, 4, 0, 5, 1])
+    np.testing.assert_array_equal(b2s.reshape(1, 4, 8, 8), ref)
+
+
+def test_fastrand_stream():
+    # include/tensor.h:371-374 is the classic 214013 / 2531011 LCG; from seed 0
+    # its first outputs are 38, 7719, 21238 (computed here independently).
+    g, exp = 0, []
+    for _ in range(5):
+        g = (214013 * g + 2531011) & 0xFFFFFFFF
+        exp.append((g >> 16) & 0x7FFF)
+    assert exp[:3] == [38, 7719, 21238]
+    np.testing.assert_array_equal(oracle.fastrand(5, 0, 0), exp)
+    np.testing.assert_array_equal(oracle.fastrand(5, 0, 10000),
+                                  [e % 10000 for e in exp])
+
+
+def test_unpinned_float_pieces_vs_torch():
+    x = rng.standard_normal((2, 3, 9, 9)).astype(np.float32)
+    xt = torch.from_numpy(x)
+    np.testing.assert_array_equal(oracle.activation(x, "relu"), np.maximum(x, 0))
+    np.testing.assert_allclose(oracle.activation(x, "sigmoid"),
+                               torch.sigmoid(xt.double()).float().numpy(), rtol=1e-6)
+    np.testing.assert_allclose(oracle.activation(x, "tanh"),
+                               torch.tanh(xt.double()).float().numpy(), rtol=1e-6)
+    np.testing.assert_allclose(oracle.activation(x, "gelu"),
+                               F.gelu(xt.double()).float().numpy(), rtol=1e-6, atol=1e-7)
+    b = rng.standard_normal(3).astype(np.float32)
+    np.testing.assert_array_equal(oracle.bias_act(x, b, "relu"),
+                                  np.maximum(x + b[None, :, None, None], 0))
+    np.testing.assert_array_equal(
+        oracle.pool2d(x, 3, 3, 1, 1, 2, 2, mode="max"),
+        F.max_pool2d(xt, 3, 2, 1).numpy())
+    np.testing.assert_allclose(
+        oracle.pool2d(x, 3, 3, 1, 1, 2, 2, mode="avg"),
+        F.avg_pool2d(xt, 3, 2, 1, count_include_pad=True).numpy(), rtol=1e-6,
+        atol=1e-7)
+    np.testing.assert_allclose(
+        oracle.pool2d(x, 9, 9, 0, 0, 1, 1, mode="avg"),
+        x.mean(axis=(2, 3), keepdims=True), rtol=1e-5, atol=1e-7)
+    s = rng.standard_normal((5, 17)).astype(np.float32)
+    np.testing.assert_allclose(oracle.softmax(s),
+                               torch.softmax(torch.from_numpy(s).double(), -1).float().numpy(),
+                               rtol=1e-6)
+    g = rng.standard_normal(17).astype(np.float32)
+    be = rng.standard_normal(17).astype(np.float32)
+    np.testing.assert_allclose(
+        oracle.layernorm(s, g, be, 1e-5),
+        F.layer_norm(torch.from_numpy(s).double(), (17,), torch.from_numpy(g).double(),
+                     torch.from_numpy(be).double(), 1e-5).float().numpy(),
+        rtol=1e-5, atol=1e-6)
