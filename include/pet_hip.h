@@ -1,0 +1,232 @@
+/*
+ * pet_hip.h -- C ABI of the MI355X (gfx950) execution backend for PET tensor
+ * programs. Every entry point is extern "C", takes plain pointers and sizes,
+ * returns 0 on success and a non-zero pet_hip_status otherwise (no exceptions,
+ * no exit() across the boundary). Device pointers are caller-owned; no call
+ * here copies between host and device except the explicit memcpy functions,
+ * and none retains a caller pointer after it returns.
+ *
+ * Citations name the reference interface (thu-pacman/PET) that each entry
+ * point replaces, as path:line.
+ *
+ * All tensors are fp32, row-major, contiguous.
+ */
+#ifndef PET_HIP_H
+#define PET_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define PET_HIP_MAX_RANK 8
+
+#if defined(__GNUC__)
+#define PET_HIP_API __attribute__((visibility("default")))
+#else
+#define PET_HIP_API
+#endif
+
+typedef enum pet_hip_status {
+    PET_HIP_OK = 0,
+    PET_HIP_ERR_INVALID = 1,     /* bad argument / shape the op rejects (reference: compute() == nullptr) */
+    PET_HIP_ERR_UNSUPPORTED = 2, /* valid but not implemented (reference: perf() == INFINITY) */
+    PET_HIP_ERR_RUNTIME = 3,     /* a HIP call failed; see pet_hip_last_error() */
+    PET_HIP_ERR_NOT_INIT = 4
+} pet_hip_status;
+
+/* Operator::ActType, include/operator.h:95-100, plus GELU (absent upstream). */
+typedef enum pet_hip_act {
+    PET_HIP_ACT_NONE = 0,
+    PET_HIP_ACT_RELU = 1,
+    PET_HIP_ACT_SIGMOID = 2,
+    PET_HIP_ACT_TANH = 3,
+    PET_HIP_ACT_GELU = 4
+} pet_hip_act;
+
+typedef enum pet_hip_eltwise_op {
+    PET_HIP_ADD = 0, /* AddOp::compute, src/Graph/operator.cc:2983-3002 */
+    PET_HIP_SUB = 1, /* SubOp::compute, src/Graph/operator.cc:3074-3090 */
+    PET_HIP_MUL = 2  /* MulOp::compute, src/Graph/operator.cc:3157-3176 */
+} pet_hip_eltwise_op;
+
+/* Opaque handles (a hipStream_t / hipEvent_t / hipGraphExec_t underneath). */
+typedef void *pet_hip_stream_t;
+typedef void *pet_hip_event_t;
+typedef void *pet_hip_graph_t;
+
+/* ---- context --------------------------------------------------------------
+ * Replaces the cudnnCreate / cublasCreate / cudaMalloc block of
+ * PerfEngine::PerfEngine and PerfEngine::allocMem (include/perf_engine.h:41-45,
+ * src/Graph/perf_engine.cc:31-56) and checkCudaError (include/common.h:30-38). */
+PET_HIP_API int pet_hip_init(int device);
+PET_HIP_API int pet_hip_shutdown(void);
+PET_HIP_API const char *pet_hip_last_error(void);
+/* name of the device's architecture ("gfx950") and number of compute units */
+PET_HIP_API int pet_hip_device_info(char *arch, size_t arch_len, int *num_cu);
+
+/* ---- memory (cudaMalloc / cudaMemcpy / cudaFree call sites,
+ * src/Graph/perf_engine.cc:31-47, src/Graph/code_engine.cc:560-643) ---------- */
+PET_HIP_API int pet_hip_malloc(void **dptr, size_t bytes);
+PET_HIP_API int pet_hip_free(void *dptr);
+PET_HIP_API int pet_hip_memcpy_h2d(void *dst, const void *src, size_t bytes, pet_hip_stream_t s);
+PET_HIP_API int pet_hip_memcpy_d2h(void *dst, const void *src, size_t bytes, pet_hip_stream_t s);
+PET_HIP_API int pet_hip_memcpy_d2d(void *dst, const void *src, size_t bytes, pet_hip_stream_t s);
+/* fills n floats with value through a kernel (safe under graph capture) */
+PET_HIP_API int pet_hip_fill_f32(float *dst, float value, size_t n, pet_hip_stream_t s);
+/* uniform [lo, hi) fill from a counter-based generator, replaces
+ * curandGenerateUniform (src/Graph/perf_engine.cc:49-55, code_engine.cc:582) */
+PET_HIP_API int pet_hip_rand_uniform_f32(float *dst, size_t n, uint64_t seed, float lo, float hi,
+                             pet_hip_stream_t s);
+
+/* ---- streams, events, graphs ---------------------------------------------
+ * Replace cudaDeviceSynchronize + std::chrono timing in Operator::perf
+ * (src/Graph/operator.cc:416-467) and the cudaEvent bracket of the emitted
+ * program (src/Graph/code_engine.cc:180-217). */
+PET_HIP_API int pet_hip_stream_create(pet_hip_stream_t *s);
+PET_HIP_API int pet_hip_stream_destroy(pet_hip_stream_t s);
+PET_HIP_API int pet_hip_stream_sync(pet_hip_stream_t s);
+PET_HIP_API int pet_hip_event_create(pet_hip_event_t *e);
+PET_HIP_API int pet_hip_event_destroy(pet_hip_event_t e);
+PET_HIP_API int pet_hip_event_record(pet_hip_event_t e, pet_hip_stream_t s);
+PET_HIP_API int pet_hip_event_sync(pet_hip_event_t e);
+PET_HIP_API int pet_hip_event_elapsed_ms(float *ms, pet_hip_event_t start, pet_hip_event_t stop);
+/* Capture every launch issued on `s` between begin and end into an executable
+ * graph; replaces the per-iteration op list of the emitted main()
+ * (src/Graph/code_engine.cc:194-215). */
+PET_HIP_API int pet_hip_graph_begin_capture(pet_hip_stream_t s);
+PET_HIP_API int pet_hip_graph_end_capture(pet_hip_stream_t s, pet_hip_graph_t *g);
+PET_HIP_API int pet_hip_graph_launch(pet_hip_graph_t g, pet_hip_stream_t s);
+PET_HIP_API int pet_hip_graph_destroy(pet_hip_graph_t g);
+
+/* ---- contractions ---------------------------------------------------------*/
+
+/* ConvOp::computeShape with explicit padding, src/Graph/operator.cc:219-221:
+ * o = (i - (k - s) * d + 2 p) / s. */
+PET_HIP_API int pet_hip_conv_out_dim(int i, int k, int p, int s, int d);
+
+/* Conv2d, NCHW x [n,c,h,w], weight [f, c/groups, r, s], y [n,f,oh,ow] with
+ * oh/ow from pet_hip_conv_out_dim. Cross-correlation, zero padding, group of
+ * output channel ff is ff / (f / groups). bias (may be NULL) is [f]; act is a
+ * pet_hip_act. Semantics: ConvOp::compute, src/Graph/operator.cc:94-158;
+ * replaces cudnnConvolutionForward / cudnnConvolutionBiasActivationForward
+ * (src/Graph/operator.cc:425-427, 478-481; src/Graph/code_engine.cc:869-977).
+ * Returns PET_HIP_ERR_INVALID when c % (c/groups) or f % groups != 0. */
+PET_HIP_API int pet_hip_conv2d_f32(const float *x, const float *w, const float *bias, float *y,
+                       int n, int c, int h, int wd, int f, int r, int s, int ph, int pw,
+                       int sh, int sw, int dh, int dw, int groups, int act,
+                       pet_hip_stream_t stream);
+
+/* Conv3d, NCTHW x [n,c,t,h,w], weight [f, c/groups, kt, r, s]. The reference
+ * snapshot has no 3-D convolution (Operator::OpType, include/operator.h:19-51);
+ * this is ConvOp::compute with one more spatial axis, needed by the ResNet3D-18
+ * programs of pet-ae/run_policy_3d.sh:13-33. */
+PET_HIP_API int pet_hip_conv3d_f32(const float *x, const float *w, const float *bias, float *y,
+                       int n, int c, int t, int h, int wd, int f, int kt, int r, int s,
+                       int pt, int ph, int pw, int st, int sh, int sw, int dt, int dh,
+                       int dw, int groups, int act, pet_hip_stream_t stream);
+
+/* Batched row-major matmul C[b,m,n] = A'[b,m,k] * B'[b,k,n]; transA: A stored
+ * [b,k,m]; transB: B stored [b,n,k]. bias (may be NULL) is [n], added per
+ * output column. Semantics: MatmulOp::compute, src/Graph/operator.cc:620-654;
+ * replaces cublasGemmStridedBatchedEx / cublasGemmEx
+ * (src/Graph/operator.cc:777-780, 807-810; src/Graph/code_engine.cc:1103-1169). */
+PET_HIP_API int pet_hip_bmm_f32(int transA, int transB, int b, int m, int n, int k, const float *A,
+                    const float *B, float *C, const float *bias, int act,
+                    pet_hip_stream_t stream);
+
+/* ---- layout operators (bit-exact copies) ---------------------------------*/
+
+/* TransposeOp::compute after the split has been resolved to flat dims,
+ * src/Graph/operator.cc:2172-2210: view x as `flat_dims` (nflat <= 8), output
+ * is that view permuted by `perm` (output dim j is flat dim perm[j]). Replaces
+ * the TVM gather kernel and kernel_transpose_3d (src/Graph/code_engine.cc:27-84,
+ * 499-530). */
+PET_HIP_API int pet_hip_transpose(const float *x, float *y, const int *flat_dims, const int *perm,
+                      int nflat, pet_hip_stream_t stream);
+
+/* A TransSplit / TransReorder / TransFuse chain with its boundary-correction
+ * parameters, src/Transpose/transpose.cc:22-42 (split: extr, copys), 136-150
+ * (reorder), 70-106 (fuse: pad, dels); what TransposeEngine::getLambda (:192-220)
+ * hands to TVM. ops holds nops records of 6 ints {kind, a, b, c, d, 0}:
+ *   kind 0 split  : a=index, b=in_dim, c=extr, d=copys
+ *   kind 1 reorder: permutation read from `perms` (rank-at-that-point ints)
+ *   kind 2 fuse   : a=index, b=pad, c=dels
+ * out_dims (PET_HIP_MAX_RANK ints) receives the result shape, *out_rank its
+ * rank. With y == NULL only the shape is computed. Positions that map outside
+ * the input, and the pad rows of a fuse, are written as 0. */
+PET_HIP_API int pet_hip_trans_chain(const float *x, float *y, const int *in_dims, int rank,
+                        const int *ops, int nops, const int *perms, int *out_dims,
+                        int *out_rank, pet_hip_stream_t stream);
+
+/* SplitOp::computeV, src/Graph/operator.cc:1978-2020: ys[i] receives the slab
+ * of extent out_sizes[i] along `dim` (sum must equal in_dims[dim]). Replaces
+ * the pointer aliasing / TVM kernels of src/Graph/code_engine.cc:133-144,
+ * 1505-1545. */
+PET_HIP_API int pet_hip_split(const float *x, float *const *ys, int k, const int *in_dims, int rank,
+                  int dim, const int *out_sizes, pet_hip_stream_t stream);
+
+/* ConcatOp::compute, src/Graph/operator.cc:1813-1850 (inputs may repeat).
+ * Replaces src/Graph/code_engine.cc:145-154, 1551-1615. */
+PET_HIP_API int pet_hip_concat(const float *const *xs, int k, float *y, const int *out_dims, int rank,
+                   int dim, const int *in_sizes, pet_hip_stream_t stream);
+
+/* PadOp::compute, src/Graph/operator.cc:1640-1662 (cudnnTransformTensorEx at
+ * src/Graph/code_engine.cc:1171-1216). */
+PET_HIP_API int pet_hip_pad(const float *x, float *y, const int *in_dims, const int *begin,
+                const int *end, int rank, pet_hip_stream_t stream);
+
+/* SliceOp::compute, src/Graph/operator.cc:1741-1756
+ * (src/Graph/code_engine.cc:1465-1499). */
+PET_HIP_API int pet_hip_slice(const float *x, float *y, const int *in_dims, const int *begin,
+                  const int *end, int rank, pet_hip_stream_t stream);
+
+/* ExtendOp::compute, src/Graph/operator.cc:2577-2597: the block from `dim`
+ * inwards repeated num+1 times (src/Graph/code_engine.cc:1621-1675). */
+PET_HIP_API int pet_hip_extend(const float *x, float *y, const int *in_dims, int rank, int dim,
+                   int num, pet_hip_stream_t stream);
+
+/* ---- element-wise ---------------------------------------------------------*/
+
+/* k-ary Add / Mul, binary Sub with flat-modulo broadcast in[i % sizes[j]]
+ * (src/Graph/operator.cc:2983-3002, 3074-3090, 3157-3176); replaces
+ * cublasSaxpy / cudnnOpTensor (src/Graph/code_engine.cc:1335-1348, 1377-1422).
+ * k <= 8. y may alias ins[j] only when sizes[j] == n. */
+PET_HIP_API int pet_hip_eltwise(int op, const float *const *ins, const size_t *sizes, int k, float *y,
+                    size_t n, pet_hip_stream_t stream);
+
+/* y = act(x); replaces cudnnActivationForward (src/Graph/code_engine.cc:1260-1274).
+ * The reference has no CPU compute for it (include/operator.h:1968-1977). */
+PET_HIP_API int pet_hip_activation(const float *x, float *y, size_t n, int act, pet_hip_stream_t stream);
+
+/* y[o, ch, i] = act(x[o, ch, i] + bias[ch]) on an [outer, ch, inner] view;
+ * replaces cudnnAddTensor + cudnnActivationForward
+ * (src/Graph/code_engine.cc:917-924, 944-952). x == y is allowed. */
+PET_HIP_API int pet_hip_bias_act(const float *x, const float *bias, float *y, size_t outer, size_t ch,
+                     size_t inner, int act, pet_hip_stream_t stream);
+
+/* ---- non-contraction network pieces without a reference CPU compute -------*/
+
+/* Max (mode 0) / average (mode 1, divisor kh*kw) pooling over NCHW with
+ * out = (in + 2p - d (k-1) - 1) / s + 1; replaces cudnnPoolingForward
+ * (src/Graph/operator.cc:2814-2827, 2937-2950; code_engine.cc:1315-1329). */
+PET_HIP_API int pet_hip_pool2d(const float *x, float *y, int n, int c, int h, int w, int kh, int kw,
+                   int ph, int pw, int sh, int sw, int dh, int dw, int mode,
+                   pet_hip_stream_t stream);
+
+/* Row softmax over the last axis of a [rows, cols] view; replaces
+ * online_softmax (src/Graph/code_engine.cc:424-486, 1707-1731). */
+PET_HIP_API int pet_hip_softmax(const float *x, float *y, size_t rows, size_t cols,
+                    pet_hip_stream_t stream);
+
+/* LayerNorm over the last axis (gamma / beta may be NULL); absent upstream,
+ * needed by the BERT-base-shaped encoder. */
+PET_HIP_API int pet_hip_layernorm(const float *x, const float *gamma, const float *beta, float *y,
+                      size_t rows, size_t cols, float eps, pet_hip_stream_t stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* PET_HIP_H */

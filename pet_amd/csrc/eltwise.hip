@@ -1,0 +1,375 @@
+// Element-wise operators, activation / bias epilogues and the small
+// non-contraction network pieces (pooling, softmax, layernorm).
+#include "common.h"
+
+#include <algorithm>
+
+using namespace pet;
+
+namespace {
+
+constexpr int kMaxEltIn = 8;
+
+struct EltParams {
+    const float *in[kMaxEltIn];
+    unsigned size[kMaxEltIn]; // 0 = same size as the output (no modulo)
+    unsigned mul[kMaxEltIn], shift[kMaxEltIn];
+    int k, op;
+    size_t n;
+};
+
+__device__ __forceinline__ unsigned mod_fast(unsigned i, unsigned d, unsigned mul, unsigned shift) {
+    unsigned q = __umulhi(i, mul) >> shift;
+    return i - q * d;
+}
+
+// VEC == 4: the host has checked n % 4 == 0, every broadcast size % 4 == 0 and
+// 16-byte alignment, so four consecutive outputs read four consecutive inputs.
+template <int VEC>
+__global__ __launch_bounds__(256) void eltwise_kernel(EltParams p, float *__restrict__ y) {
+    size_t i = ((size_t)blockIdx.x * 256 + threadIdx.x) * VEC;
+    const size_t step = (size_t)gridDim.x * 256 * VEC;
+    for (; i < p.n; i += step) {
+        float acc[VEC];
+#pragma unroll
+        for (int v = 0; v < VEC; ++v)
+            acc[v] = p.op == PET_HIP_MUL ? 1.f : 0.f;
+#pragma unroll
+        for (int j = 0; j < kMaxEltIn; ++j) {
+            if (j < p.k) {
+                size_t src = i;
+                if (p.size[j] == 1)
+                    src = 0;
+                else if (p.size[j])
+                    src = mod_fast((unsigned)i, p.size[j], p.mul[j], p.shift[j]);
+                float val[VEC];
+                if (VEC == 4 && p.size[j] != 1) {
+                    float4 t = *reinterpret_cast<const float4 *>(p.in[j] + src);
+                    val[0] = t.x;
+                    val[1 % VEC] = t.y;
+                    val[2 % VEC] = t.z;
+                    val[3 % VEC] = t.w;
+                } else {
+#pragma unroll
+                    for (int v = 0; v < VEC; ++v)
+                        val[v] = p.in[j][p.size[j] == 1 ? 0 : src + v];
+                }
+#pragma unroll
+                for (int v = 0; v < VEC; ++v) {
+                    if (p.op == PET_HIP_ADD)
+                        acc[v] += val[v];
+                    else if (p.op == PET_HIP_MUL)
+                        acc[v] *= val[v];
+                    else
+                        acc[v] = j == 0 ? val[v] : acc[v] - val[v];
+                }
+            }
+        }
+        if (VEC == 4)
+            *reinterpret_cast<float4 *>(y + i) = make_float4(acc[0], acc[1 % VEC], acc[2 % VEC],
+                                                             acc[3 % VEC]);
+        else
+            y[i] = acc[0];
+    }
+}
+
+template <int VEC>
+__global__ __launch_bounds__(256) void activation_kernel(const float *__restrict__ x,
+                                                         float *__restrict__ y, size_t n,
+                                                         int act) {
+    size_t i = ((size_t)blockIdx.x * 256 + threadIdx.x) * VEC;
+    const size_t step = (size_t)gridDim.x * 256 * VEC;
+    for (; i < n; i += step) {
+        if (VEC == 4) {
+            float4 v = *reinterpret_cast<const float4 *>(x + i);
+            v.x = apply_act(v.x, act);
+            v.y = apply_act(v.y, act);
+            v.z = apply_act(v.z, act);
+            v.w = apply_act(v.w, act);
+            *reinterpret_cast<float4 *>(y + i) = v;
+        } else {
+            y[i] = apply_act(x[i], act);
+        }
+    }
+}
+
+__global__ __launch_bounds__(256) void bias_act_kernel(const float *__restrict__ x,
+                                                       const float *__restrict__ bias,
+                                                       float *__restrict__ y, size_t total,
+                                                       unsigned ch, unsigned inner, int act) {
+    size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    const size_t step = (size_t)gridDim.x * 256;
+    for (; i < total; i += step) {
+        unsigned c = (unsigned)((i / inner) % ch);
+        float v = x[i] + (bias ? bias[c] : 0.f);
+        y[i] = apply_act(v, act);
+    }
+}
+
+__global__ __launch_bounds__(256) void pool2d_kernel(const float *__restrict__ x,
+                                                     float *__restrict__ y, int nc, int h, int w,
+                                                     int kh, int kw, int ph, int pw, int sh,
+                                                     int sw, int dh, int dw, int oh, int ow,
+                                                     int mode) {
+    size_t total = (size_t)nc * oh * ow;
+    size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    const size_t step = (size_t)gridDim.x * 256;
+    for (; i < total; i += step) {
+        int j = (int)(i % ow);
+        int ii = (int)((i / ow) % oh);
+        size_t plane = i / ((size_t)ow * oh);
+        const float *xp = x + plane * (size_t)h * w;
+        float acc = mode == 0 ? -INFINITY : 0.f;
+        for (int r = 0; r < kh; ++r) {
+            int ih = ii * sh + r * dh - ph;
+            if (ih < 0 || ih >= h)
+                continue;
+            for (int s = 0; s < kw; ++s) {
+                int iw = j * sw + s * dw - pw;
+                if (iw < 0 || iw >= w)
+                    continue;
+                float v = xp[(size_t)ih * w + iw];
+                acc = mode == 0 ? fmaxf(acc, v) : acc + v;
+            }
+        }
+        y[i] = mode == 0 ? acc : acc / (float)(kh * kw);
+    }
+}
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1)
+        v += __shfl_xor(v, o, 64);
+    return v;
+}
+
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1)
+        v = fmaxf(v, __shfl_xor(v, o, 64));
+    return v;
+}
+
+// Global average pooling: one wave per (n, c) plane.
+__global__ __launch_bounds__(256) void global_avgpool_kernel(const float *__restrict__ x,
+                                                             float *__restrict__ y, int nc,
+                                                             int hw) {
+    int plane = blockIdx.x * 4 + (threadIdx.x >> 6);
+    int lane = threadIdx.x & 63;
+    if (plane >= nc)
+        return;
+    const float *xp = x + (size_t)plane * hw;
+    float acc = 0.f;
+    for (int i = lane; i < hw; i += 64)
+        acc += xp[i];
+    acc = wave_sum(acc);
+    if (lane == 0)
+        y[plane] = acc / (float)hw;
+}
+
+// One wave per row; rows of any length.
+__global__ __launch_bounds__(256) void softmax_kernel(const float *__restrict__ x,
+                                                      float *__restrict__ y, size_t rows,
+                                                      size_t cols) {
+    size_t row = (size_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    int lane = threadIdx.x & 63;
+    if (row >= rows)
+        return;
+    const float *xp = x + row * cols;
+    float *yp = y + row * cols;
+    float mx = -INFINITY;
+    for (size_t j = lane; j < cols; j += 64)
+        mx = fmaxf(mx, xp[j]);
+    mx = wave_max(mx);
+    float sum = 0.f;
+    for (size_t j = lane; j < cols; j += 64)
+        sum += expf(xp[j] - mx);
+    sum = wave_sum(sum);
+    float inv = 1.f / sum;
+    for (size_t j = lane; j < cols; j += 64)
+        yp[j] = expf(xp[j] - mx) * inv;
+}
+
+__global__ __launch_bounds__(256) void layernorm_kernel(const float *__restrict__ x,
+                                                        const float *__restrict__ gamma,
+                                                        const float *__restrict__ beta,
+                                                        float *__restrict__ y, size_t rows,
+                                                        size_t cols, float eps) {
+    size_t row = (size_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    int lane = threadIdx.x & 63;
+    if (row >= rows)
+        return;
+    const float *xp = x + row * cols;
+    float *yp = y + row * cols;
+    float s = 0.f;
+    for (size_t j = lane; j < cols; j += 64)
+        s += xp[j];
+    float mean = wave_sum(s) / (float)cols;
+    float v = 0.f;
+    for (size_t j = lane; j < cols; j += 64) {
+        float d = xp[j] - mean;
+        v += d * d;
+    }
+    float inv = rsqrtf(wave_sum(v) / (float)cols + eps);
+    for (size_t j = lane; j < cols; j += 64) {
+        float o = (xp[j] - mean) * inv;
+        if (gamma)
+            o *= gamma[j];
+        if (beta)
+            o += beta[j];
+        yp[j] = o;
+    }
+}
+
+unsigned grid_for(size_t items) {
+    size_t g = (items + 255) / 256;
+    return (unsigned)std::min<size_t>(std::max<size_t>(g, 1), 1u << 20);
+}
+
+bool aligned16(const void *p) { return ((uintptr_t)p & 15) == 0; }
+
+} // namespace
+
+extern "C" {
+
+int pet_hip_eltwise(int op, const float *const *ins, const size_t *sizes, int k, float *y,
+                    size_t n, pet_hip_stream_t stream) {
+    PET_REQUIRE_INIT();
+    if (op != PET_HIP_ADD && op != PET_HIP_SUB && op != PET_HIP_MUL)
+        return set_error(PET_HIP_ERR_INVALID, "unknown element-wise op %d", op);
+    if (k < 1 || k > kMaxEltIn || !ins || !sizes)
+        return set_error(PET_HIP_ERR_INVALID, "element-wise ops take 1..%d inputs", kMaxEltIn);
+    if (op == PET_HIP_SUB && k != 2)
+        return set_error(PET_HIP_ERR_INVALID, "Sub is binary");
+    if (n == 0)
+        return PET_HIP_OK;
+    if (!y)
+        return set_error(PET_HIP_ERR_INVALID, "null output");
+    if (n >= (1ull << 31))
+        return set_error(PET_HIP_ERR_UNSUPPORTED, "element-wise ops are limited to 2^31 elements");
+    EltParams p;
+    memset(&p, 0, sizeof(p));
+    p.k = k;
+    p.op = op;
+    p.n = n;
+    bool vec = (n % 4 == 0) && aligned16(y);
+    for (int j = 0; j < k; ++j) {
+        if (!ins[j] || sizes[j] == 0)
+            return set_error(PET_HIP_ERR_INVALID, "input %d is empty", j);
+        p.in[j] = ins[j];
+        if (sizes[j] >= n) {
+            p.size[j] = 0; // i % size == i
+        } else {
+            unsigned d = (unsigned)sizes[j];
+            p.size[j] = d;
+            if (d > 1) {
+                unsigned l = 0;
+                while ((1ull << l) < d)
+                    ++l;
+                unsigned pw = 31 + l;
+                p.mul[j] = (unsigned)(((1ull << pw) + d - 1) / d);
+                p.shift[j] = pw - 32;
+            }
+            if (d != 1 && d % 4)
+                vec = false;
+        }
+        if (!aligned16(ins[j]))
+            vec = false;
+    }
+    if (vec)
+        hipLaunchKernelGGL(eltwise_kernel<4>, dim3(grid_for(n / 4)), dim3(256), 0,
+                           as_stream(stream), p, y);
+    else
+        hipLaunchKernelGGL(eltwise_kernel<1>, dim3(grid_for(n)), dim3(256), 0, as_stream(stream),
+                           p, y);
+    return check_launch("eltwise_kernel");
+}
+
+int pet_hip_activation(const float *x, float *y, size_t n, int act, pet_hip_stream_t stream) {
+    PET_REQUIRE_INIT();
+    if (act < PET_HIP_ACT_NONE || act > PET_HIP_ACT_GELU)
+        return set_error(PET_HIP_ERR_INVALID, "unknown activation %d", act);
+    if (n == 0)
+        return PET_HIP_OK;
+    if (!x || !y)
+        return set_error(PET_HIP_ERR_INVALID, "null pointer");
+    if (n % 4 == 0 && aligned16(x) && aligned16(y))
+        hipLaunchKernelGGL(activation_kernel<4>, dim3(grid_for(n / 4)), dim3(256), 0,
+                           as_stream(stream), x, y, n, act);
+    else
+        hipLaunchKernelGGL(activation_kernel<1>, dim3(grid_for(n)), dim3(256), 0,
+                           as_stream(stream), x, y, n, act);
+    return check_launch("activation_kernel");
+}
+
+int pet_hip_bias_act(const float *x, const float *bias, float *y, size_t outer, size_t ch,
+                     size_t inner, int act, pet_hip_stream_t stream) {
+    PET_REQUIRE_INIT();
+    if (act < PET_HIP_ACT_NONE || act > PET_HIP_ACT_GELU)
+        return set_error(PET_HIP_ERR_INVALID, "unknown activation %d", act);
+    size_t total = outer * ch * inner;
+    if (total == 0)
+        return PET_HIP_OK;
+    if (!x || !y)
+        return set_error(PET_HIP_ERR_INVALID, "null pointer");
+    if (ch >= (1ull << 31) || inner >= (1ull << 31))
+        return set_error(PET_HIP_ERR_UNSUPPORTED, "bias_act dims too large");
+    hipLaunchKernelGGL(bias_act_kernel, dim3(grid_for(total)), dim3(256), 0, as_stream(stream), x,
+                       bias, y, total, (unsigned)ch, (unsigned)inner, act);
+    return check_launch("bias_act_kernel");
+}
+
+int pet_hip_pool2d(const float *x, float *y, int n, int c, int h, int w, int kh, int kw, int ph,
+                   int pw, int sh, int sw, int dh, int dw, int mode, pet_hip_stream_t stream) {
+    PET_REQUIRE_INIT();
+    if (n < 0 || c < 0 || h <= 0 || w <= 0 || kh <= 0 || kw <= 0 || sh <= 0 || sw <= 0 ||
+        dh <= 0 || dw <= 0 || ph < 0 || pw < 0 || (mode != 0 && mode != 1))
+        return set_error(PET_HIP_ERR_INVALID, "bad pooling arguments");
+    int oh = (h + 2 * ph - dh * (kh - 1) - 1) / sh + 1;
+    int ow = (w + 2 * pw - dw * (kw - 1) - 1) / sw + 1;
+    if (oh <= 0 || ow <= 0)
+        return set_error(PET_HIP_ERR_INVALID, "pooling window larger than the image");
+    size_t total = (size_t)n * c * oh * ow;
+    if (total == 0)
+        return PET_HIP_OK;
+    if (!x || !y)
+        return set_error(PET_HIP_ERR_INVALID, "null pointer");
+    if (mode == 1 && kh == h && kw == w && ph == 0 && pw == 0 && dh == 1 && dw == 1) {
+        int nc = n * c;
+        hipLaunchKernelGGL(global_avgpool_kernel, dim3((nc + 3) / 4), dim3(256), 0,
+                           as_stream(stream), x, y, nc, h * w);
+        return check_launch("global_avgpool_kernel");
+    }
+    hipLaunchKernelGGL(pool2d_kernel, dim3(grid_for(total)), dim3(256), 0, as_stream(stream), x, y,
+                       n * c, h, w, kh, kw, ph, pw, sh, sw, dh, dw, oh, ow, mode);
+    return check_launch("pool2d_kernel");
+}
+
+int pet_hip_softmax(const float *x, float *y, size_t rows, size_t cols, pet_hip_stream_t stream) {
+    PET_REQUIRE_INIT();
+    if (rows == 0 || cols == 0)
+        return PET_HIP_OK;
+    if (!x || !y)
+        return set_error(PET_HIP_ERR_INVALID, "null pointer");
+    if ((rows + 3) / 4 >= (1ull << 31))
+        return set_error(PET_HIP_ERR_UNSUPPORTED, "too many rows");
+    hipLaunchKernelGGL(softmax_kernel, dim3((unsigned)((rows + 3) / 4)), dim3(256), 0,
+                       as_stream(stream), x, y, rows, cols);
+    return check_launch("softmax_kernel");
+}
+
+int pet_hip_layernorm(const float *x, const float *gamma, const float *beta, float *y, size_t rows,
+                      size_t cols, float eps, pet_hip_stream_t stream) {
+    PET_REQUIRE_INIT();
+    if (rows == 0 || cols == 0)
+        return PET_HIP_OK;
+    if (!x || !y)
+        return set_error(PET_HIP_ERR_INVALID, "null pointer");
+    if ((rows + 3) / 4 >= (1ull << 31))
+        return set_error(PET_HIP_ERR_UNSUPPORTED, "too many rows");
+    hipLaunchKernelGGL(layernorm_kernel, dim3((unsigned)((rows + 3) / 4)), dim3(256), 0,
+                       as_stream(stream), x, gamma, beta, y, rows, cols, eps);
+    return check_launch("layernorm_kernel");
+}
+
+} // extern "C"

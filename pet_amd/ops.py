@@ -1,0 +1,305 @@
+"""Operator calls on torch device tensors, each one a single C-ABI call.
+
+torch only owns the memory and names the stream; shapes are worked out here
+with the same rules as the reference's ``computeShape`` methods so callers can
+allocate outputs. All tensors must be contiguous fp32 CUDA(HIP) tensors.
+"""
+import ctypes
+
+import torch
+
+from . import abi
+
+
+def _stream():
+    return ctypes.c_void_p(torch.cuda.current_stream().cuda_stream)
+
+
+def _chk(*ts):
+    abi.init(torch.cuda.current_device())
+    for t in ts:
+        if t is None:
+            continue
+        if not (t.is_cuda and t.dtype == torch.float32 and t.is_contiguous()):
+            raise ValueError("expected contiguous fp32 device tensors")
+
+
+def _ptr(t):
+    return ctypes.c_void_p(0 if t is None else t.data_ptr())
+
+
+def conv_out_dim(i, k, p, s, d):
+    """ConvOp::computeShape, src/Graph/operator.cc:219-221."""
+    return (i - (k - s) * d + 2 * p) // s if (i - (k - s) * d + 2 * p) >= 0 else -1
+
+
+def conv2d(x, w, ph, pw, sh=1, sw=1, dh=1, dw=1, bias=None, act="none", out=None):
+    _chk(x, w, bias, out)
+    n, c, h, wd = x.shape
+    f, cpg, r, s = w.shape
+    if cpg <= 0 or c % cpg:
+        raise abi.PetHipError(1, "input channels not divisible by weight channels")
+    groups = c // cpg
+    oh, ow = conv_out_dim(h, r, ph, sh, dh), conv_out_dim(wd, s, pw, sw, dw)
+    if out is None:
+        out = torch.empty((n, f, max(oh, 0), max(ow, 0)), device=x.device, dtype=torch.float32)
+    abi.call("pet_hip_conv2d_f32", _ptr(x), _ptr(w), _ptr(bias), _ptr(out), n, c, h, wd, f, r, s,
+             ph, pw, sh, sw, dh, dw, groups, abi.ACT[act], _stream())
+    return out
+
+
+def conv3d(x, w, pad, stride=(1, 1, 1), dil=(1, 1, 1), bias=None, act="none", out=None):
+    _chk(x, w, bias, out)
+    n, c, t, h, wd = x.shape
+    f, cpg, kt, r, s = w.shape
+    if cpg <= 0 or c % cpg:
+        raise abi.PetHipError(1, "input channels not divisible by weight channels")
+    groups = c // cpg
+    ot = conv_out_dim(t, kt, pad[0], stride[0], dil[0])
+    oh = conv_out_dim(h, r, pad[1], stride[1], dil[1])
+    ow = conv_out_dim(wd, s, pad[2], stride[2], dil[2])
+    if out is None:
+        out = torch.empty((n, f, ot, oh, ow), device=x.device, dtype=torch.float32)
+    abi.call("pet_hip_conv3d_f32", _ptr(x), _ptr(w), _ptr(bias), _ptr(out), n, c, t, h, wd, f, kt,
+             r, s, *pad, *stride, *dil, groups, abi.ACT[act], _stream())
+    return out
+
+
+def matmul(A, B, transA=False, transB=False, bias=None, act="none", out=None):
+    """MatmulOp on [b, ., .] tensors (MatmulOp::computeShape, operator.cc:717-726)."""
+    _chk(A, B, bias, out)
+    b = A.shape[0]
+    m = A.shape[2] if transA else A.shape[1]
+    k = A.shape[1] if transA else A.shape[2]
+    n = B.shape[1] if transB else B.shape[2]
+    kb = B.shape[2] if transB else B.shape[1]
+    if B.shape[0] != b or kb != k:
+        raise abi.PetHipError(1, "matmul shapes do not agree")
+    if out is None:
+        out = torch.empty((b, m, n), device=A.device, dtype=torch.float32)
+    abi.call("pet_hip_bmm_f32", int(transA), int(transB), b, m, n, k, _ptr(A), _ptr(B), _ptr(out),
+             _ptr(bias), abi.ACT[act], _stream())
+    return out
+
+
+def transpose_params(in_dims, split, after, factor):
+    """TransposeOp::setParam (include/operator.h:1124-1144) and the flat-dim
+    rule of TransposeOp::computeShape (src/Graph/operator.cc:2340-2381).
+    Returns (flat_dims, perm, out_dims) or None when the split does not divide."""
+    items = [list(a) if isinstance(a, (list, tuple)) else [a] for a in after]
+    if split >= 0:
+        if factor == 0:
+            return None
+        items = [[(split + 1) if i == -1 else (i + 1 if i > split else i) for i in it]
+                 for it in items]
+    flat = []
+    for i, d in enumerate(in_dims):
+        if i != split:
+            flat.append(d)
+        elif factor > 0:
+            if d % factor or d < factor:
+                return None
+            flat += [d // factor, factor]
+        else:
+            if d % (-factor) or d < -factor:
+                return None
+            flat += [-factor, d // (-factor)]
+    perm = [i for it in items for i in it]
+    if sorted(perm) != list(range(len(flat))) or sum(len(it) > 1 for it in items) > 1:
+        return None
+    out = []
+    for it in items:
+        e = 1
+        for i in it:
+            e *= flat[i]
+        out.append(e)
+    return flat, perm, out
+
+
+def transpose(x, split, after, factor=2, out=None):
+    """TransposeOp(input, split, after, factor)."""
+    _chk(x, out)
+    prm = transpose_params(list(x.shape), split, after, factor)
+    if prm is None:
+        return None
+    flat, perm, oshape = prm
+    if out is None:
+        out = torch.empty(oshape, device=x.device, dtype=torch.float32)
+    abi.call("pet_hip_transpose", _ptr(x), _ptr(out), abi.ints(flat), abi.ints(perm), len(flat),
+             _stream())
+    return out
+
+
+def permute_flat(x, flat, perm, out=None):
+    _chk(x, out)
+    if out is None:
+        out = torch.empty([flat[i] for i in perm], device=x.device, dtype=torch.float32)
+    abi.call("pet_hip_transpose", _ptr(x), _ptr(out), abi.ints(flat), abi.ints(perm), len(flat),
+             _stream())
+    return out
+
+
+def _encode_chain(micro_ops):
+    enc, perms = [], []
+    for op in micro_ops:
+        if op[0] == "split":
+            enc += [0, op[1], op[2], op[3], op[4], 0]
+        elif op[0] == "reorder":
+            enc += [1, 0, 0, 0, 0, 0]
+            perms += list(op[1])
+        elif op[0] == "fuse":
+            enc += [2, op[1], op[2], op[3], 0, 0]
+        else:
+            raise ValueError(op[0])
+    return enc, perms
+
+
+def trans_chain(x, micro_ops, out=None):
+    """A TransSplit / TransReorder / TransFuse chain (src/Transpose/transpose.cc)."""
+    _chk(x, out)
+    enc, perms = _encode_chain(micro_ops)
+    odims = (ctypes.c_int * 8)()
+    ork = ctypes.c_int(0)
+    args = (abi.ints(x.shape), x.dim(), abi.ints(enc), len(micro_ops), abi.ints(perms), odims,
+            ctypes.byref(ork), _stream())
+    abi.call("pet_hip_trans_chain", _ptr(x), ctypes.c_void_p(0), *args)
+    oshape = [odims[i] for i in range(ork.value)]
+    if out is None:
+        out = torch.empty(oshape, device=x.device, dtype=torch.float32)
+    abi.call("pet_hip_trans_chain", _ptr(x), _ptr(out), *args)
+    return out
+
+
+def split_sizes(dim_size, sizes=None, num=None):
+    """SplitOp::computeShapeV ratio rule, src/Graph/operator.cc:2074-2101."""
+    if not sizes:
+        if num is None or num <= 0:
+            return None
+        sizes = [1] * num
+    total = sum(sizes)
+    if total <= 0 or dim_size % total:
+        return None
+    return [dim_size // total * s for s in sizes]
+
+
+def split(x, dim, sizes=None, num=None):
+    _chk(x)
+    szs = split_sizes(x.shape[dim], sizes, num)
+    if szs is None:
+        return None
+    outs = []
+    for s in szs:
+        shp = list(x.shape)
+        shp[dim] = s
+        outs.append(torch.empty(shp, device=x.device, dtype=torch.float32))
+    ptrs = (ctypes.c_void_p * len(outs))(*[o.data_ptr() for o in outs])
+    abi.call("pet_hip_split", _ptr(x), ptrs, len(outs), abi.ints(x.shape), x.dim(), dim,
+             abi.ints(szs), _stream())
+    return outs
+
+
+def concat(xs, dim, out=None):
+    _chk(*xs)
+    shp = list(xs[0].shape)
+    shp[dim] = sum(x.shape[dim] for x in xs)
+    if out is None:
+        out = torch.empty(shp, device=xs[0].device, dtype=torch.float32)
+    ptrs = (ctypes.c_void_p * len(xs))(*[x.data_ptr() for x in xs])
+    abi.call("pet_hip_concat", ptrs, len(xs), _ptr(out), abi.ints(shp), len(shp), dim,
+             abi.ints([x.shape[dim] for x in xs]), _stream())
+    return out
+
+
+def pad(x, begin, end, out=None):
+    _chk(x, out)
+    shp = [d + b + e for d, b, e in zip(x.shape, begin, end)]
+    if out is None:
+        out = torch.empty(shp, device=x.device, dtype=torch.float32)
+    abi.call("pet_hip_pad", _ptr(x), _ptr(out), abi.ints(x.shape), abi.ints(begin), abi.ints(end),
+             x.dim(), _stream())
+    return out
+
+
+def slice_(x, begin, end, out=None):
+    _chk(x, out)
+    shp = [max(d - b - e, 0) for d, b, e in zip(x.shape, begin, end)]
+    if out is None:
+        out = torch.empty(shp, device=x.device, dtype=torch.float32)
+    abi.call("pet_hip_slice", _ptr(x), _ptr(out), abi.ints(x.shape), abi.ints(begin),
+             abi.ints(end), x.dim(), _stream())
+    return out
+
+
+def extend(x, dim, num, out=None):
+    _chk(x, out)
+    shp = list(x.shape)
+    shp[dim] *= num + 1
+    if out is None:
+        out = torch.empty(shp, device=x.device, dtype=torch.float32)
+    abi.call("pet_hip_extend", _ptr(x), _ptr(out), abi.ints(x.shape), x.dim(), dim, num, _stream())
+    return out
+
+
+def eltwise(op, xs, out_shape=None, out=None):
+    _chk(*xs)
+    if out is None:
+        out = torch.empty(out_shape, device=xs[0].device, dtype=torch.float32)
+    ptrs = (ctypes.c_void_p * len(xs))(*[x.data_ptr() for x in xs])
+    sizes = (ctypes.c_size_t * len(xs))(*[x.numel() for x in xs])
+    abi.call("pet_hip_eltwise", abi.ELT[op], ptrs, sizes, len(xs), _ptr(out), out.numel(),
+             _stream())
+    return out
+
+
+def activation(x, act, out=None):
+    _chk(x, out)
+    if out is None:
+        out = torch.empty_like(x)
+    abi.call("pet_hip_activation", _ptr(x), _ptr(out), x.numel(), abi.ACT[act], _stream())
+    return out
+
+
+def bias_act(x, bias, act="none", ch_axis=1, out=None):
+    _chk(x, bias, out)
+    outer = 1
+    for d in x.shape[:ch_axis]:
+        outer *= d
+    inner = 1
+    for d in x.shape[ch_axis + 1:]:
+        inner *= d
+    if out is None:
+        out = torch.empty_like(x)
+    abi.call("pet_hip_bias_act", _ptr(x), _ptr(bias), _ptr(out), outer, x.shape[ch_axis], inner,
+             abi.ACT[act], _stream())
+    return out
+
+
+def pool2d(x, kh, kw, ph, pw, sh, sw, dh=1, dw=1, mode="max", out=None):
+    _chk(x, out)
+    n, c, h, w = x.shape
+    oh = (h + 2 * ph - dh * (kh - 1) - 1) // sh + 1
+    ow = (w + 2 * pw - dw * (kw - 1) - 1) // sw + 1
+    if out is None:
+        out = torch.empty((n, c, oh, ow), device=x.device, dtype=torch.float32)
+    abi.call("pet_hip_pool2d", _ptr(x), _ptr(out), n, c, h, w, kh, kw, ph, pw, sh, sw, dh, dw,
+             0 if mode == "max" else 1, _stream())
+    return out
+
+
+def softmax(x, out=None):
+    _chk(x, out)
+    if out is None:
+        out = torch.empty_like(x)
+    cols = x.shape[-1]
+    abi.call("pet_hip_softmax", _ptr(x), _ptr(out), x.numel() // cols, cols, _stream())
+    return out
+
+
+def layernorm(x, gamma, beta, eps=1e-5, out=None):
+    _chk(x, gamma, beta, out)
+    if out is None:
+        out = torch.empty_like(x)
+    cols = x.shape[-1]
+    abi.call("pet_hip_layernorm", _ptr(x), _ptr(gamma), _ptr(beta), _ptr(out), x.numel() // cols,
+             cols, ctypes.c_float(eps), _stream())
+    return out

@@ -1,0 +1,425 @@
+"""GPU parity: every C-ABI operator against the CPU oracle on the same seeded
+inputs. Layout / indexing ops must be bit-exact. Contractions are checked in two
+tiers: small-integer inputs (exact in fp32, so bit-exact against the oracle) and
+real-valued inputs within max relative error 1e-4 (denominator floor as in the
+reference's checker, src/Test/dat/transpose_test/checker_tf.py:66)."""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+
+pytestmark = pytest.mark.gpu
+
+REL_TOL = 1e-4
+
+
+def dev(a):
+    return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+
+def host(t):
+    torch.cuda.synchronize()
+    return t.cpu().numpy()
+
+
+def ints(rng, shape, lo=-3, hi=4):
+    return rng.integers(lo, hi, size=shape).astype(np.float32)
+
+
+def max_rel_err(got, ref):
+    return float(np.max(np.abs(got - ref) / (np.abs(ref) + 0.01))) if ref.size else 0.0
+
+
+@pytest.fixture(scope="module")
+def ops():
+    from pet_amd import ops as _ops
+    return _ops
+
+
+CONV_CASES = [
+    # n, c, h, w, f, cpg, r, s, ph, pw, sh, sw, dh, dw
+    (1, 4, 9, 9, 6, 4, 3, 3, 1, 1, 1, 1, 1, 1),
+    (2, 3, 12, 10, 5, 3, 3, 3, 0, 0, 1, 1, 1, 1),
+    (1, 4, 11, 13, 8, 4, 3, 3, 1, 1, 2, 2, 1, 1),
+    (1, 8, 12, 12, 8, 8, 3, 3, 2, 2, 1, 1, 2, 2),
+    (1, 8, 10, 10, 12, 2, 3, 3, 1, 1, 1, 1, 1, 1),      # groups = 4
+    (2, 6, 8, 8, 6, 1, 3, 3, 1, 1, 1, 1, 1, 1),         # depthwise
+    (1, 5, 14, 14, 7, 5, 1, 1, 0, 0, 2, 2, 1, 1),       # 1x1 / s2
+    (1, 3, 30, 30, 64, 3, 7, 7, 3, 3, 2, 2, 1, 1),      # 7x7 / s2 stem, K = 147
+    (1, 2, 9, 15, 3, 2, 1, 3, 0, 1, 1, 1, 1, 1),        # 1xk
+    (1, 2, 9, 15, 3, 2, 3, 1, 2, 0, 1, 2, 1, 1),
+    (1, 1, 16, 16, 1, 1, 3, 3, 0, 0, 2, 2, 2, 2),       # reference out-dim quirk
+    (1, 64, 28, 28, 64, 64, 3, 3, 1, 1, 1, 1, 1, 1),    # 64x64-tile path
+    (1, 96, 20, 20, 160, 96, 3, 3, 1, 1, 1, 1, 1, 1),   # ragged M and N tiles
+    (2, 128, 32, 32, 128, 128, 3, 3, 1, 1, 1, 1, 1, 1), # larger tiles, batch in pixels
+    (4, 32, 16, 16, 256, 32, 3, 3, 1, 1, 1, 1, 1, 1),
+    (1, 512, 7, 7, 512, 512, 3, 3, 1, 1, 1, 1, 1, 1),   # ResNet layer4 shape
+]
+
+
+@pytest.mark.parametrize("case", CONV_CASES)
+def test_conv2d_integer_tier_bit_exact(ops, case):
+    n, c, h, w, f, cpg, r, s, ph, pw, sh, sw, dh, dw = case
+    rng = np.random.default_rng(hash(case) % (1 << 31))
+    x, wt = ints(rng, (n, c, h, w)), ints(rng, (f, cpg, r, s))
+    ref = oracle.conv2d(x, wt, ph, pw, sh, sw, dh, dw)
+    got = host(ops.conv2d(dev(x), dev(wt), ph, pw, sh, sw, dh, dw))
+    assert got.shape == ref.shape
+    np.testing.assert_array_equal(got, ref)
+
+
+@pytest.mark.parametrize("case", CONV_CASES[:4] + CONV_CASES[11:])
+def test_conv2d_float_tier(ops, case):
+    n, c, h, w, f, cpg, r, s, ph, pw, sh, sw, dh, dw = case
+    rng = np.random.default_rng(7)
+    x = rng.uniform(-1, 1, (n, c, h, w)).astype(np.float32)
+    wt = rng.uniform(-1, 1, (f, cpg, r, s)).astype(np.float32)
+    ref = oracle.conv2d(x, wt, ph, pw, sh, sw, dh, dw)
+    got = host(ops.conv2d(dev(x), dev(wt), ph, pw, sh, sw, dh, dw))
+    assert max_rel_err(got, ref) <= REL_TOL
+
+
+def test_conv2d_bias_act_epilogue(ops):
+    rng = np.random.default_rng(11)
+    x, wt = ints(rng, (2, 8, 10, 10)), ints(rng, (16, 8, 3, 3))
+    b = ints(rng, (16,))
+    ref = oracle.bias_act(oracle.conv2d(x, wt, 1, 1), b, "relu")
+    got = host(ops.conv2d(dev(x), dev(wt), 1, 1, bias=dev(b), act="relu"))
+    np.testing.assert_array_equal(got, ref)
+
+
+def test_conv2d_rejects_bad_groups(ops):
+    from pet_amd import abi
+    x = torch.zeros((1, 4, 5, 5), device="cuda")
+    w = torch.zeros((3, 2, 3, 3), device="cuda")
+    with pytest.raises(abi.PetHipError) as e:
+        ops.conv2d(x, w, 1, 1)
+    assert e.value.status == 1
+
+
+def test_conv2d_empty_batch(ops):
+    x = torch.zeros((0, 4, 5, 5), device="cuda")
+    w = torch.zeros((4, 4, 3, 3), device="cuda")
+    assert ops.conv2d(x, w, 1, 1).shape == (0, 4, 5, 5)
+
+
+CONV3D_CASES = [
+    # n, c, t, h, w, f, cpg, kt, r, s, pad, stride, dil
+    (1, 3, 1, 8, 8, 4, 3, 1, 3, 3, (0, 1, 1), (1, 1, 1), (1, 1, 1)),
+    (1, 3, 6, 14, 14, 8, 3, 3, 7, 7, (1, 3, 3), (1, 2, 2), (1, 1, 1)),
+    (2, 4, 6, 9, 10, 6, 4, 3, 3, 3, (1, 1, 1), (2, 2, 2), (1, 1, 1)),
+    (1, 4, 6, 9, 10, 6, 2, 3, 3, 3, (2, 2, 2), (1, 1, 1), (2, 2, 2)),
+    (1, 64, 4, 14, 14, 64, 64, 3, 3, 3, (1, 1, 1), (1, 1, 1), (1, 1, 1)),
+]
+
+
+@pytest.mark.parametrize("case", CONV3D_CASES)
+def test_conv3d_integer_tier_bit_exact(ops, case):
+    n, c, t, h, w, f, cpg, kt, r, s, pad, st, dl = case
+    rng = np.random.default_rng(5)
+    x, wt = ints(rng, (n, c, t, h, w), -2, 3), ints(rng, (f, cpg, kt, r, s), -2, 3)
+    ref = oracle.conv3d(x, wt, pad, st, dl)
+    got = host(ops.conv3d(dev(x), dev(wt), pad, st, dl))
+    assert got.shape == ref.shape
+    np.testing.assert_array_equal(got, ref)
+
+
+def test_conv3d_kt1_equals_conv2d(ops):
+    rng = np.random.default_rng(6)
+    x, wt = ints(rng, (1, 8, 1, 12, 12)), ints(rng, (8, 8, 1, 3, 3))
+    y3 = host(ops.conv3d(dev(x), dev(wt), (0, 1, 1)))
+    y2 = host(ops.conv2d(dev(x[:, :, 0]), dev(wt[:, :, 0]), 1, 1))
+    np.testing.assert_array_equal(y3[:, :, 0], y2)
+
+
+MATMUL_CASES = [
+    # b, m, n, k
+    (1, 8, 8, 4),
+    (3, 5, 7, 4),
+    (2, 33, 65, 17),
+    (1, 1, 1000, 512),       # ResNet FC
+    (3, 128, 768, 768),      # merged QKV
+    (12, 128, 128, 64),      # attention scores
+    (12, 128, 64, 128),      # attention * V
+    (1, 128, 3072, 768),
+    (2, 130, 260, 36),
+]
+
+
+@pytest.mark.parametrize("case", MATMUL_CASES)
+@pytest.mark.parametrize("tA", [False, True])
+@pytest.mark.parametrize("tB", [False, True])
+def test_matmul_integer_tier_bit_exact(ops, case, tA, tB):
+    b, m, n, k = case
+    rng = np.random.default_rng(b * 1000 + m + n + k)
+    A = ints(rng, (b, k, m) if tA else (b, m, k))
+    B = ints(rng, (b, n, k) if tB else (b, k, n))
+    ref = oracle.matmul(A, B, tA, tB)
+    got = host(ops.matmul(dev(A), dev(B), tA, tB))
+    np.testing.assert_array_equal(got, ref)
+
+
+def test_matmul_float_tier_and_bias_gelu(ops):
+    rng = np.random.default_rng(3)
+    A = rng.standard_normal((2, 128, 768)).astype(np.float32)
+    B = (0.02 * rng.standard_normal((2, 768, 256))).astype(np.float32)
+    ref = oracle.matmul(A, B)
+    got = host(ops.matmul(dev(A), dev(B)))
+    assert max_rel_err(got, ref) <= REL_TOL
+    bias = rng.standard_normal(256).astype(np.float32)
+    ref2 = oracle.bias_act(ref, bias, "gelu", ch_axis=2)
+    got2 = host(ops.matmul(dev(A), dev(B), bias=dev(bias), act="gelu"))
+    assert max_rel_err(got2, ref2) <= REL_TOL
+
+
+def test_batch_gemm_merge_identity(ops):
+    # src/Test/batch_gemm_test.cc: concat lhs, concat rhs, bmm, split == two matmuls
+    m, n, k = 8, 8, 4
+    A = np.arange(m * k, dtype=np.float32).reshape(1, m, k)
+    W0 = (3 * np.arange(k * n, dtype=np.float32)).reshape(1, k, n)
+    W1 = (7 * np.arange(k * n, dtype=np.float32)).reshape(1, k, n)
+    dA, d0, d1 = dev(A), dev(W0), dev(W1)
+    o0, o1 = host(ops.matmul(dA, d0)), host(ops.matmul(dA, d1))
+    merged = ops.matmul(ops.concat([dA, dA], 0), ops.concat([d0, d1], 0))
+    a0, a1 = ops.split(merged, 0, sizes=[1, 1])
+    np.testing.assert_array_equal(host(a0), o0)
+    np.testing.assert_array_equal(host(a1), o1)
+    assert o0[0, 0, 0] == 336
+
+
+TRANSPOSE_CASES = [
+    # dims, split, after, factor
+    ((16, 16, 32, 32), 0, [0, 1, [-1, 2], 3], 2),      # N2H (transpose_test_1.cc)
+    ((2, 64, 56, 56), 0, [0, 1, [-1, 2], 3], 2),       # N2H at config-1 size
+    ((1, 64, 56, 56), 2, [[0, 2], 1, -1, 3], -2),      # H2N at config-1 size
+    ((4, 6, 8, 10), 0, [0, 1, 2, [-1, 3]], 2),         # N2W
+    ((2, 6, 8, 20), 3, [[0, 3], 1, 2, -1], -2),        # W2N
+    ((4, 6, 8, 10), 1, [0, 1, [2, -1], 3], 2),         # C2H
+    ((4, 6, 8, 10), 1, [0, 1, 2, [3, -1]], 2),         # C2W
+    ((1, 8, 64, 64), 2, [0, 1, [-1, 2], 3], 2),        # D2H
+    ((1, 8, 64, 64), 3, [0, 1, 2, [-1, 3]], 2),        # D2W
+    ((1, 8, 64, 64), 2, [0, 1, [-1, 2], 3], -2),       # D2H inverse
+    ((1, 8, 64, 64), 3, [0, 1, 2, [-1, 3]], -2),       # D2W inverse
+    ((3, 5, 7, 9), -1, [0, 1, 3, 2], 2),               # kernel transpose
+    ((12, 128, 64), -1, [0, 2, 1], 2),                 # matmul operand transpose
+    ((128, 768), 1, [1, 0, -1], 64),                   # head split 128x768 -> 12x128x64
+    ((2, 3, 4, 6, 10), 3, [[0, 3], 1, 2, -1, 4], -2),  # 5-D H2N
+    ((1, 3, 4, 6, 10), 2, [[0, 2], 1, -1, 3, 4], -2),  # 5-D T2N
+    ((5, 300, 70), -1, [2, 0, 1], 2),
+    ((33, 65), -1, [1, 0], 2),
+    ((1, 1, 1, 1), -1, [3, 2, 1, 0], 2),
+]
+
+
+@pytest.mark.parametrize("case", TRANSPOSE_CASES)
+def test_transpose_bit_exact(ops, case):
+    dims, split, after, factor = case
+    rng = np.random.default_rng(sum(dims))
+    x = rng.standard_normal(dims).astype(np.float32)
+    ref = oracle.transpose(x, split, after, factor)
+    got = host(ops.transpose(dev(x), split, after, factor))
+    assert got.shape == ref.shape
+    assert got.tobytes() == ref.tobytes()
+
+
+def test_transpose_not_divisible_returns_none(ops):
+    x = torch.zeros((3, 2, 4, 4), device="cuda")
+    assert ops.transpose(x, 0, [0, 1, [-1, 2], 3], 2) is None
+
+
+def test_transpose_reciprocal_pairs(ops):
+    # src/Graph/trans_eliminator.cc:7-17: H2N/N2H and D2H(+2)/D2H(-2) undo each other
+    x = dev(np.random.default_rng(0).standard_normal((2, 8, 16, 12)).astype(np.float32))
+    y = ops.transpose(ops.transpose(x, 2, [[0, 2], 1, -1, 3], -2), 0, [0, 1, [-1, 2], 3], 2)
+    assert torch.equal(x, y)
+    y = ops.transpose(ops.transpose(x, 2, [0, 1, [-1, 2], 3], 2), 2, [0, 1, [-1, 2], 3], -2)
+    assert torch.equal(x, y)
+
+
+def test_space_to_batch_permute_bit_exact(ops):
+    rng = np.random.default_rng(2)
+    for c, hw, d in [(8, 16, 2), (512, 64, 2), (6, 12, 3)]:
+        x = rng.standard_normal((1, c, hw, hw)).astype(np.float32)
+        flat, perm = [1, c, hw // d, d, hw // d, d], [3, 5, 0, 1, 2, 4]
+        ref = oracle.permute_flat(x, flat, perm)
+        got = host(ops.permute_flat(dev(x), flat, perm))
+        assert got.tobytes() == ref.tobytes()
+        flat2, perm2 = [d, d, 1, c, hw // d, hw // d], [2, 3, 4, 0, 5, 1]
+        back = host(ops.permute_flat(dev(ref), flat2, perm2))
+        assert back.reshape(x.shape).tobytes() == x.tobytes()
+
+
+CHAINS = [
+    # dims, micro-ops
+    ((1, 2, 8, 5), [("split", 2, 4, 0, 1), ("reorder", [0, 2, 1, 3, 4]), ("fuse", 0, 0, 0)]),
+    ((2, 2, 5, 5), [("split", 0, 2, 0, 0), ("reorder", [0, 2, 1, 3, 4]), ("fuse", 2, 0, 1)]),
+    ((1, 64, 56, 56), [("split", 2, 28, 0, 1), ("reorder", [0, 2, 1, 3, 4]), ("fuse", 0, 0, 0)]),
+    ((2, 64, 29, 56), [("split", 0, 2, 0, 0), ("reorder", [0, 2, 1, 3, 4]), ("fuse", 2, 0, 1)]),
+    ((2, 2, 3, 4), [("split", 0, 2, 0, 0), ("reorder", [0, 2, 1, 3, 4]), ("fuse", 2, 1, 0)]),
+    ((1, 2, 7, 4), [("split", 2, 3, 1, 0), ("reorder", [0, 2, 1, 3, 4]), ("fuse", 0, 0, 0)]),
+    ((1, 3, 6, 8), [("split", 3, 4, 0, 2), ("reorder", [0, 3, 1, 2, 4]), ("fuse", 0, 0, 0)]),  # W2N halo
+    ((2, 3, 6, 6), [("split", 0, 2, 0, 0), ("reorder", [0, 2, 3, 1, 4]), ("fuse", 3, 0, 2)]),  # N2W drop
+    # two TransposeOps back to back (fuse then a different split): interpreter path
+    ((2, 3, 4, 6), [("split", 0, 2, 0, 0), ("reorder", [0, 2, 1, 3, 4]), ("fuse", 2, 0, 0),
+                    ("split", 2, 2, 0, 0), ("reorder", [0, 1, 3, 2, 4]), ("fuse", 2, 0, 0)]),
+    ((4, 5), [("reorder", [1, 0])]),
+]
+
+
+@pytest.mark.parametrize("case", CHAINS)
+def test_trans_chain_bit_exact(ops, case):
+    dims, chain = case
+    x = np.random.default_rng(9).standard_normal(dims).astype(np.float32)
+    ref = oracle.trans_chain(x, chain)
+    got = host(ops.trans_chain(dev(x), chain))
+    assert got.shape == ref.shape
+    assert got.tobytes() == ref.tobytes()
+
+
+def test_trans_chain_rejects_bad_halo(ops):
+    from pet_amd import abi
+    x = torch.zeros((1, 2, 9, 5), device="cuda")
+    with pytest.raises(abi.PetHipError):
+        ops.trans_chain(x, [("split", 2, 4, 0, 1)])   # 9 != 2 * 4
+
+
+def test_split_concat_pad_slice_extend_bit_exact(ops):
+    rng = np.random.default_rng(4)
+    x = rng.standard_normal((2, 6, 4, 8)).astype(np.float32)
+    dx = dev(x)
+    for dim in range(4):
+        outs = ops.split(dx, dim, num=2)
+        for a, b in zip(outs, oracle.split(x, dim, num=2)):
+            assert host(a).tobytes() == b.tobytes()
+        assert torch.equal(ops.concat(outs, dim), dx)
+    o = ops.split(dx, 1, sizes=[1, 2])
+    r = oracle.split(x, 1, sizes=[1, 2])
+    assert [t.shape[1] for t in o] == [2, 4]
+    for a, b in zip(o, r):
+        assert host(a).tobytes() == b.tobytes()
+    assert ops.split(dx, 1, sizes=[1, 3]) is None
+    parts = [x[:, :1], x[:, :4], x[:, :1]]
+    got = host(ops.concat([dev(p) for p in parts], 1))
+    assert got.tobytes() == oracle.concat(parts, 1).tobytes()
+    # ragged last dim (no vector path)
+    z = rng.standard_normal((3, 5, 7)).astype(np.float32)
+    got = host(ops.concat([dev(z), dev(z[:, :, :3])], 2))
+    assert got.tobytes() == oracle.concat([z, z[:, :, :3]], 2).tobytes()
+    b, e = [0, 1, 2, 0], [1, 0, 1, 3]
+    assert host(ops.pad(dx, b, e)).tobytes() == oracle.pad(x, b, e).tobytes()
+    b4, e4 = [0, 0, 1, 4], [0, 0, 0, 4]
+    assert host(ops.pad(dx, b4, e4)).tobytes() == oracle.pad(x, b4, e4).tobytes()
+    bs, es = [0, 1, 1, 2], [1, 2, 0, 1]
+    assert host(ops.slice_(dx, bs, es)).tobytes() == oracle.slice_(x, bs, es).tobytes()
+    for dim in range(4):
+        assert host(ops.extend(dx, dim, 2)).tobytes() == oracle.extend(x, dim, 2).tobytes()
+
+
+def test_slice_rejects_oversized(ops):
+    from pet_amd import abi
+    x = torch.zeros((2, 3), device="cuda")
+    with pytest.raises(abi.PetHipError):
+        ops.slice_(x, [2, 0], [1, 0])
+
+
+def test_empty_tensors_are_noops(ops):
+    x = torch.zeros((0, 3, 4), device="cuda")
+    assert ops.transpose(x, -1, [0, 2, 1]).shape == (0, 4, 3)
+    assert ops.pad(x, [0, 0, 0], [0, 1, 0]).shape == (0, 4, 4)
+    assert ops.eltwise("add", [x, x], (0, 3, 4)).shape == (0, 3, 4)
+
+
+def test_eltwise_bit_exact(ops):
+    rng = np.random.default_rng(8)
+    a = rng.standard_normal((2, 3, 8)).astype(np.float32)
+    b = rng.standard_normal((8,)).astype(np.float32)
+    c = rng.standard_normal((3, 8)).astype(np.float32)
+    d = rng.standard_normal((5,)).astype(np.float32)
+    one = rng.standard_normal((1,)).astype(np.float32)
+    for op, ins in [("add", [a, b, c]), ("mul", [a, b]), ("sub", [a, b]), ("add", [a, d]),
+                    ("add", [a, a]), ("mul", [a, one]), ("add", [a])]:
+        ref = oracle.eltwise(op, ins, a.shape)
+        got = host(ops.eltwise(op, [dev(t) for t in ins], a.shape))
+        assert got.tobytes() == ref.tobytes(), (op, len(ins))
+    # residual add at a ResNet size
+    r0 = rng.standard_normal((1, 64, 56, 56)).astype(np.float32)
+    r1 = rng.standard_normal((1, 64, 56, 56)).astype(np.float32)
+    got = host(ops.eltwise("add", [dev(r0), dev(r1)], r0.shape))
+    assert got.tobytes() == oracle.eltwise("add", [r0, r1], r0.shape).tobytes()
+
+
+def test_activation_pool_softmax_layernorm(ops):
+    rng = np.random.default_rng(10)
+    x = rng.standard_normal((2, 3, 9, 9)).astype(np.float32)
+    dx = dev(x)
+    assert host(ops.activation(dx, "relu")).tobytes() == oracle.activation(x, "relu").tobytes()
+    for act in ("sigmoid", "tanh", "gelu"):
+        np.testing.assert_allclose(host(ops.activation(dx, act)), oracle.activation(x, act),
+                                   rtol=1e-5, atol=1e-6)
+    b = rng.standard_normal(3).astype(np.float32)
+    assert host(ops.bias_act(dx, dev(b), "relu")).tobytes() == \
+        oracle.bias_act(x, b, "relu").tobytes()
+    assert host(ops.pool2d(dx, 3, 3, 1, 1, 2, 2, mode="max")).tobytes() == \
+        oracle.pool2d(x, 3, 3, 1, 1, 2, 2, mode="max").tobytes()
+    np.testing.assert_allclose(host(ops.pool2d(dx, 3, 3, 1, 1, 2, 2, mode="avg")),
+                               oracle.pool2d(x, 3, 3, 1, 1, 2, 2, mode="avg"), rtol=1e-5, atol=1e-6)
+    np.testing.assert_allclose(host(ops.pool2d(dx, 9, 9, 0, 0, 1, 1, mode="avg")),
+                               oracle.pool2d(x, 9, 9, 0, 0, 1, 1, mode="avg"), rtol=1e-5, atol=1e-6)
+    s = rng.standard_normal((12, 128, 128)).astype(np.float32)
+    np.testing.assert_allclose(host(ops.softmax(dev(s))), oracle.softmax(s), rtol=1e-5, atol=1e-7)
+    g = rng.standard_normal(768).astype(np.float32)
+    be = rng.standard_normal(768).astype(np.float32)
+    h = rng.standard_normal((128, 768)).astype(np.float32)
+    np.testing.assert_allclose(host(ops.layernorm(dev(h), dev(g), dev(be))),
+                               oracle.layernorm(h, g, be), rtol=1e-4, atol=1e-5)
+
+
+def test_config1_original_vs_corrected_transform(ops):
+    # BASELINE config 1: conv 1x64x56x56, 3x3 p1, U[-1,1] from seed 0 (x then w);
+    # original op vs H2N(halo 1) -> conv -> N2H(drop 1).
+    rng = np.random.default_rng(0)
+    x = rng.uniform(-1, 1, (1, 64, 56, 56)).astype(np.float32)
+    w = rng.uniform(-1, 1, (64, 64, 3, 3)).astype(np.float32)
+    ref = oracle.conv2d(x, w, 1, 1)
+    dx, dw = dev(x), dev(w)
+    y0 = host(ops.conv2d(dx, dw, 1, 1))
+    assert max_rel_err(y0, ref) <= REL_TOL
+    halo = ops.trans_chain(dx, [("split", 2, 28, 0, 1), ("reorder", [0, 2, 1, 3, 4]),
+                                ("fuse", 0, 0, 0)])
+    assert tuple(halo.shape) == (2, 64, 29, 56)
+    yt = ops.conv2d(halo, dw, 1, 1)
+    y1 = host(ops.trans_chain(yt, [("split", 0, 2, 0, 0), ("reorder", [0, 2, 1, 3, 4]),
+                                   ("fuse", 2, 0, 1)]))
+    assert y1.shape == ref.shape
+    assert max_rel_err(y1, ref) <= REL_TOL
+    # the oracle's own transformed program agrees with its original one exactly
+    oh = oracle.trans_chain(x, [("split", 2, 28, 0, 1), ("reorder", [0, 2, 1, 3, 4]),
+                                ("fuse", 0, 0, 0)])
+    assert host(halo).tobytes() == oh.tobytes()
+
+
+def test_graph_capture_replays_match_eager(ops):
+    import ctypes
+    from pet_amd import abi
+    rng = np.random.default_rng(12)
+    x = dev(ints(rng, (1, 16, 12, 12)))
+    w = dev(ints(rng, (16, 16, 3, 3)))
+    eager = ops.activation(ops.conv2d(x, w, 1, 1), "relu").clone()
+    st = torch.cuda.Stream()
+    out = torch.empty_like(eager)
+    tmp = torch.empty_like(eager)
+    with torch.cuda.stream(st):
+        sp = ctypes.c_void_p(st.cuda_stream)
+        abi.call("pet_hip_graph_begin_capture", sp)
+        ops.conv2d(x, w, 1, 1, out=tmp)
+        ops.activation(tmp, "relu", out=out)
+        g = ctypes.c_void_p(0)
+        abi.call("pet_hip_graph_end_capture", sp, ctypes.byref(g))
+        for _ in range(3):
+            out.zero_()
+            torch.cuda.synchronize()
+            abi.call("pet_hip_graph_launch", g, sp)
+            st.synchronize()
+            assert torch.equal(out, eager)
+        abi.call("pet_hip_graph_destroy", g)
