@@ -1,0 +1,232 @@
+#!/usr/bin/env python3
+"""Benchmark: batch-1 latency of the PET-optimised dilated-conv block on one MI355X.
+
+Workload (BASELINE config 2): six fp32 3x3 convolutions, dilation 2 / pad 2,
+channels 512->512->512->512->256->128->64 on a 1x512x64x64 input, ReLU after
+each, weights N(0, 0.01). The PET-optimised program is space-to-batch (4 phase
+images of 32x32), six dense convolutions (dilation 1, pad 1) with fused ReLU,
+batch-to-space. One "step" is one launch of that program as a HIP graph with
+inputs and weights resident in HBM.
+
+Prints one JSON line: the latency (`value`, ms), the roofline of the dominant
+kernel (the 512->512 implicit-GEMM convolution, against the fp32 MFMA peak) from
+HIP events around that kernel alone, and the CPU oracle timed on a bounded
+sample of the same workload on this box's host cores.
+"""
+import argparse
+import ctypes
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+CHANNELS = [512, 512, 512, 512, 256, 128, 64]
+HW = 64
+DIL = 2
+MFMA_FP32_PEAK_TFLOPS = 157.3
+HBM_PEAK_GBS = 8000.0
+
+
+def conv_flop(n, f, oh, ow, c, r, s):
+    return 2.0 * n * f * oh * ow * c * r * s
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--cpu-seconds", type=float, default=15.0)
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py measures one MI355X; this build has no multi-GPU path "
+                 "(run with --gpus 1)")
+
+    import numpy as np
+    import torch
+    from pet_amd import abi, ops
+
+    if not torch.cuda.is_available():
+        sys.exit("bench.py needs a GPU")
+    torch.cuda.set_device(0)
+    abi.init(0)
+    dev = torch.device("cuda:0")
+
+    g = torch.Generator(device="cpu").manual_seed(0)
+    x = torch.randn((1, CHANNELS[0], HW, HW), generator=g).to(dev)
+    ws = [(0.01 * torch.randn((CHANNELS[i + 1], CHANNELS[i], 3, 3), generator=g)).to(dev)
+          for i in range(6)]
+
+    hs = HW // DIL
+    s2b_flat, s2b_perm = [1, CHANNELS[0], hs, DIL, hs, DIL], [3, 5, 0, 1, 2, 4]
+    b2s_flat, b2s_perm = [DIL, DIL, 1, CHANNELS[-1], hs, hs], [2, 3, 4, 0, 5, 1]
+
+    # pre-allocated activations: nothing is allocated inside a step
+    t_s2b = torch.empty((DIL * DIL, CHANNELS[0], hs, hs), device=dev)
+    t_act = [torch.empty((DIL * DIL, CHANNELS[i + 1], hs, hs), device=dev) for i in range(6)]
+    t_out = torch.empty((1, CHANNELS[-1], HW, HW), device=dev)
+    o_act = [torch.empty((1, CHANNELS[i + 1], HW, HW), device=dev) for i in range(6)]
+
+    def optimised():
+        ops.permute_flat(x, s2b_flat, s2b_perm, out=t_s2b)
+        cur = t_s2b
+        for i in range(6):
+            ops.conv2d(cur, ws[i], 1, 1, act="relu", out=t_act[i])
+            cur = t_act[i]
+        ops.permute_flat(cur, b2s_flat, b2s_perm, out=t_out)
+
+    def original():
+        cur = x
+        for i in range(6):
+            ops.conv2d(cur, ws[i], DIL, DIL, 1, 1, DIL, DIL, act="relu", out=o_act[i])
+            cur = o_act[i]
+
+    stream = torch.cuda.Stream()
+    sp = ctypes.c_void_p(stream.cuda_stream)
+
+    def capture(fn):
+        with torch.cuda.stream(stream):
+            fn()  # eager once (also warms up code objects)
+            stream.synchronize()
+            abi.call("pet_hip_graph_begin_capture", sp)
+            fn()
+            gh = ctypes.c_void_p(0)
+            abi.call("pet_hip_graph_end_capture", sp, ctypes.byref(gh))
+        return gh
+
+    def time_graph(gh, steps, warmup):
+        for _ in range(warmup):
+            abi.call("pet_hip_graph_launch", gh, sp)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for _ in range(steps):
+            abi.call("pet_hip_graph_launch", gh, sp)
+        torch.cuda.synchronize()
+        return (time.perf_counter() - t0) * 1e3 / steps
+
+    g_opt = capture(optimised)
+    g_org = capture(original)
+    # the two programs agree (fp32 summation order differs between them)
+    torch.cuda.synchronize()
+    diff = (t_out - o_act[-1]).abs().max().item()
+    scale = o_act[-1].abs().max().item()
+    if not diff <= 1e-4 * max(scale, 1e-30):
+        sys.exit("optimised and original programs disagree: %g vs scale %g" % (diff, scale))
+
+    ms_opt = time_graph(g_opt, args.steps, args.warmup)
+    ms_org = time_graph(g_org, max(10, args.steps // 4), max(2, args.warmup // 4))
+
+    # ---- per-kernel timing with HIP events on the launch stream
+    ev0, ev1 = ctypes.c_void_p(0), ctypes.c_void_p(0)
+    abi.call("pet_hip_event_create", ctypes.byref(ev0))
+    abi.call("pet_hip_event_create", ctypes.byref(ev1))
+
+    def time_kernel(fn, reps=50, warm=5):
+        with torch.cuda.stream(stream):
+            for _ in range(warm):
+                fn()
+            abi.call("pet_hip_event_record", ev0, sp)
+            for _ in range(reps):
+                fn()
+            abi.call("pet_hip_event_record", ev1, sp)
+            abi.call("pet_hip_event_sync", ev1)
+            ms = ctypes.c_float(0)
+            abi.call("pet_hip_event_elapsed_ms", ctypes.byref(ms), ev0, ev1)
+        return ms.value / reps
+
+    per_op = []
+    s2b_bytes = 4.0 * 2 * x.numel()
+    ms = time_kernel(lambda: ops.permute_flat(x, s2b_flat, s2b_perm, out=t_s2b))
+    per_op.append({"op": "space_to_batch 1x512x64x64", "ms": ms, "GB/s": s2b_bytes / ms / 1e6,
+                   "frac_hbm": s2b_bytes / ms / 1e6 / HBM_PEAK_GBS})
+    conv_ms = []
+    for i in range(6):
+        src = t_s2b if i == 0 else t_act[i - 1]
+        fl = conv_flop(DIL * DIL, CHANNELS[i + 1], hs, hs, CHANNELS[i], 3, 3)
+        ms = time_kernel(lambda s=src, i=i: ops.conv2d(s, ws[i], 1, 1, act="relu", out=t_act[i]))
+        conv_ms.append(ms)
+        per_op.append({"op": "conv3x3 %d->%d @4x32x32" % (CHANNELS[i], CHANNELS[i + 1]),
+                       "ms": ms, "TFLOP/s": fl / ms / 1e9,
+                       "frac_mfma": fl / ms / 1e9 / MFMA_FP32_PEAK_TFLOPS})
+    b2s_bytes = 4.0 * 2 * t_out.numel()
+    ms = time_kernel(lambda: ops.permute_flat(t_act[5], b2s_flat, b2s_perm, out=t_out))
+    per_op.append({"op": "batch_to_space 4x64x32x32", "ms": ms, "GB/s": b2s_bytes / ms / 1e6,
+                   "frac_hbm": b2s_bytes / ms / 1e6 / HBM_PEAK_GBS})
+    # HBM-bound layout kernel at a size that cannot hide in cache: 1 GiB each way
+    big = torch.empty((1, 4096, 256, 256), device=dev)
+    big_out = torch.empty((4, 4096, 128, 128), device=dev)
+    bflat, bperm = [1, 4096, 128, 2, 128, 2], [3, 5, 0, 1, 2, 4]
+    big_bytes = 4.0 * 2 * big.numel()
+    ms = time_kernel(lambda: ops.permute_flat(big, bflat, bperm, out=big_out), reps=10, warm=2)
+    per_op.append({"op": "space_to_batch 1x4096x256x256 (1 GiB)", "ms": ms,
+                   "GB/s": big_bytes / ms / 1e6, "frac_hbm": big_bytes / ms / 1e6 / HBM_PEAK_GBS})
+    del big, big_out
+
+    dom_flop = conv_flop(DIL * DIL, 512, hs, hs, 512, 3, 3)
+    dom_ms = conv_ms[0]
+    achieved = dom_flop / dom_ms / 1e9
+    roofline = {"bound": "mfma", "kernel": "conv_igemm_kernel (512->512, 4x32x32, 3x3)",
+                "achieved": achieved, "peak": MFMA_FP32_PEAK_TFLOPS, "unit": "TFLOP/s",
+                "frac": achieved / MFMA_FP32_PEAK_TFLOPS, "traffic": None,
+                "flop_per_launch": dom_flop, "avg_launch_ms": dom_ms}
+
+    total_flop = sum(conv_flop(1, CHANNELS[i + 1], HW, HW, CHANNELS[i], 3, 3) for i in range(6))
+
+    # ---- CPU baseline: the oracle's conv loop nest on the original (dilated) program
+    cpu = None
+    if not args.no_cpu:
+        import oracle
+        xs = [x.cpu().numpy()] + [t.cpu().numpy() for t in o_act[:-1]]
+        wn = [w.cpu().numpy() for w in ws]
+        spent, done_flop, layers = 0.0, 0.0, []
+        for i in reversed(range(6)):  # cheapest layers first
+            fl = conv_flop(1, CHANNELS[i + 1], HW, HW, CHANNELS[i], 3, 3)
+            if layers and spent > 0 and spent + fl * (spent / done_flop) > args.cpu_seconds:
+                break
+            t0 = time.perf_counter()
+            y = oracle.conv2d(xs[i], wn[i], DIL, DIL, 1, 1, DIL, DIL)
+            oracle.activation(y, "relu")
+            spent += time.perf_counter() - t0
+            done_flop += fl
+            layers.append(i + 1)
+        cpu = {"value": spent * 1e3 * total_flop / done_flop, "unit": "ms",
+               "cores": oracle.num_threads(), "kind": "port",
+               "sample": "oracle conv+ReLU on layers %s of the original dilated block "
+                         "(%.2f of %.2f GFLOP, %.1f s measured), scaled to the whole block by FLOP"
+                         % (sorted(layers), done_flop / 1e9, total_flop / 1e9, spent),
+               "measured_s": spent, "GFLOP/s": done_flop / spent / 1e9}
+
+    out = {
+        "metric": "batch-1 e2e latency ms per PET-optimized graph",
+        "value": ms_opt,
+        "unit": "ms",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": ms_opt,
+        "higher_is_better": False,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f32",
+        "data": "synthetic",
+        "config": {"workload": "dilated-conv block (CSRNet back-end), six 3x3 convs "
+                               "512-512-512-512-256-128-64 on 1x512x64x64, PET space-to-batch "
+                               "program (4x32x32 dense convs + fused ReLU) as one HIP graph",
+                   "global_batch": 1},
+        "original_graph_ms": ms_org,
+        "e2e_TFLOP/s": total_flop / ms_opt / 1e9,
+        "e2e_frac_mfma": total_flop / ms_opt / 1e9 / MFMA_FP32_PEAK_TFLOPS,
+        "roofline": roofline,
+        "cpu_baseline": cpu,
+        "per_op": per_op,
+    }
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

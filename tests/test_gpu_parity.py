@@ -1,8 +1,15 @@
 """GPU parity: every C-ABI operator against the CPU oracle on the same seeded
 inputs. Layout / indexing ops must be bit-exact. Contractions are checked in two
 tiers: small-integer inputs (exact in fp32, so bit-exact against the oracle) and
-real-valued inputs within max relative error 1e-4 (denominator floor as in the
-reference's checker, src/Test/dat/transpose_test/checker_tf.py:66)."""
+real-valued inputs within max relative error 1e-4.
+
+Relative error of output i is |got_i - ref_i| / max(|ref_i|, 1e-3 * A_i), where
+ref is the fp64-accumulated oracle and A_i = sum_k |a_ik| |b_kj| is the same
+contraction on absolute values (also from the oracle). The floor only matters
+for outputs that cancel to below a thousandth of their own terms, where no fp32
+summation order can hold a relative bound; the reference's checker floors the
+denominator for the same reason (src/Test/dat/transpose_test/checker_tf.py:66).
+The normwise error max|got - ref| / max|ref| must meet the same 1e-4."""
 import numpy as np
 import pytest
 import torch
@@ -27,8 +34,13 @@ def ints(rng, shape, lo=-3, hi=4):
     return rng.integers(lo, hi, size=shape).astype(np.float32)
 
 
-def max_rel_err(got, ref):
-    return float(np.max(np.abs(got - ref) / (np.abs(ref) + 0.01))) if ref.size else 0.0
+def max_rel_err(got, ref, mag):
+    """mag: the contraction of |a| and |b| (term magnitude per output)."""
+    if not ref.size:
+        return 0.0
+    elem = np.max(np.abs(got - ref) / np.maximum(np.abs(ref), 1e-3 * mag))
+    norm = np.max(np.abs(got - ref)) / np.max(np.abs(ref))
+    return float(max(elem, norm))
 
 
 @pytest.fixture(scope="module")
@@ -76,8 +88,9 @@ def test_conv2d_float_tier(ops, case):
     x = rng.uniform(-1, 1, (n, c, h, w)).astype(np.float32)
     wt = rng.uniform(-1, 1, (f, cpg, r, s)).astype(np.float32)
     ref = oracle.conv2d(x, wt, ph, pw, sh, sw, dh, dw)
+    mag = oracle.conv2d(np.abs(x), np.abs(wt), ph, pw, sh, sw, dh, dw)
     got = host(ops.conv2d(dev(x), dev(wt), ph, pw, sh, sw, dh, dw))
-    assert max_rel_err(got, ref) <= REL_TOL
+    assert max_rel_err(got, ref, mag) <= REL_TOL
 
 
 def test_conv2d_bias_act_epilogue(ops):
@@ -165,12 +178,13 @@ def test_matmul_float_tier_and_bias_gelu(ops):
     A = rng.standard_normal((2, 128, 768)).astype(np.float32)
     B = (0.02 * rng.standard_normal((2, 768, 256))).astype(np.float32)
     ref = oracle.matmul(A, B)
+    mag = oracle.matmul(np.abs(A), np.abs(B))
     got = host(ops.matmul(dev(A), dev(B)))
-    assert max_rel_err(got, ref) <= REL_TOL
+    assert max_rel_err(got, ref, mag) <= REL_TOL
     bias = rng.standard_normal(256).astype(np.float32)
     ref2 = oracle.bias_act(ref, bias, "gelu", ch_axis=2)
     got2 = host(ops.matmul(dev(A), dev(B), bias=dev(bias), act="gelu"))
-    assert max_rel_err(got2, ref2) <= REL_TOL
+    assert max_rel_err(got2, ref2, mag + np.abs(bias)) <= REL_TOL
 
 
 def test_batch_gemm_merge_identity(ops):
@@ -382,9 +396,10 @@ def test_config1_original_vs_corrected_transform(ops):
     x = rng.uniform(-1, 1, (1, 64, 56, 56)).astype(np.float32)
     w = rng.uniform(-1, 1, (64, 64, 3, 3)).astype(np.float32)
     ref = oracle.conv2d(x, w, 1, 1)
+    mag = oracle.conv2d(np.abs(x), np.abs(w), 1, 1)
     dx, dw = dev(x), dev(w)
     y0 = host(ops.conv2d(dx, dw, 1, 1))
-    assert max_rel_err(y0, ref) <= REL_TOL
+    assert max_rel_err(y0, ref, mag) <= REL_TOL
     halo = ops.trans_chain(dx, [("split", 2, 28, 0, 1), ("reorder", [0, 2, 1, 3, 4]),
                                 ("fuse", 0, 0, 0)])
     assert tuple(halo.shape) == (2, 64, 29, 56)
@@ -392,7 +407,7 @@ def test_config1_original_vs_corrected_transform(ops):
     y1 = host(ops.trans_chain(yt, [("split", 0, 2, 0, 0), ("reorder", [0, 2, 1, 3, 4]),
                                    ("fuse", 2, 0, 1)]))
     assert y1.shape == ref.shape
-    assert max_rel_err(y1, ref) <= REL_TOL
+    assert max_rel_err(y1, ref, mag) <= REL_TOL
     # the oracle's own transformed program agrees with its original one exactly
     oh = oracle.trans_chain(x, [("split", 2, 28, 0, 1), ("reorder", [0, 2, 1, 3, 4]),
                                 ("fuse", 0, 0, 0)])
