@@ -14,6 +14,8 @@
 #include "common.h"
 
 #include <algorithm>
+#include <cstdlib>
+#include <type_traits>
 
 using namespace pet;
 
@@ -21,8 +23,10 @@ namespace {
 
 typedef float floatx16 __attribute__((ext_vector_type(16)));
 
+// Division by a run-time invariant, branch-free: q = (mulhi(n, mul) + (n & add)) >> shift.
+// For d == 1 the multiply contributes nothing and `add` passes n through.
 struct FastDiv {
-    unsigned d, mul, shift;
+    unsigned d, mul, shift, add;
 };
 
 FastDiv make_fastdiv(unsigned d) {
@@ -30,8 +34,10 @@ FastDiv make_fastdiv(unsigned d) {
     f.d = d;
     f.mul = 0;
     f.shift = 0;
+    f.add = 0xFFFFFFFFu;
     if (d <= 1)
         return f;
+    f.add = 0;
     unsigned l = 0;
     while ((1ull << l) < d)
         ++l;
@@ -42,7 +48,7 @@ FastDiv make_fastdiv(unsigned d) {
 }
 
 __device__ __forceinline__ unsigned fd_div(unsigned n, const FastDiv &f) {
-    return f.d == 1 ? n : (__umulhi(n, f.mul) >> f.shift);
+    return (__umulhi(n, f.mul) + (n & f.add)) >> f.shift;
 }
 
 template <int BM_, int BN_, int BK_, int WGM_, int WGN_>
@@ -108,14 +114,32 @@ __device__ __forceinline__ void mma_block(const float *__restrict__ As,
     }
 }
 
+// Sixteen bytes of zeros: a load that must yield 0 (a padding tap, the K tail)
+// is pointed here instead of being masked after the fact, so that no
+// instruction depends on the loaded value until it is written to LDS.
+__device__ __attribute__((aligned(16))) const float g_zero16[4] = {0.f, 0.f, 0.f, 0.f};
+
+// Zeroes v when keep is false without giving the compiler a branch to make.
+__device__ __forceinline__ float keep_if(float v, bool keep) {
+    return __int_as_float(__float_as_int(v) & (keep ? -1 : 0));
+}
+
+__device__ __forceinline__ float4 keep_if(float4 v, bool keep) {
+    const int m = keep ? -1 : 0;
+    return make_float4(__int_as_float(__float_as_int(v.x) & m), __int_as_float(__float_as_int(v.y) & m),
+                       __int_as_float(__float_as_int(v.z) & m), __int_as_float(__float_as_int(v.w) & m));
+}
+
 // ---- operand loaders -----------------------------------------------------------
 // "KC": the operand is stored with K contiguous (weights [f][k], A [m][k],
 // B^T [n][k]); "XC": the non-K index is contiguous (A^T [k][m], B [k][n]).
 // rows = extent of the non-K index, ld = source row stride.
 
-// K-contiguous source -> registers. VEC: ld % 4 == 0 and 16-byte aligned base.
+// K-contiguous source -> registers, branch-free: rows past the end re-read the
+// last row (those accumulator rows are never stored), the K tail is zeroed by a
+// select. VEC: ld % 4 == 0, K % 4 == 0 and a 16-byte aligned base.
 template <int ROWS, int BK, int NT, bool VEC>
-__device__ __forceinline__ void load_kc(const float *__restrict__ src, long long ld, int row0,
+__device__ __forceinline__ void load_kc(const float *__restrict__ src, unsigned ld, int row0,
                                         int rows, int k0, int K, int tid,
                                         float4 (&regs)[ROWS * BK / 4 / NT]) {
     constexpr int VPT = ROWS * BK / 4 / NT;
@@ -123,23 +147,18 @@ __device__ __forceinline__ void load_kc(const float *__restrict__ src, long long
     for (int i = 0; i < VPT; ++i) {
         int v = tid + i * NT;
         int row = v / (BK / 4), kq = (v % (BK / 4)) * 4;
-        int gr = row0 + row, gk = k0 + kq;
-        float4 val = make_float4(0.f, 0.f, 0.f, 0.f);
-        if (gr < rows) {
-            const float *p = src + (long long)gr * ld + gk;
-            if (VEC) {
-                if (gk < K)
-                    val = *reinterpret_cast<const float4 *>(p);
-            } else {
-                if (gk < K)
-                    val.x = p[0];
-                if (gk + 1 < K)
-                    val.y = p[1];
-                if (gk + 2 < K)
-                    val.z = p[2];
-                if (gk + 3 < K)
-                    val.w = p[3];
-            }
+        int gr = min(row0 + row, rows - 1), gk = k0 + kq;
+        const unsigned rbase = (unsigned)gr * ld;
+        float4 val;
+        const float *pz = g_zero16;
+        if (VEC) {
+            const float *q = gk < K ? src + (rbase + (unsigned)gk) : pz;
+            val = *reinterpret_cast<const float4 *>(q);
+        } else {
+            val.x = *(gk < K ? src + (rbase + (unsigned)gk) : pz);
+            val.y = *(gk + 1 < K ? src + (rbase + (unsigned)gk + 1u) : pz);
+            val.z = *(gk + 2 < K ? src + (rbase + (unsigned)gk + 2u) : pz);
+            val.w = *(gk + 3 < K ? src + (rbase + (unsigned)gk + 3u) : pz);
         }
         regs[i] = val;
     }
@@ -174,9 +193,10 @@ __device__ __forceinline__ void store_kc_transposed(float *__restrict__ dst, int
     }
 }
 
-// X-contiguous source (element (x, k) at src[k * ld + x]) -> registers.
+// X-contiguous source (element (x, k) at src[k * ld + x]) -> registers,
+// branch-free in the same way (columns past the end are never stored).
 template <int COLS, int BK, int NT, bool VEC>
-__device__ __forceinline__ void load_xc(const float *__restrict__ src, long long ld, int col0,
+__device__ __forceinline__ void load_xc(const float *__restrict__ src, unsigned ld, int col0,
                                         int cols, int k0, int K, int tid,
                                         float4 (&regs)[COLS * BK / 4 / NT]) {
     constexpr int VPT = COLS * BK / 4 / NT;
@@ -185,22 +205,18 @@ __device__ __forceinline__ void load_xc(const float *__restrict__ src, long long
         int v = tid + i * NT;
         int k = v / (COLS / 4), cq = (v % (COLS / 4)) * 4;
         int gk = k0 + k, gc = col0 + cq;
-        float4 val = make_float4(0.f, 0.f, 0.f, 0.f);
-        if (gk < K) {
-            const float *p = src + (long long)gk * ld + gc;
-            if (VEC) {
-                if (gc < cols)
-                    val = *reinterpret_cast<const float4 *>(p);
-            } else {
-                if (gc < cols)
-                    val.x = p[0];
-                if (gc + 1 < cols)
-                    val.y = p[1];
-                if (gc + 2 < cols)
-                    val.z = p[2];
-                if (gc + 3 < cols)
-                    val.w = p[3];
-            }
+        const unsigned kbase = (unsigned)min(gk, K - 1) * ld;
+        const float *pz = g_zero16;
+        const bool kok = gk < K;
+        float4 val;
+        if (VEC) {
+            const float *q = kok ? src + (kbase + (unsigned)min(gc, cols - 4)) : pz;
+            val = *reinterpret_cast<const float4 *>(q);
+        } else {
+            val.x = *(kok ? src + (kbase + (unsigned)min(gc, cols - 1)) : pz);
+            val.y = *(kok ? src + (kbase + (unsigned)min(gc + 1, cols - 1)) : pz);
+            val.z = *(kok ? src + (kbase + (unsigned)min(gc + 2, cols - 1)) : pz);
+            val.w = *(kok ? src + (kbase + (unsigned)min(gc + 3, cols - 1)) : pz);
         }
         regs[i] = val;
     }
@@ -255,7 +271,7 @@ struct ConvParams {
     int tiles_n;                     // pixel tiles (for the workgroup swizzle)
 };
 
-template <class Cfg, bool VECA>
+template <class Cfg, bool VECA, bool IS3D>
 __global__ __launch_bounds__(Cfg::NT) void conv_igemm_kernel(ConvParams p) {
     __shared__ __attribute__((aligned(16))) float lds[2 * Cfg::STAGE];
     const int tid = threadIdx.x;
@@ -271,39 +287,44 @@ __global__ __launch_bounds__(Cfg::NT) void conv_igemm_kernel(ConvParams p) {
     const float *__restrict__ wg_w = p.w + (long long)g * p.M * p.K;
     const float *__restrict__ wg_x = p.x + (long long)g * p.cpg * THW;
 
-    // per-lane pixel state: PPL pixels, fixed for the whole kernel
+    // per-lane pixel state: PPL pixels, fixed for the whole kernel. Pixels past
+    // the end alias the last pixel; their accumulator columns are never stored.
     int pbase[Cfg::PPL], it0[Cfg::PPL], ih0[Cfg::PPL], iw0[Cfg::PPL];
 #pragma unroll
     for (int pp = 0; pp < Cfg::PPL; ++pp) {
-        int pix = n0 + lane + pp * 64;
-        if (pix < p.NPIX) {
-            unsigned n = fd_div(pix, p.fd_opix);
-            unsigned rem = pix - n * p.OPIX;
-            unsigned ot = fd_div(rem, p.fd_ohw);
+        int pix = min(n0 + lane + pp * 64, p.NPIX - 1);
+        unsigned n = fd_div(pix, p.fd_opix);
+        unsigned rem = pix - n * p.OPIX;
+        unsigned ot = 0;
+        if (IS3D) {
+            ot = fd_div(rem, p.fd_ohw);
             rem -= ot * (p.OH * p.OW);
-            unsigned oh = fd_div(rem, p.fd_ow);
-            unsigned ow = rem - oh * p.OW;
-            it0[pp] = (int)ot * p.st - p.pt;
-            ih0[pp] = (int)oh * p.sh - p.ph;
-            iw0[pp] = (int)ow * p.sw - p.pw;
-            pbase[pp] = (int)n * p.C * THW + it0[pp] * HW + ih0[pp] * p.W + iw0[pp];
-        } else {
-            it0[pp] = ih0[pp] = iw0[pp] = -(1 << 28); // never in range
-            pbase[pp] = 0;
         }
+        unsigned oh = fd_div(rem, p.fd_ow);
+        unsigned ow = rem - oh * p.OW;
+        it0[pp] = IS3D ? (int)ot * p.st - p.pt : 0;
+        ih0[pp] = (int)oh * p.sh - p.ph;
+        iw0[pp] = (int)ow * p.sw - p.pw;
+        pbase[pp] = (int)n * p.C * THW + it0[pp] * HW + ih0[pp] * p.W + iw0[pp];
     }
 
     float4 areg[Cfg::A_VPT];
     float breg[Cfg::RPW][Cfg::PPL];
 
+    // Branch-free im2col gather: the k index of a row is wave-uniform, so its
+    // (c, kt, r, s) split runs on the scalar unit; a tap outside the image (or
+    // past K) reads offset 0 and is replaced by 0 with a select.
     auto gather_b = [&](int k0) {
 #pragma unroll
         for (int i = 0; i < Cfg::RPW; ++i) {
-            const int k = k0 + wave + Cfg::NW * i; // wave-uniform
+            const int k = k0 + wave + Cfg::NW * i;
             const unsigned c = fd_div(k, p.fd_krs);
             unsigned rem = k - c * p.fd_krs.d;
-            const unsigned q = fd_div(rem, p.fd_rs);
-            rem -= q * p.fd_rs.d;
+            unsigned q = 0;
+            if (IS3D) {
+                q = fd_div(rem, p.fd_rs);
+                rem -= q * p.fd_rs.d;
+            }
             const unsigned r = fd_div(rem, p.fd_s);
             const unsigned s = rem - r * p.fd_s.d;
             const int qt = (int)q * p.dt, rh = (int)r * p.dh, sw_ = (int)s * p.dw;
@@ -311,13 +332,12 @@ __global__ __launch_bounds__(Cfg::NT) void conv_igemm_kernel(ConvParams p) {
             const bool kok = k < p.K;
 #pragma unroll
             for (int pp = 0; pp < Cfg::PPL; ++pp) {
-                bool ok = kok && (unsigned)(it0[pp] + qt) < (unsigned)p.T &&
-                          (unsigned)(ih0[pp] + rh) < (unsigned)p.H &&
-                          (unsigned)(iw0[pp] + sw_) < (unsigned)p.W;
-                float v = 0.f;
-                if (ok)
-                    v = wg_x[pbase[pp] + koff];
-                breg[i][pp] = v;
+                bool ok = kok & ((unsigned)(ih0[pp] + rh) < (unsigned)p.H) &
+                          ((unsigned)(iw0[pp] + sw_) < (unsigned)p.W);
+                if (IS3D)
+                    ok = ok & ((unsigned)(it0[pp] + qt) < (unsigned)p.T);
+                const float *q = ok ? wg_x + (unsigned)(pbase[pp] + koff) : g_zero16;
+                breg[i][pp] = *q;
             }
         }
     };
@@ -345,21 +365,23 @@ __global__ __launch_bounds__(Cfg::NT) void conv_igemm_kernel(ConvParams p) {
     store_b(lds + Cfg::A_ELEMS);
     __syncthreads();
 
-    for (int kt = 0; kt < nk; ++kt) {
+    // main loop (all but the last K block): prefetch kt+1 while computing kt
+    for (int kt = 0; kt < nk - 1; ++kt) {
         float *cur = lds + (kt & 1) * Cfg::STAGE;
         float *nxt = lds + ((kt + 1) & 1) * Cfg::STAGE;
-        const bool more = kt + 1 < nk;
-        if (more) {
-            load_kc<Cfg::BM, Cfg::BK, Cfg::NT, VECA>(wg_w, p.K, m0, p.M, (kt + 1) * Cfg::BK, p.K,
-                                                     tid, areg);
-            gather_b((kt + 1) * Cfg::BK);
-        }
+        load_kc<Cfg::BM, Cfg::BK, Cfg::NT, VECA>(wg_w, p.K, m0, p.M, (kt + 1) * Cfg::BK, p.K, tid,
+                                                 areg);
+        gather_b((kt + 1) * Cfg::BK);
+        __builtin_amdgcn_sched_barrier(0); // keep the prefetch ahead of the MFMA block
         mma_block<Cfg>(cur, cur + Cfg::A_ELEMS, acc, wm0, wn0, lane);
-        if (more) {
-            store_kc_rowmajor<Cfg::BM, Cfg::BK, Cfg::NT, Cfg::A_LD>(nxt, tid, areg);
-            store_b(nxt + Cfg::A_ELEMS);
-        }
+        __builtin_amdgcn_sched_barrier(0);
+        store_kc_rowmajor<Cfg::BM, Cfg::BK, Cfg::NT, Cfg::A_LD>(nxt, tid, areg);
+        store_b(nxt + Cfg::A_ELEMS);
         __syncthreads();
+    }
+    {
+        float *cur = lds + ((nk - 1) & 1) * Cfg::STAGE;
+        mma_block<Cfg>(cur, cur + Cfg::A_ELEMS, acc, wm0, wn0, lane);
     }
 
     // epilogue: bias + activation, NC(T)HW store. Lane holds column l%32 and
@@ -372,7 +394,8 @@ __global__ __launch_bounds__(Cfg::NT) void conv_igemm_kernel(ConvParams p) {
             continue;
         unsigned n = fd_div(pix, p.fd_opix);
         unsigned rem = pix - n * p.OPIX;
-        long long obase = ((long long)n * p.F + (long long)g * p.M) * p.OPIX + rem;
+        float *__restrict__ yb = p.y + (((long long)n * p.F + (long long)g * p.M) * p.OPIX + rem);
+        const float *__restrict__ bias = p.bias ? p.bias + g * p.M : nullptr;
 #pragma unroll
         for (int tm = 0; tm < Cfg::TM; ++tm) {
 #pragma unroll
@@ -380,9 +403,556 @@ __global__ __launch_bounds__(Cfg::NT) void conv_igemm_kernel(ConvParams p) {
                 int f = m0 + wm0 + tm * 32 + (r / 4) * 8 + hk * 4 + (r % 4);
                 if (f < p.M) {
                     float v = acc[tm][tn][r];
-                    if (p.bias)
-                        v += p.bias[g * p.M + f];
-                    p.y[obase + (long long)f * p.OPIX] = apply_act(v, p.act);
+                    if (bias)
+                        v += bias[f];
+                    yb[(unsigned)f * (unsigned)p.OPIX] = apply_act(v, p.act);
+                }
+            }
+        }
+    }
+}
+
+// Software-pipelined variant of the convolution kernel. With one or two waves
+// per SIMD nothing but the wave's own instruction stream can hide latency, so
+// the K loop is written as NM "slots", one MFMA each, and the other work of the
+// iteration is dealt out between them in a fixed order:
+//   G(kt+2): global -> prefetch registers   (two register sets, so a load has
+//                                            more than a full iteration to land)
+//   W(kt+1): prefetch registers -> LDS
+//   barrier
+//   R(kt+1): LDS -> fragment registers      (two sets: MFMAs of tile kt read
+//                                            one while the other is filled)
+// The MFMAs of tile kt therefore straddle the barrier and never wait on LDS.
+template <class Cfg, bool VECA, bool IS3D>
+__global__ __launch_bounds__(Cfg::NT) void conv_pipe_kernel(ConvParams p) {
+    __shared__ __attribute__((aligned(16))) float lds[2 * Cfg::STAGE];
+    constexpr int KH = Cfg::KH, TM = Cfg::TM, TN = Cfg::TN;
+    constexpr int BK = Cfg::BK, NT = Cfg::NT, NW = Cfg::NW;
+    constexpr int A_VPT = Cfg::A_VPT, RPW = Cfg::RPW, PPL = Cfg::PPL;
+    constexpr int A_LD = Cfg::A_LD, B_LD = Cfg::B_LD;
+    constexpr int NM = KH * TM * TN;       // MFMAs (slots) per iteration
+    constexpr int NG = A_VPT + RPW;        // prefetch pieces
+    constexpr int NWP = NG;                // LDS-write pieces
+    constexpr int NRA = TM * (KH / 4);     // A fragment pieces (128-bit reads)
+    constexpr int NR = NRA + KH;           // fragment pieces
+    constexpr int NP = NG + NWP + 1 + NR;  // + the barrier
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wm0 = (wave / Cfg::WGN) * Cfg::WM;
+    const int wn0 = (wave % Cfg::WGN) * Cfg::WN;
+    const int l32 = lane & 31, hk = lane >> 5;
+    const int g = blockIdx.z;
+    const int m0 = blockIdx.y * Cfg::BM;
+    const int n0 = blockIdx.x * Cfg::BN;
+
+    const int THW = p.T * p.H * p.W, HW = p.H * p.W;
+    const float *__restrict__ wg_w = p.w + (long long)g * p.M * p.K;
+    const float *__restrict__ wg_x = p.x + (long long)g * p.cpg * THW;
+
+    int pbase[PPL], it0[PPL], ih0[PPL], iw0[PPL];
+#pragma unroll
+    for (int pp = 0; pp < PPL; ++pp) {
+        int pix = min(n0 + lane + pp * 64, p.NPIX - 1);
+        unsigned n = fd_div(pix, p.fd_opix);
+        unsigned rem = pix - n * p.OPIX;
+        unsigned ot = 0;
+        if (IS3D) {
+            ot = fd_div(rem, p.fd_ohw);
+            rem -= ot * (p.OH * p.OW);
+        }
+        unsigned oh = fd_div(rem, p.fd_ow);
+        unsigned ow = rem - oh * p.OW;
+        it0[pp] = IS3D ? (int)ot * p.st - p.pt : 0;
+        ih0[pp] = (int)oh * p.sh - p.ph;
+        iw0[pp] = (int)ow * p.sw - p.pw;
+        pbase[pp] = (int)n * p.C * THW + it0[pp] * HW + ih0[pp] * p.W + iw0[pp];
+    }
+    // fixed A-load coordinates of this thread
+    unsigned a_rbase[A_VPT];
+    int a_kq[A_VPT], a_lds[A_VPT];
+#pragma unroll
+    for (int i = 0; i < A_VPT; ++i) {
+        int v = tid + i * NT;
+        int row = v / (BK / 4);
+        a_kq[i] = (v % (BK / 4)) * 4;
+        a_rbase[i] = (unsigned)min(m0 + row, p.M - 1) * (unsigned)p.K;
+        a_lds[i] = row * A_LD + a_kq[i];
+    }
+    const int a_frag = (wm0 + l32) * A_LD + hk * KH;         // + tm*32*A_LD + j
+    const int b_frag = hk * KH * B_LD + wn0 + l32;            // + j*B_LD + tn*32
+    const int b_lds = wave * B_LD + lane;                     // + NW*i*B_LD + pp*64
+
+    float4 preA[2][A_VPT];
+    float preB[2][RPW][PPL];
+    float fa[2][TM][KH];
+    float fb[2][KH][TN];
+    floatx16 acc[TM][TN];
+#pragma unroll
+    for (int tm = 0; tm < TM; ++tm)
+#pragma unroll
+        for (int tn = 0; tn < TN; ++tn)
+#pragma unroll
+            for (int r = 0; r < 16; ++r)
+                acc[tm][tn][r] = 0.f;
+
+    // ---- the pieces; `i` and `set` are constants once the callers are unrolled
+    auto g_piece = [&](int set, int i, int k0) __attribute__((always_inline)) {
+        if (i < A_VPT) {
+            const int gk = k0 + a_kq[i];
+            float4 val;
+            const float *pz = g_zero16;
+            if (VECA) {
+                const float *q = gk < p.K ? wg_w + (a_rbase[i] + (unsigned)gk) : pz;
+                val = *reinterpret_cast<const float4 *>(q);
+            } else {
+                val.x = *(gk < p.K ? wg_w + (a_rbase[i] + (unsigned)gk) : pz);
+                val.y = *(gk + 1 < p.K ? wg_w + (a_rbase[i] + (unsigned)gk + 1u) : pz);
+                val.z = *(gk + 2 < p.K ? wg_w + (a_rbase[i] + (unsigned)gk + 2u) : pz);
+                val.w = *(gk + 3 < p.K ? wg_w + (a_rbase[i] + (unsigned)gk + 3u) : pz);
+            }
+            preA[set][i] = val;
+        } else {
+            const int row = i - A_VPT;
+            const int k = k0 + wave + NW * row; // wave-uniform: scalar unit
+            const unsigned c = fd_div(k, p.fd_krs);
+            unsigned rem = k - c * p.fd_krs.d;
+            unsigned q = 0;
+            if (IS3D) {
+                q = fd_div(rem, p.fd_rs);
+                rem -= q * p.fd_rs.d;
+            }
+            const unsigned r = fd_div(rem, p.fd_s);
+            const unsigned s = rem - r * p.fd_s.d;
+            const int qt = (int)q * p.dt, rh = (int)r * p.dh, sw_ = (int)s * p.dw;
+            const int koff = (int)c * THW + qt * HW + rh * p.W + sw_;
+            const bool kok = k < p.K;
+#pragma unroll
+            for (int pp = 0; pp < PPL; ++pp) {
+                bool ok = kok & ((unsigned)(ih0[pp] + rh) < (unsigned)p.H) &
+                          ((unsigned)(iw0[pp] + sw_) < (unsigned)p.W);
+                if (IS3D)
+                    ok = ok & ((unsigned)(it0[pp] + qt) < (unsigned)p.T);
+                const float *q = ok ? wg_x + (unsigned)(pbase[pp] + koff) : g_zero16;
+                preB[set][row][pp] = *q;
+            }
+        }
+    };
+    auto w_piece = [&](int set, int i, float *st) __attribute__((always_inline)) {
+        if (i < A_VPT) {
+            *reinterpret_cast<float4 *>(st + a_lds[i]) = preA[set][i];
+        } else {
+            const int row = i - A_VPT;
+#pragma unroll
+            for (int pp = 0; pp < PPL; ++pp)
+                st[Cfg::A_ELEMS + b_lds + NW * row * B_LD + pp * 64] = preB[set][row][pp];
+        }
+    };
+    auto r_piece = [&](int set, int i, const float *st) __attribute__((always_inline)) {
+        if (i < NRA) {
+            const int tm = i / (KH / 4), jq = (i % (KH / 4)) * 4;
+            float4 v = *reinterpret_cast<const float4 *>(st + a_frag + tm * 32 * A_LD + jq);
+            fa[set][tm][jq] = v.x;
+            fa[set][tm][jq + 1] = v.y;
+            fa[set][tm][jq + 2] = v.z;
+            fa[set][tm][jq + 3] = v.w;
+        } else {
+            const int j = i - NRA;
+#pragma unroll
+            for (int tn = 0; tn < TN; ++tn)
+                fb[set][j][tn] = st[Cfg::A_ELEMS + b_frag + j * B_LD + tn * 32];
+        }
+    };
+    auto wg_barrier = [&]() __attribute__((always_inline)) {
+        // LDS writes done, then the workgroup barrier; global prefetches stay in flight
+        asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+    };
+
+    const int nk = (p.K + BK - 1) / BK;
+
+    // ---- prologue: tiles 0 and 1 into the prefetch sets, tile 0 into LDS and fragments
+#pragma unroll
+    for (int i = 0; i < NG; ++i)
+        g_piece(0, i, 0);
+#pragma unroll
+    for (int i = 0; i < NG; ++i)
+        g_piece(1, i, BK);
+#pragma unroll
+    for (int i = 0; i < NWP; ++i)
+        w_piece(0, i, lds);
+    wg_barrier();
+#pragma unroll
+    for (int i = 0; i < NR; ++i)
+        r_piece(0, i, lds);
+
+    // one iteration: PAR = kt & 1 selects the register sets
+    auto iteration = [&](auto parc, int kt) __attribute__((always_inline)) {
+        constexpr int PAR = decltype(parc)::value;
+        float *nxt = lds + (PAR ^ 1) * Cfg::STAGE;
+        const int kpre = (kt + 2) * BK;
+#pragma unroll
+        for (int s = 0; s < NM; ++s) {
+            const int j = s / (TM * TN), tm = (s / TN) % TM, tn = s % TN;
+            acc[tm][tn] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[PAR][tm][j], fb[PAR][j][tn],
+                                                               acc[tm][tn], 0, 0, 0);
+            const int pb = (s * NP + NM - 1) / NM, pe = ((s + 1) * NP + NM - 1) / NM;
+#pragma unroll
+            for (int q = pb; q < pe; ++q) {
+                if (q < NG)
+                    g_piece(PAR, q, kpre);
+                else if (q < NG + NWP)
+                    w_piece(PAR ^ 1, q - NG, nxt);
+                else if (q == NG + NWP)
+                    wg_barrier();
+                else
+                    r_piece(PAR ^ 1, q - NG - NWP - 1, nxt);
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        }
+    };
+    int kt = 0;
+    for (; kt + 1 < nk; kt += 2) {
+        iteration(std::integral_constant<int, 0>{}, kt);
+        iteration(std::integral_constant<int, 1>{}, kt + 1);
+    }
+    if (kt < nk)
+        iteration(std::integral_constant<int, 0>{}, kt);
+
+    // epilogue: bias + activation, NC(T)HW store
+#pragma unroll
+    for (int tn = 0; tn < TN; ++tn) {
+        int pix = n0 + wn0 + tn * 32 + l32;
+        if (pix >= p.NPIX)
+            continue;
+        unsigned n = fd_div(pix, p.fd_opix);
+        unsigned rem = pix - n * p.OPIX;
+        float *__restrict__ yb = p.y + (((long long)n * p.F + (long long)g * p.M) * p.OPIX + rem);
+        const float *__restrict__ bias = p.bias ? p.bias + g * p.M : nullptr;
+#pragma unroll
+        for (int tm = 0; tm < TM; ++tm) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                int f = m0 + wm0 + tm * 32 + (r / 4) * 8 + hk * 4 + (r % 4);
+                if (f < p.M) {
+                    float v = acc[tm][tn][r];
+                    if (bias)
+                        v += bias[f];
+                    yb[(unsigned)f * (unsigned)p.OPIX] = apply_act(v, p.act);
+                }
+            }
+        }
+    }
+}
+
+// ---- "plane" convolution kernel ----------------------------------------------------
+// The fast path for filters whose (r, s) plane is small (3x3, 1x1, also 3x3x3
+// taken one kt slice at a time). One K step covers CB input channels times the
+// whole RS = r*s plane, so the tap of a B-tile row, its offset inside the image
+// and whether it falls into the padding are the same in every step: they are
+// worked out once per thread. The loads are raw buffer loads whose voffset is
+// that fixed byte offset, or 2^31 for a padding tap, which the buffer range
+// check answers with 0; the step only moves the scalar base. Per element and
+// step the wave issues one load and half a ds_write and no address arithmetic,
+// which is what lets one wave per SIMD keep the MFMA pipe busy: a wave issues
+// at most one instruction every four cycles, so the whole step has to fit in
+// 16 instructions per MFMA.
+//
+// Schedule of step kt (NM slots, one MFMA each): first half, W(kt+1): prefetch
+// registers -> LDS; barrier; second half, R(kt+1): LDS -> the other fragment
+// register set, and G(kt+2): global -> prefetch registers.
+template <int BM_, int BN_, int WGM_, int WGN_, int RS_, int CB_>
+struct PlaneCfg {
+    static constexpr int BM = BM_, BN = BN_, WGM = WGM_, WGN = WGN_, RS = RS_, CB = CB_;
+    static constexpr int BK = RS * CB;
+    static constexpr int NW = WGM * WGN, NT = NW * 64;
+    static constexpr int WM = BM / WGM, WN = BN / WGN;
+    static constexpr int TM = WM / 32, TN = WN / 32;
+    static constexpr int KH = BK / 2;
+    static constexpr int A_LD = BK + 4, B_LD = BN + 4;
+    static constexpr int A_ELEMS = BM * A_LD, B_ELEMS = BK * B_LD;
+    static constexpr int STAGE = A_ELEMS + B_ELEMS;
+    static constexpr int RPW = BK / NW, PPL = BN / 64;
+    static constexpr int A_V4 = BM * BK / 4;              // float4 per A tile (2-D)
+    static constexpr int A_VPT = (A_V4 + NT - 1) / NT;
+    static constexpr int A_SPT = BM * BK / NT;            // scalars per thread (3-D)
+    static_assert(WM % 32 == 0 && WN % 32 == 0 && KH % 4 == 0 && BK % NW == 0 && BN % 64 == 0 &&
+                      (BM * BK) % NT == 0,
+                  "bad plane tile");
+};
+
+typedef unsigned uintx4 __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void *base) {
+    // raw buffer, stride 0, 2 GiB of records, 32-bit float format
+    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(base), 0, 0x80000000, 0x00020000);
+}
+
+constexpr unsigned kOob = 0x80000000u; // voffset that the range check rejects
+
+template <class Cfg, bool IS3D>
+__global__ __launch_bounds__(Cfg::NT) void conv_plane_kernel(ConvParams p) {
+    extern __shared__ __attribute__((aligned(16))) float lds[];
+    constexpr int KH = Cfg::KH, TM = Cfg::TM, TN = Cfg::TN, RS = Cfg::RS, CB = Cfg::CB;
+    constexpr int BK = Cfg::BK, NT = Cfg::NT, NW = Cfg::NW;
+    constexpr int RPW = Cfg::RPW, PPL = Cfg::PPL;
+    constexpr int A_LD = Cfg::A_LD, B_LD = Cfg::B_LD;
+    constexpr int NA = IS3D ? Cfg::A_SPT : Cfg::A_VPT; // A pieces per thread
+    constexpr int NM = KH * TM * TN;                   // slots per step
+    constexpr int HALF = NM / 2;
+    constexpr int NWP = NA + RPW;                      // W pieces (first half)
+    constexpr int NRA = TM * (KH / 4);
+    constexpr int NR = NRA + KH;                       // R pieces
+    constexpr int NG = NA + RPW;                       // G pieces
+    constexpr int NPOST = NR + NG;                     // second half
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const int wm0 = (wave / Cfg::WGN) * Cfg::WM;
+    const int wn0 = (wave % Cfg::WGN) * Cfg::WN;
+    const int l32 = lane & 31, hk = lane >> 5;
+    const int g = blockIdx.z;
+    const int m0 = blockIdx.y * Cfg::BM;
+    const int n0 = blockIdx.x * Cfg::BN;
+
+    const int THW = p.T * p.H * p.W, HW = p.H * p.W;
+    const int KRS = p.KT * RS; // weights per (f, c)
+    // bases: the pad offset is folded into the image base so every voffset is >= 0
+    const int padoff = p.pt * HW + p.ph * p.W + p.pw;
+    const float *xg = p.x + (long long)g * p.cpg * THW - padoff;
+    const float *wg = p.w + (long long)g * p.M * p.K;
+
+    // ---- per-thread invariants of the B gather
+    unsigned voffB[RPW][PPL];
+    int it0[PPL];
+    {
+        int oh_[PPL], ow_[PPL];
+        unsigned pb[PPL];
+#pragma unroll
+        for (int pp = 0; pp < PPL; ++pp) {
+            int pix = min(n0 + lane + pp * 64, p.NPIX - 1);
+            unsigned n = fd_div(pix, p.fd_opix);
+            unsigned rem = pix - n * p.OPIX;
+            unsigned ot = 0;
+            if (IS3D) {
+                ot = fd_div(rem, p.fd_ohw);
+                rem -= ot * (p.OH * p.OW);
+            }
+            unsigned oh = fd_div(rem, p.fd_ow);
+            unsigned ow = rem - oh * p.OW;
+            it0[pp] = (int)ot * p.st - p.pt;
+            oh_[pp] = (int)oh * p.sh;
+            ow_[pp] = (int)ow * p.sw;
+            pb[pp] = n * (unsigned)(p.C * THW) + ot * (unsigned)(p.st * HW) + oh_[pp] * p.W + ow_[pp];
+        }
+#pragma unroll
+        for (int i = 0; i < RPW; ++i) {
+            const int kl = wave + NW * i; // row of the B tile: (c_local, r, s)
+            const int cl = kl / RS, t = kl % RS;
+            const int r = t / p.S, s = t - r * p.S;
+            const int rh = r * p.dh, sw_ = s * p.dw;
+            const unsigned roff = (unsigned)(cl * THW + rh * p.W + sw_);
+#pragma unroll
+            for (int pp = 0; pp < PPL; ++pp) {
+                const bool ok = ((unsigned)(oh_[pp] + rh - p.ph) < (unsigned)p.H) &
+                                ((unsigned)(ow_[pp] + sw_ - p.pw) < (unsigned)p.W);
+                voffB[i][pp] = ok ? (pb[pp] + roff) * 4u : kOob;
+            }
+        }
+    }
+    // ---- per-thread invariants of the A loads
+    unsigned voffA[NA];
+    int ldsA[NA];
+#pragma unroll
+    for (int i = 0; i < NA; ++i) {
+        if (IS3D) {
+            const int e = tid + i * NT;
+            const int f = e / BK, kl = e % BK;
+            const int cl = kl / RS, t = kl % RS;
+            voffA[i] = ((unsigned)min(m0 + f, p.M - 1) * (unsigned)p.K + cl * KRS + t) * 4u;
+            ldsA[i] = f * A_LD + kl;
+        } else {
+            const int v = tid + i * NT;
+            const int row = v / (BK / 4), kq = (v % (BK / 4)) * 4;
+            voffA[i] = v < Cfg::A_V4
+                           ? ((unsigned)min(m0 + row, p.M - 1) * (unsigned)p.K + kq) * 4u
+                           : kOob;
+            ldsA[i] = min(row, Cfg::BM - 1) * A_LD + kq;
+        }
+    }
+    const int a_frag = (wm0 + l32) * A_LD + hk * KH;
+    const int b_frag = Cfg::A_ELEMS + hk * KH * B_LD + wn0 + l32;
+    const int b_lds = Cfg::A_ELEMS + wave * B_LD + lane;
+
+    float4 preA4[IS3D ? 1 : NA];
+    float preA1[IS3D ? NA : 1];
+    float preB[RPW][PPL];
+    float fa[2][TM][KH];
+    float fb[2][KH][TN];
+    floatx16 acc[TM][TN];
+#pragma unroll
+    for (int tm = 0; tm < TM; ++tm)
+#pragma unroll
+        for (int tn = 0; tn < TN; ++tn)
+#pragma unroll
+            for (int r = 0; r < 16; ++r)
+                acc[tm][tn][r] = 0.f;
+
+    // step counters of the prefetch stream: channel block and kt slice
+    const int ncb = p.cpg / CB;
+    const int nit = ncb * p.KT;
+    int pcb = 0, pq = 0;
+    auto advance_prefetch = [&]() __attribute__((always_inline)) {
+        // stays on the last step once the end is reached (harmless re-load)
+        if (pcb * p.KT + pq + 1 < nit) {
+            if (++pq == p.KT) {
+                pq = 0;
+                ++pcb;
+            }
+        }
+    };
+
+    // ---- pieces ---------------------------------------------------------------
+    auto g_piece = [&](int i) __attribute__((always_inline)) {
+        if (i < NA) {
+            const unsigned so = (unsigned)(pcb * CB * KRS + pq * RS) * 4u;
+            const __amdgpu_buffer_rsrc_t ra = make_rsrc(wg);
+            if (IS3D) {
+                preA1[i] = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(ra, voffA[i], so, 0));
+            } else {
+                uintx4 v = __builtin_amdgcn_raw_buffer_load_b128(ra, voffA[i], so, 0);
+                preA4[i] = make_float4(__uint_as_float(v.x), __uint_as_float(v.y),
+                                       __uint_as_float(v.z), __uint_as_float(v.w));
+            }
+        } else {
+            const int row = i - NA;
+            const unsigned so = (unsigned)(pcb * CB * THW + pq * p.dt * HW) * 4u;
+            const __amdgpu_buffer_rsrc_t rb = make_rsrc(xg);
+#pragma unroll
+            for (int pp = 0; pp < PPL; ++pp) {
+                unsigned vo = voffB[row][pp];
+                if (IS3D)
+                    vo = (unsigned)(it0[pp] + pq * p.dt) < (unsigned)p.T ? vo : kOob;
+                preB[row][pp] = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(rb, vo, so, 0));
+            }
+        }
+    };
+    auto w_piece = [&](int i, float *st) __attribute__((always_inline)) {
+        if (i < NA) {
+            if (IS3D) {
+                st[ldsA[i]] = preA1[i];
+            } else {
+                // the last, partly filled round only exists for the first threads
+                if ((i + 1) * NT <= Cfg::A_V4 || tid + i * NT < Cfg::A_V4)
+                    *reinterpret_cast<float4 *>(st + ldsA[i]) = preA4[i];
+            }
+        } else {
+            const int row = i - NA;
+#pragma unroll
+            for (int pp = 0; pp < PPL; ++pp)
+                st[b_lds + NW * row * B_LD + pp * 64] = preB[row][pp];
+        }
+    };
+    auto r_piece = [&](int set, int i, const float *st) __attribute__((always_inline)) {
+        if (i < NRA) {
+            const int tm = i / (KH / 4), jq = (i % (KH / 4)) * 4;
+            float4 v = *reinterpret_cast<const float4 *>(st + a_frag + tm * 32 * A_LD + jq);
+            fa[set][tm][jq] = v.x;
+            fa[set][tm][jq + 1] = v.y;
+            fa[set][tm][jq + 2] = v.z;
+            fa[set][tm][jq + 3] = v.w;
+        } else {
+            const int j = i - NRA;
+#pragma unroll
+            for (int tn = 0; tn < TN; ++tn)
+                fb[set][j][tn] = st[b_frag + j * B_LD + tn * 32];
+        }
+    };
+    auto wg_barrier = [&]() __attribute__((always_inline)) {
+        asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+    };
+
+    // ---- prologue: step 0 into LDS and fragment set 0, step 1 into the prefetch registers
+#pragma unroll
+    for (int i = 0; i < NG; ++i)
+        g_piece(i);
+    advance_prefetch();
+#pragma unroll
+    for (int i = 0; i < NWP; ++i)
+        w_piece(i, lds);
+    wg_barrier();
+#pragma unroll
+    for (int i = 0; i < NR; ++i)
+        r_piece(0, i, lds);
+#pragma unroll
+    for (int i = 0; i < NG; ++i)
+        g_piece(i);
+    advance_prefetch();
+
+    auto step = [&](auto parc) __attribute__((always_inline)) {
+        constexpr int PAR = decltype(parc)::value;
+        float *nxt = lds + (PAR ^ 1) * Cfg::STAGE;
+#pragma unroll
+        for (int s = 0; s < NM; ++s) {
+            const int j = s / (TM * TN), tm = (s / TN) % TM, tn = s % TN;
+            acc[tm][tn] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[PAR][tm][j], fb[PAR][j][tn],
+                                                               acc[tm][tn], 0, 0, 0);
+            if (s < HALF) {
+                const int pb_ = (s * NWP + HALF - 1) / HALF, pe_ = ((s + 1) * NWP + HALF - 1) / HALF;
+#pragma unroll
+                for (int q = pb_; q < pe_; ++q)
+                    w_piece(q, nxt);
+                if (s == HALF - 1)
+                    wg_barrier();
+            } else {
+                const int h = s - HALF, HN = NM - HALF;
+                const int pb_ = (h * NPOST + HN - 1) / HN, pe_ = ((h + 1) * NPOST + HN - 1) / HN;
+#pragma unroll
+                for (int q = pb_; q < pe_; ++q) {
+                    // fragment reads first in each pair, prefetches after
+                    if (q < 2 * NG) {
+                        if (q & 1)
+                            g_piece(q >> 1);
+                        else
+                            r_piece(PAR ^ 1, q >> 1, nxt);
+                    } else {
+                        r_piece(PAR ^ 1, q - NG, nxt);
+                    }
+                }
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        advance_prefetch();
+    };
+    int kt = 0;
+    for (; kt + 1 < nit; kt += 2) {
+        step(std::integral_constant<int, 0>{});
+        step(std::integral_constant<int, 1>{});
+    }
+    if (kt < nit)
+        step(std::integral_constant<int, 0>{});
+
+    // epilogue: bias + activation, NC(T)HW store
+#pragma unroll
+    for (int tn = 0; tn < TN; ++tn) {
+        int pix = n0 + wn0 + tn * 32 + l32;
+        if (pix >= p.NPIX)
+            continue;
+        unsigned n = fd_div(pix, p.fd_opix);
+        unsigned rem = pix - n * p.OPIX;
+        float *__restrict__ yb = p.y + (((long long)n * p.F + (long long)g * p.M) * p.OPIX + rem);
+        const float *__restrict__ bias = p.bias ? p.bias + g * p.M : nullptr;
+#pragma unroll
+        for (int tm = 0; tm < TM; ++tm) {
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                int f = m0 + wm0 + tm * 32 + (r / 4) * 8 + hk * 4 + (r % 4);
+                if (f < p.M) {
+                    float v = acc[tm][tn][r];
+                    if (bias)
+                        v += bias[f];
+                    yb[(unsigned)f * (unsigned)p.OPIX] = apply_act(v, p.act);
                 }
             }
         }
@@ -451,16 +1021,19 @@ __global__ __launch_bounds__(Cfg::NT) void bmm_kernel(GemmParams p) {
     load_tiles(0);
     store_tiles(lds);
     __syncthreads();
-    for (int kt = 0; kt < nk; ++kt) {
+    for (int kt = 0; kt < nk - 1; ++kt) {
         float *cur = lds + (kt & 1) * Cfg::STAGE;
         float *nxt = lds + ((kt + 1) & 1) * Cfg::STAGE;
-        const bool more = kt + 1 < nk;
-        if (more)
-            load_tiles((kt + 1) * Cfg::BK);
+        load_tiles((kt + 1) * Cfg::BK);
+        __builtin_amdgcn_sched_barrier(0); // keep the prefetch ahead of the MFMA block
         mma_block<Cfg>(cur, cur + Cfg::A_ELEMS, acc, wm0, wn0, lane);
-        if (more)
-            store_tiles(nxt);
+        __builtin_amdgcn_sched_barrier(0);
+        store_tiles(nxt);
         __syncthreads();
+    }
+    {
+        float *cur = lds + ((nk - 1) & 1) * Cfg::STAGE;
+        mma_block<Cfg>(cur, cur + Cfg::A_ELEMS, acc, wm0, wn0, lane);
     }
 
     const int l32 = lane & 31, hk = lane >> 5;
@@ -487,14 +1060,49 @@ using Cfg128x128 = TileCfg<128, 128, 16, 2, 2>;
 using Cfg64x128 = TileCfg<64, 128, 16, 2, 2>;
 using Cfg64x64 = TileCfg<64, 64, 16, 2, 2>;
 using Cfg32x64 = TileCfg<32, 64, 16, 1, 2>;
+using Cfg64x64k32 = TileCfg<64, 64, 32, 2, 2>;
+using Cfg64x64k64 = TileCfg<64, 64, 64, 2, 2>;
+using Cfg64x128k32 = TileCfg<64, 128, 32, 2, 2>;
+using Cfg128x128k32 = TileCfg<128, 128, 32, 2, 2>;
 
 template <class Cfg>
 int launch_conv_cfg(const ConvParams &p, bool veca, hipStream_t stream) {
     dim3 grid((p.NPIX + Cfg::BN - 1) / Cfg::BN, (p.M + Cfg::BM - 1) / Cfg::BM, p.G);
-    if (veca)
-        hipLaunchKernelGGL((conv_igemm_kernel<Cfg, true>), grid, dim3(Cfg::NT), 0, stream, p);
-    else
-        hipLaunchKernelGGL((conv_igemm_kernel<Cfg, false>), grid, dim3(Cfg::NT), 0, stream, p);
+    const bool is3d = p.T > 1 || p.KT > 1 || p.pt > 0 || p.st > 1;
+    static const bool pipe = !(getenv("PET_HIP_PIPE") && atoi(getenv("PET_HIP_PIPE")) == 0);
+    if (pipe) {
+        if (is3d) {
+            if (veca)
+                hipLaunchKernelGGL((conv_pipe_kernel<Cfg, true, true>), grid, dim3(Cfg::NT), 0,
+                                   stream, p);
+            else
+                hipLaunchKernelGGL((conv_pipe_kernel<Cfg, false, true>), grid, dim3(Cfg::NT), 0,
+                                   stream, p);
+        } else {
+            if (veca)
+                hipLaunchKernelGGL((conv_pipe_kernel<Cfg, true, false>), grid, dim3(Cfg::NT), 0,
+                                   stream, p);
+            else
+                hipLaunchKernelGGL((conv_pipe_kernel<Cfg, false, false>), grid, dim3(Cfg::NT), 0,
+                                   stream, p);
+        }
+        return check_launch("conv_pipe_kernel");
+    }
+    if (is3d) {
+        if (veca)
+            hipLaunchKernelGGL((conv_igemm_kernel<Cfg, true, true>), grid, dim3(Cfg::NT), 0,
+                               stream, p);
+        else
+            hipLaunchKernelGGL((conv_igemm_kernel<Cfg, false, true>), grid, dim3(Cfg::NT), 0,
+                               stream, p);
+    } else {
+        if (veca)
+            hipLaunchKernelGGL((conv_igemm_kernel<Cfg, true, false>), grid, dim3(Cfg::NT), 0,
+                               stream, p);
+        else
+            hipLaunchKernelGGL((conv_igemm_kernel<Cfg, false, false>), grid, dim3(Cfg::NT), 0,
+                               stream, p);
+    }
     return check_launch("conv_igemm_kernel");
 }
 
@@ -502,8 +1110,19 @@ long long tiles_for(int m, int n, int bm, int bn, int batch) {
     return (long long)((m + bm - 1) / bm) * ((n + bn - 1) / bn) * batch;
 }
 
+// Tuning knob: PET_HIP_TILE=<0..3> forces a tile shape (read once).
+int forced_tile() {
+    static int v = [] {
+        const char *e = getenv("PET_HIP_TILE");
+        return e ? atoi(e) : -1;
+    }();
+    return v;
+}
+
 // 0: 128x128, 1: 64x128, 2: 64x64, 3: 32x64
 int pick_tile(int M, int N, int batch) {
+    if (forced_tile() >= 0)
+        return forced_tile();
     const long long want = 256; // one workgroup per CU at least
     if (M >= 128 && tiles_for(M, N, 128, 128, batch) >= 2 * want)
         return 0;
@@ -516,7 +1135,61 @@ int pick_tile(int M, int N, int batch) {
     return 3;
 }
 
+template <class Cfg, bool IS3D>
+int launch_plane_cfg(const ConvParams &p, hipStream_t stream) {
+    const size_t lds_bytes = 2 * (size_t)Cfg::STAGE * sizeof(float);
+    static int attr_status = [&] {
+        hipError_t e = hipFuncSetAttribute(
+            reinterpret_cast<const void *>(&conv_plane_kernel<Cfg, IS3D>),
+            hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
+        return e == hipSuccess ? 0 : 1;
+    }();
+    if (attr_status)
+        return -1; // caller falls back to the general kernel
+    dim3 grid((p.NPIX + Cfg::BN - 1) / Cfg::BN, (p.M + Cfg::BM - 1) / Cfg::BM, p.G);
+    hipLaunchKernelGGL((conv_plane_kernel<Cfg, IS3D>), grid, dim3(Cfg::NT), lds_bytes, stream, p);
+    return check_launch("conv_plane_kernel");
+}
+
+template <int RS, int CB>
+int launch_plane(const ConvParams &p, bool is3d, hipStream_t stream) {
+    using C64x128 = PlaneCfg<64, 128, 2, 2, RS, CB>;
+    using C64x64 = PlaneCfg<64, 64, 2, 2, RS, CB>;
+    const long long t128 = tiles_for(p.M, p.NPIX, 64, 128, p.G);
+    int tile = (p.M >= 64 && t128 >= 200) ? 0 : 1;
+    if (forced_tile() >= 0)
+        tile = forced_tile() & 1;
+    if (tile == 0)
+        return is3d ? launch_plane_cfg<C64x128, true>(p, stream)
+                    : launch_plane_cfg<C64x128, false>(p, stream);
+    return is3d ? launch_plane_cfg<C64x64, true>(p, stream)
+                : launch_plane_cfg<C64x64, false>(p, stream);
+}
+
+// Returns -1 when the plane kernel does not apply.
+int try_launch_plane(const ConvParams &p, hipStream_t stream) {
+    static const bool off = getenv("PET_HIP_PLANE") && atoi(getenv("PET_HIP_PLANE")) == 0;
+    if (off)
+        return -1;
+    const long long in_bytes = 4ll * p.N * p.C * p.T * p.H * p.W;
+    const long long w_bytes = 4ll * p.F * p.K;
+    if (in_bytes >= (1ll << 31) || w_bytes >= (1ll << 31))
+        return -1;
+    if (((uintptr_t)p.w & 15) != 0)
+        return -1;
+    const bool is3d = p.T > 1 || p.KT > 1 || p.pt > 0 || p.st > 1;
+    const int rs = p.R * p.S;
+    if (rs == 9 && p.cpg % 8 == 0)
+        return launch_plane<9, 8>(p, is3d, stream);
+    if (rs == 1 && p.cpg % 32 == 0)
+        return launch_plane<1, 32>(p, is3d, stream);
+    return -1;
+}
+
 int launch_conv(ConvParams &p, hipStream_t stream) {
+    int rc = try_launch_plane(p, stream);
+    if (rc >= 0)
+        return rc;
     bool veca = (p.K % 4 == 0) && (((uintptr_t)p.w & 15) == 0);
     switch (pick_tile(p.M, p.NPIX, p.G)) {
     case 0:
@@ -525,6 +1198,14 @@ int launch_conv(ConvParams &p, hipStream_t stream) {
         return launch_conv_cfg<Cfg64x128>(p, veca, stream);
     case 2:
         return launch_conv_cfg<Cfg64x64>(p, veca, stream);
+    case 4:
+        return launch_conv_cfg<Cfg64x64k32>(p, veca, stream);
+    case 5:
+        return launch_conv_cfg<Cfg64x64k64>(p, veca, stream);
+    case 6:
+        return launch_conv_cfg<Cfg64x128k32>(p, veca, stream);
+    case 7:
+        return launch_conv_cfg<Cfg128x128k32>(p, veca, stream);
     default:
         return launch_conv_cfg<Cfg32x64>(p, veca, stream);
     }
@@ -658,7 +1339,16 @@ int pet_hip_bmm_f32(int transA, int transB, int b, int m, int n, int k, const fl
         return set_error(PET_HIP_ERR_INVALID, "unknown activation %d", act);
     if ((long long)b * m * n == 0)
         return PET_HIP_OK;
-    if (!A || !B || !C)
+    if (!C)
+        return set_error(PET_HIP_ERR_INVALID, "null tensor pointer");
+    if (k == 0) {
+        // empty contraction: C = act(bias)
+        int rc = pet_hip_fill_f32(C, 0.f, (size_t)b * m * n, stream);
+        if (rc == PET_HIP_OK && (bias || act != PET_HIP_ACT_NONE))
+            rc = pet_hip_bias_act(C, bias, C, (size_t)b * m, (size_t)n, 1, act, stream);
+        return rc;
+    }
+    if (!A || !B)
         return set_error(PET_HIP_ERR_INVALID, "null tensor pointer");
     if ((long long)m * k >= (1ll << 31) || (long long)k * n >= (1ll << 31) ||
         (long long)m * n >= (1ll << 31) || b > 65535)
