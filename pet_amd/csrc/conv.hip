@@ -1,255 +1,20 @@
-// fp32 MFMA contractions for gfx950: implicit-GEMM convolution (2-D and 3-D,
-// strided / dilated / grouped, fused bias + activation) and batched matmul.
+// fp32 MFMA implicit-GEMM convolution for gfx950 (2-D and 3-D, strided, dilated,
+// grouped, fused bias + activation). M = output channels of a group, N = output
+// pixels (batch folded in), K = (channels per group) x (filter taps).
 //
-// One tiling serves both. A workgroup of NW waves owns a BM x BN tile of the
-// output (M = output channels or matmul rows, N = output pixels or matmul
-// columns) and walks K in steps of BK:
-//   global -> registers (tile kt+1)   overlapped with
-//   LDS -> v_mfma_f32_32x32x2_f32     (tile kt), then registers -> LDS.
-// LDS holds A as [m][k] (k contiguous, row stride BK+4 so that a lane's BK/2
-// k-values are two 128-bit reads) and B as [k][n] (n contiguous). Within a BK
-// block MFMA step j feeds lanes 0-31 with k = j and lanes 32-63 with
-// k = BK/2 + j, for both operands, so the products pair up correctly whatever
-// the order.
-#include "common.h"
-
-#include <algorithm>
-#include <cstdlib>
-#include <type_traits>
+// Two kernels:
+//  * conv_plane_kernel: the fast path for 3x3 / 1x1 (and 3x3x3, one kt slice per
+//    K step) filters; see the comment at the kernel.
+//  * conv_pipe_kernel: any filter shape, stride, dilation and channel count.
+// Both keep A (weights) in LDS as [m][k] and B (the im2col tile) as [k][n] and
+// feed v_mfma_f32_32x32x2_f32; within a K block MFMA step j gives lanes 0-31
+// k = j and lanes 32-63 k = BK/2 + j on both operands.
+#include "mfma_common.h"
 
 using namespace pet;
+using namespace pet::mfma;
 
 namespace {
-
-typedef float floatx16 __attribute__((ext_vector_type(16)));
-
-// Division by a run-time invariant, branch-free: q = (mulhi(n, mul) + (n & add)) >> shift.
-// For d == 1 the multiply contributes nothing and `add` passes n through.
-struct FastDiv {
-    unsigned d, mul, shift, add;
-};
-
-FastDiv make_fastdiv(unsigned d) {
-    FastDiv f;
-    f.d = d;
-    f.mul = 0;
-    f.shift = 0;
-    f.add = 0xFFFFFFFFu;
-    if (d <= 1)
-        return f;
-    f.add = 0;
-    unsigned l = 0;
-    while ((1ull << l) < d)
-        ++l;
-    unsigned p = 31 + l;
-    f.mul = (unsigned)(((1ull << p) + d - 1) / d);
-    f.shift = p - 32;
-    return f;
-}
-
-__device__ __forceinline__ unsigned fd_div(unsigned n, const FastDiv &f) {
-    return (__umulhi(n, f.mul) + (n & f.add)) >> f.shift;
-}
-
-template <int BM_, int BN_, int BK_, int WGM_, int WGN_>
-struct TileCfg {
-    static constexpr int BM = BM_, BN = BN_, BK = BK_;
-    static constexpr int WGM = WGM_, WGN = WGN_;
-    static constexpr int NW = WGM * WGN;
-    static constexpr int NT = NW * 64;
-    static constexpr int WM = BM / WGM, WN = BN / WGN;
-    static constexpr int TM = WM / 32, TN = WN / 32;
-    static constexpr int KH = BK / 2;
-    static constexpr int A_LD = BK + 4;
-    static constexpr int B_LD = BN + 4;
-    static constexpr int A_ELEMS = BM * A_LD;
-    static constexpr int B_ELEMS = BK * B_LD;
-    static constexpr int STAGE = A_ELEMS + B_ELEMS;
-    // loader shapes
-    static constexpr int A_VPT = BM * BK / 4 / NT; // float4 per thread, k-contiguous A
-    static constexpr int B_VPT = BK * BN / 4 / NT; // float4 per thread, n-contiguous B
-    static constexpr int RPW = BK / NW;            // gather rows per wave (conv)
-    static constexpr int PPL = BN / 64;            // gather pixels per lane (conv)
-    static_assert(WM % 32 == 0 && WN % 32 == 0, "wave tile must be a multiple of 32x32");
-    static_assert(BK % 8 == 0, "BK must be a multiple of 8");
-    static_assert(A_VPT >= 1 && B_VPT >= 1 && RPW >= 1 && PPL >= 1, "tile too small");
-    static_assert(BM * BK / 4 % NT == 0 && BK * BN / 4 % NT == 0 && BK % NW == 0 &&
-                      BN % 64 == 0,
-                  "loader shapes must divide evenly");
-};
-
-// ---- the MFMA inner product over one BK block ---------------------------------
-template <class Cfg>
-__device__ __forceinline__ void mma_block(const float *__restrict__ As,
-                                          const float *__restrict__ Bs,
-                                          floatx16 (&acc)[Cfg::TM][Cfg::TN], int wm0, int wn0,
-                                          int lane) {
-    const int l32 = lane & 31, hk = lane >> 5;
-    float a[Cfg::TM][Cfg::KH];
-#pragma unroll
-    for (int tm = 0; tm < Cfg::TM; ++tm) {
-        const float *ap = As + (wm0 + tm * 32 + l32) * Cfg::A_LD + hk * Cfg::KH;
-#pragma unroll
-        for (int j = 0; j < Cfg::KH; j += 4) {
-            float4 v = *reinterpret_cast<const float4 *>(ap + j);
-            a[tm][j] = v.x;
-            a[tm][j + 1] = v.y;
-            a[tm][j + 2] = v.z;
-            a[tm][j + 3] = v.w;
-        }
-    }
-#pragma unroll
-    for (int j = 0; j < Cfg::KH; ++j) {
-        float b[Cfg::TN];
-        const float *bp = Bs + (hk * Cfg::KH + j) * Cfg::B_LD + wn0 + l32;
-#pragma unroll
-        for (int tn = 0; tn < Cfg::TN; ++tn)
-            b[tn] = bp[tn * 32];
-#pragma unroll
-        for (int tm = 0; tm < Cfg::TM; ++tm)
-#pragma unroll
-            for (int tn = 0; tn < Cfg::TN; ++tn)
-                acc[tm][tn] =
-                    __builtin_amdgcn_mfma_f32_32x32x2f32(a[tm][j], b[tn], acc[tm][tn], 0, 0, 0);
-    }
-}
-
-// Sixteen bytes of zeros: a load that must yield 0 (a padding tap, the K tail)
-// is pointed here instead of being masked after the fact, so that no
-// instruction depends on the loaded value until it is written to LDS.
-__device__ __attribute__((aligned(16))) const float g_zero16[4] = {0.f, 0.f, 0.f, 0.f};
-
-// Zeroes v when keep is false without giving the compiler a branch to make.
-__device__ __forceinline__ float keep_if(float v, bool keep) {
-    return __int_as_float(__float_as_int(v) & (keep ? -1 : 0));
-}
-
-__device__ __forceinline__ float4 keep_if(float4 v, bool keep) {
-    const int m = keep ? -1 : 0;
-    return make_float4(__int_as_float(__float_as_int(v.x) & m), __int_as_float(__float_as_int(v.y) & m),
-                       __int_as_float(__float_as_int(v.z) & m), __int_as_float(__float_as_int(v.w) & m));
-}
-
-// ---- operand loaders -----------------------------------------------------------
-// "KC": the operand is stored with K contiguous (weights [f][k], A [m][k],
-// B^T [n][k]); "XC": the non-K index is contiguous (A^T [k][m], B [k][n]).
-// rows = extent of the non-K index, ld = source row stride.
-
-// K-contiguous source -> registers, branch-free: rows past the end re-read the
-// last row (those accumulator rows are never stored), the K tail is zeroed by a
-// select. VEC: ld % 4 == 0, K % 4 == 0 and a 16-byte aligned base.
-template <int ROWS, int BK, int NT, bool VEC>
-__device__ __forceinline__ void load_kc(const float *__restrict__ src, unsigned ld, int row0,
-                                        int rows, int k0, int K, int tid,
-                                        float4 (&regs)[ROWS * BK / 4 / NT]) {
-    constexpr int VPT = ROWS * BK / 4 / NT;
-#pragma unroll
-    for (int i = 0; i < VPT; ++i) {
-        int v = tid + i * NT;
-        int row = v / (BK / 4), kq = (v % (BK / 4)) * 4;
-        int gr = min(row0 + row, rows - 1), gk = k0 + kq;
-        const unsigned rbase = (unsigned)gr * ld;
-        float4 val;
-        const float *pz = g_zero16;
-        if (VEC) {
-            const float *q = gk < K ? src + (rbase + (unsigned)gk) : pz;
-            val = *reinterpret_cast<const float4 *>(q);
-        } else {
-            val.x = *(gk < K ? src + (rbase + (unsigned)gk) : pz);
-            val.y = *(gk + 1 < K ? src + (rbase + (unsigned)gk + 1u) : pz);
-            val.z = *(gk + 2 < K ? src + (rbase + (unsigned)gk + 2u) : pz);
-            val.w = *(gk + 3 < K ? src + (rbase + (unsigned)gk + 3u) : pz);
-        }
-        regs[i] = val;
-    }
-}
-
-// registers (from load_kc) -> LDS laid out [row][k] with stride LD (used for A)
-template <int ROWS, int BK, int NT, int LD>
-__device__ __forceinline__ void store_kc_rowmajor(float *__restrict__ dst, int tid,
-                                                  const float4 (&regs)[ROWS * BK / 4 / NT]) {
-    constexpr int VPT = ROWS * BK / 4 / NT;
-#pragma unroll
-    for (int i = 0; i < VPT; ++i) {
-        int v = tid + i * NT;
-        int row = v / (BK / 4), kq = (v % (BK / 4)) * 4;
-        *reinterpret_cast<float4 *>(dst + row * LD + kq) = regs[i];
-    }
-}
-
-// registers (from load_kc) -> LDS laid out [k][row] with stride LD (used for B^T)
-template <int ROWS, int BK, int NT, int LD>
-__device__ __forceinline__ void store_kc_transposed(float *__restrict__ dst, int tid,
-                                                    const float4 (&regs)[ROWS * BK / 4 / NT]) {
-    constexpr int VPT = ROWS * BK / 4 / NT;
-#pragma unroll
-    for (int i = 0; i < VPT; ++i) {
-        int v = tid + i * NT;
-        int row = v / (BK / 4), kq = (v % (BK / 4)) * 4;
-        dst[(kq + 0) * LD + row] = regs[i].x;
-        dst[(kq + 1) * LD + row] = regs[i].y;
-        dst[(kq + 2) * LD + row] = regs[i].z;
-        dst[(kq + 3) * LD + row] = regs[i].w;
-    }
-}
-
-// X-contiguous source (element (x, k) at src[k * ld + x]) -> registers,
-// branch-free in the same way (columns past the end are never stored).
-template <int COLS, int BK, int NT, bool VEC>
-__device__ __forceinline__ void load_xc(const float *__restrict__ src, unsigned ld, int col0,
-                                        int cols, int k0, int K, int tid,
-                                        float4 (&regs)[COLS * BK / 4 / NT]) {
-    constexpr int VPT = COLS * BK / 4 / NT;
-#pragma unroll
-    for (int i = 0; i < VPT; ++i) {
-        int v = tid + i * NT;
-        int k = v / (COLS / 4), cq = (v % (COLS / 4)) * 4;
-        int gk = k0 + k, gc = col0 + cq;
-        const unsigned kbase = (unsigned)min(gk, K - 1) * ld;
-        const float *pz = g_zero16;
-        const bool kok = gk < K;
-        float4 val;
-        if (VEC) {
-            const float *q = kok ? src + (kbase + (unsigned)min(gc, cols - 4)) : pz;
-            val = *reinterpret_cast<const float4 *>(q);
-        } else {
-            val.x = *(kok ? src + (kbase + (unsigned)min(gc, cols - 1)) : pz);
-            val.y = *(kok ? src + (kbase + (unsigned)min(gc + 1, cols - 1)) : pz);
-            val.z = *(kok ? src + (kbase + (unsigned)min(gc + 2, cols - 1)) : pz);
-            val.w = *(kok ? src + (kbase + (unsigned)min(gc + 3, cols - 1)) : pz);
-        }
-        regs[i] = val;
-    }
-}
-
-// registers (from load_xc) -> LDS [k][col] with stride LD (used for B)
-template <int COLS, int BK, int NT, int LD>
-__device__ __forceinline__ void store_xc_rowmajor(float *__restrict__ dst, int tid,
-                                                  const float4 (&regs)[COLS * BK / 4 / NT]) {
-    constexpr int VPT = COLS * BK / 4 / NT;
-#pragma unroll
-    for (int i = 0; i < VPT; ++i) {
-        int v = tid + i * NT;
-        int k = v / (COLS / 4), cq = (v % (COLS / 4)) * 4;
-        *reinterpret_cast<float4 *>(dst + k * LD + cq) = regs[i];
-    }
-}
-
-// registers (from load_xc) -> LDS [col][k] with stride LD (used for A^T)
-template <int COLS, int BK, int NT, int LD>
-__device__ __forceinline__ void store_xc_transposed(float *__restrict__ dst, int tid,
-                                                    const float4 (&regs)[COLS * BK / 4 / NT]) {
-    constexpr int VPT = COLS * BK / 4 / NT;
-#pragma unroll
-    for (int i = 0; i < VPT; ++i) {
-        int v = tid + i * NT;
-        int k = v / (COLS / 4), cq = (v % (COLS / 4)) * 4;
-        dst[(cq + 0) * LD + k] = regs[i].x;
-        dst[(cq + 1) * LD + k] = regs[i].y;
-        dst[(cq + 2) * LD + k] = regs[i].z;
-        dst[(cq + 3) * LD + k] = regs[i].w;
-    }
-}
 
 // ---- convolution -----------------------------------------------------------------
 
@@ -271,158 +36,7 @@ struct ConvParams {
     int tiles_n;                     // pixel tiles (for the workgroup swizzle)
 };
 
-template <class Cfg, bool VECA, bool IS3D>
-__global__ __launch_bounds__(Cfg::NT) void conv_igemm_kernel(ConvParams p) {
-    __shared__ __attribute__((aligned(16))) float lds[2 * Cfg::STAGE];
-    const int tid = threadIdx.x;
-    const int lane = tid & 63;
-    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int wm0 = (wave / Cfg::WGN) * Cfg::WM;
-    const int wn0 = (wave % Cfg::WGN) * Cfg::WN;
-    const int g = blockIdx.z;
-    const int m0 = blockIdx.y * Cfg::BM;
-    const int n0 = blockIdx.x * Cfg::BN;
 
-    const int THW = p.T * p.H * p.W, HW = p.H * p.W;
-    const float *__restrict__ wg_w = p.w + (long long)g * p.M * p.K;
-    const float *__restrict__ wg_x = p.x + (long long)g * p.cpg * THW;
-
-    // per-lane pixel state: PPL pixels, fixed for the whole kernel. Pixels past
-    // the end alias the last pixel; their accumulator columns are never stored.
-    int pbase[Cfg::PPL], it0[Cfg::PPL], ih0[Cfg::PPL], iw0[Cfg::PPL];
-#pragma unroll
-    for (int pp = 0; pp < Cfg::PPL; ++pp) {
-        int pix = min(n0 + lane + pp * 64, p.NPIX - 1);
-        unsigned n = fd_div(pix, p.fd_opix);
-        unsigned rem = pix - n * p.OPIX;
-        unsigned ot = 0;
-        if (IS3D) {
-            ot = fd_div(rem, p.fd_ohw);
-            rem -= ot * (p.OH * p.OW);
-        }
-        unsigned oh = fd_div(rem, p.fd_ow);
-        unsigned ow = rem - oh * p.OW;
-        it0[pp] = IS3D ? (int)ot * p.st - p.pt : 0;
-        ih0[pp] = (int)oh * p.sh - p.ph;
-        iw0[pp] = (int)ow * p.sw - p.pw;
-        pbase[pp] = (int)n * p.C * THW + it0[pp] * HW + ih0[pp] * p.W + iw0[pp];
-    }
-
-    float4 areg[Cfg::A_VPT];
-    float breg[Cfg::RPW][Cfg::PPL];
-
-    // Branch-free im2col gather: the k index of a row is wave-uniform, so its
-    // (c, kt, r, s) split runs on the scalar unit; a tap outside the image (or
-    // past K) reads offset 0 and is replaced by 0 with a select.
-    auto gather_b = [&](int k0) {
-#pragma unroll
-        for (int i = 0; i < Cfg::RPW; ++i) {
-            const int k = k0 + wave + Cfg::NW * i;
-            const unsigned c = fd_div(k, p.fd_krs);
-            unsigned rem = k - c * p.fd_krs.d;
-            unsigned q = 0;
-            if (IS3D) {
-                q = fd_div(rem, p.fd_rs);
-                rem -= q * p.fd_rs.d;
-            }
-            const unsigned r = fd_div(rem, p.fd_s);
-            const unsigned s = rem - r * p.fd_s.d;
-            const int qt = (int)q * p.dt, rh = (int)r * p.dh, sw_ = (int)s * p.dw;
-            const int koff = (int)c * THW + qt * HW + rh * p.W + sw_;
-            const bool kok = k < p.K;
-#pragma unroll
-            for (int pp = 0; pp < Cfg::PPL; ++pp) {
-                bool ok = kok & ((unsigned)(ih0[pp] + rh) < (unsigned)p.H) &
-                          ((unsigned)(iw0[pp] + sw_) < (unsigned)p.W);
-                if (IS3D)
-                    ok = ok & ((unsigned)(it0[pp] + qt) < (unsigned)p.T);
-                const float *q = ok ? wg_x + (unsigned)(pbase[pp] + koff) : g_zero16;
-                breg[i][pp] = *q;
-            }
-        }
-    };
-    auto store_b = [&](float *Bs) {
-#pragma unroll
-        for (int i = 0; i < Cfg::RPW; ++i)
-#pragma unroll
-            for (int pp = 0; pp < Cfg::PPL; ++pp)
-                Bs[(wave + Cfg::NW * i) * Cfg::B_LD + lane + pp * 64] = breg[i][pp];
-    };
-
-    floatx16 acc[Cfg::TM][Cfg::TN];
-#pragma unroll
-    for (int tm = 0; tm < Cfg::TM; ++tm)
-#pragma unroll
-        for (int tn = 0; tn < Cfg::TN; ++tn)
-#pragma unroll
-            for (int r = 0; r < 16; ++r)
-                acc[tm][tn][r] = 0.f;
-
-    const int nk = (p.K + Cfg::BK - 1) / Cfg::BK;
-    load_kc<Cfg::BM, Cfg::BK, Cfg::NT, VECA>(wg_w, p.K, m0, p.M, 0, p.K, tid, areg);
-    gather_b(0);
-    store_kc_rowmajor<Cfg::BM, Cfg::BK, Cfg::NT, Cfg::A_LD>(lds, tid, areg);
-    store_b(lds + Cfg::A_ELEMS);
-    __syncthreads();
-
-    // main loop (all but the last K block): prefetch kt+1 while computing kt
-    for (int kt = 0; kt < nk - 1; ++kt) {
-        float *cur = lds + (kt & 1) * Cfg::STAGE;
-        float *nxt = lds + ((kt + 1) & 1) * Cfg::STAGE;
-        load_kc<Cfg::BM, Cfg::BK, Cfg::NT, VECA>(wg_w, p.K, m0, p.M, (kt + 1) * Cfg::BK, p.K, tid,
-                                                 areg);
-        gather_b((kt + 1) * Cfg::BK);
-        __builtin_amdgcn_sched_barrier(0); // keep the prefetch ahead of the MFMA block
-        mma_block<Cfg>(cur, cur + Cfg::A_ELEMS, acc, wm0, wn0, lane);
-        __builtin_amdgcn_sched_barrier(0);
-        store_kc_rowmajor<Cfg::BM, Cfg::BK, Cfg::NT, Cfg::A_LD>(nxt, tid, areg);
-        store_b(nxt + Cfg::A_ELEMS);
-        __syncthreads();
-    }
-    {
-        float *cur = lds + ((nk - 1) & 1) * Cfg::STAGE;
-        mma_block<Cfg>(cur, cur + Cfg::A_ELEMS, acc, wm0, wn0, lane);
-    }
-
-    // epilogue: bias + activation, NC(T)HW store. Lane holds column l%32 and
-    // rows (r/4)*8 + (l/32)*4 + r%4 of each 32x32 block.
-    const int l32 = lane & 31, hk = lane >> 5;
-#pragma unroll
-    for (int tn = 0; tn < Cfg::TN; ++tn) {
-        int pix = n0 + wn0 + tn * 32 + l32;
-        if (pix >= p.NPIX)
-            continue;
-        unsigned n = fd_div(pix, p.fd_opix);
-        unsigned rem = pix - n * p.OPIX;
-        float *__restrict__ yb = p.y + (((long long)n * p.F + (long long)g * p.M) * p.OPIX + rem);
-        const float *__restrict__ bias = p.bias ? p.bias + g * p.M : nullptr;
-#pragma unroll
-        for (int tm = 0; tm < Cfg::TM; ++tm) {
-#pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                int f = m0 + wm0 + tm * 32 + (r / 4) * 8 + hk * 4 + (r % 4);
-                if (f < p.M) {
-                    float v = acc[tm][tn][r];
-                    if (bias)
-                        v += bias[f];
-                    yb[(unsigned)f * (unsigned)p.OPIX] = apply_act(v, p.act);
-                }
-            }
-        }
-    }
-}
-
-// Software-pipelined variant of the convolution kernel. With one or two waves
-// per SIMD nothing but the wave's own instruction stream can hide latency, so
-// the K loop is written as NM "slots", one MFMA each, and the other work of the
-// iteration is dealt out between them in a fixed order:
-//   G(kt+2): global -> prefetch registers   (two register sets, so a load has
-//                                            more than a full iteration to land)
-//   W(kt+1): prefetch registers -> LDS
-//   barrier
-//   R(kt+1): LDS -> fragment registers      (two sets: MFMAs of tile kt read
-//                                            one while the other is filled)
-// The MFMAs of tile kt therefore straddle the barrier and never wait on LDS.
 template <class Cfg, bool VECA, bool IS3D>
 __global__ __launch_bounds__(Cfg::NT) void conv_pipe_kernel(ConvParams p) {
     __shared__ __attribute__((aligned(16))) float lds[2 * Cfg::STAGE];
@@ -910,14 +524,17 @@ __global__ __launch_bounds__(Cfg::NT) void conv_plane_kernel(ConvParams p) {
                 const int pb_ = (h * NPOST + HN - 1) / HN, pe_ = ((h + 1) * NPOST + HN - 1) / HN;
 #pragma unroll
                 for (int q = pb_; q < pe_; ++q) {
-                    // fragment reads first in each pair, prefetches after
-                    if (q < 2 * NG) {
+                    // fragment reads and prefetches alternate, the longer list runs on
+                    constexpr int NMIN = NR < NG ? NR : NG;
+                    if (q < 2 * NMIN) {
                         if (q & 1)
                             g_piece(q >> 1);
                         else
                             r_piece(PAR ^ 1, q >> 1, nxt);
+                    } else if (NR > NG) {
+                        r_piece(PAR ^ 1, q - NMIN, nxt);
                     } else {
-                        r_piece(PAR ^ 1, q - NG, nxt);
+                        g_piece(q - NMIN);
                     }
                 }
             }
@@ -959,177 +576,43 @@ __global__ __launch_bounds__(Cfg::NT) void conv_plane_kernel(ConvParams p) {
     }
 }
 
-// ---- batched matmul ----------------------------------------------------------------
-
-struct GemmParams {
-    const float *A, *B, *bias;
-    float *C;
-    int M, N, K;
-    long long sA, sB, sC; // batch strides
-    int act;
-};
-
-template <class Cfg, bool TA, bool TB, bool VEC>
-__global__ __launch_bounds__(Cfg::NT) void bmm_kernel(GemmParams p) {
-    __shared__ __attribute__((aligned(16))) float lds[2 * Cfg::STAGE];
-    const int tid = threadIdx.x;
-    const int lane = tid & 63;
-    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const int wm0 = (wave / Cfg::WGN) * Cfg::WM;
-    const int wn0 = (wave % Cfg::WGN) * Cfg::WN;
-    const int b = blockIdx.z;
-    const int m0 = blockIdx.y * Cfg::BM;
-    const int n0 = blockIdx.x * Cfg::BN;
-    const float *__restrict__ A = p.A + (long long)b * p.sA;
-    const float *__restrict__ B = p.B + (long long)b * p.sB;
-    float *__restrict__ C = p.C + (long long)b * p.sC;
-
-    float4 areg[Cfg::A_VPT];
-    float4 breg[Cfg::B_VPT];
-
-    auto load_tiles = [&](int k0) {
-        if (TA)
-            load_xc<Cfg::BM, Cfg::BK, Cfg::NT, VEC>(A, p.M, m0, p.M, k0, p.K, tid, areg);
-        else
-            load_kc<Cfg::BM, Cfg::BK, Cfg::NT, VEC>(A, p.K, m0, p.M, k0, p.K, tid, areg);
-        if (TB)
-            load_kc<Cfg::BN, Cfg::BK, Cfg::NT, VEC>(B, p.K, n0, p.N, k0, p.K, tid, breg);
-        else
-            load_xc<Cfg::BN, Cfg::BK, Cfg::NT, VEC>(B, p.N, n0, p.N, k0, p.K, tid, breg);
-    };
-    auto store_tiles = [&](float *st) {
-        if (TA)
-            store_xc_transposed<Cfg::BM, Cfg::BK, Cfg::NT, Cfg::A_LD>(st, tid, areg);
-        else
-            store_kc_rowmajor<Cfg::BM, Cfg::BK, Cfg::NT, Cfg::A_LD>(st, tid, areg);
-        if (TB)
-            store_kc_transposed<Cfg::BN, Cfg::BK, Cfg::NT, Cfg::B_LD>(st + Cfg::A_ELEMS, tid, breg);
-        else
-            store_xc_rowmajor<Cfg::BN, Cfg::BK, Cfg::NT, Cfg::B_LD>(st + Cfg::A_ELEMS, tid, breg);
-    };
-
-    floatx16 acc[Cfg::TM][Cfg::TN];
-#pragma unroll
-    for (int tm = 0; tm < Cfg::TM; ++tm)
-#pragma unroll
-        for (int tn = 0; tn < Cfg::TN; ++tn)
-#pragma unroll
-            for (int r = 0; r < 16; ++r)
-                acc[tm][tn][r] = 0.f;
-
-    const int nk = (p.K + Cfg::BK - 1) / Cfg::BK;
-    load_tiles(0);
-    store_tiles(lds);
-    __syncthreads();
-    for (int kt = 0; kt < nk - 1; ++kt) {
-        float *cur = lds + (kt & 1) * Cfg::STAGE;
-        float *nxt = lds + ((kt + 1) & 1) * Cfg::STAGE;
-        load_tiles((kt + 1) * Cfg::BK);
-        __builtin_amdgcn_sched_barrier(0); // keep the prefetch ahead of the MFMA block
-        mma_block<Cfg>(cur, cur + Cfg::A_ELEMS, acc, wm0, wn0, lane);
-        __builtin_amdgcn_sched_barrier(0);
-        store_tiles(nxt);
-        __syncthreads();
-    }
-    {
-        float *cur = lds + ((nk - 1) & 1) * Cfg::STAGE;
-        mma_block<Cfg>(cur, cur + Cfg::A_ELEMS, acc, wm0, wn0, lane);
-    }
-
-    const int l32 = lane & 31, hk = lane >> 5;
-#pragma unroll
-    for (int tn = 0; tn < Cfg::TN; ++tn) {
-        int col = n0 + wn0 + tn * 32 + l32;
-        if (col >= p.N)
-            continue;
-        float bv = p.bias ? p.bias[col] : 0.f;
-#pragma unroll
-        for (int tm = 0; tm < Cfg::TM; ++tm) {
-#pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                int row = m0 + wm0 + tm * 32 + (r / 4) * 8 + hk * 4 + (r % 4);
-                if (row < p.M)
-                    C[(long long)row * p.N + col] = apply_act(acc[tm][tn][r] + bv, p.act);
-            }
-        }
-    }
-}
-
-// Tile menu. Picked per problem so that the grid fills the 256 CUs.
 using Cfg128x128 = TileCfg<128, 128, 16, 2, 2>;
-using Cfg64x128 = TileCfg<64, 128, 16, 2, 2>;
-using Cfg64x64 = TileCfg<64, 64, 16, 2, 2>;
+using Cfg64x128 = TileCfg<64, 128, 32, 2, 2>;
+using Cfg64x64 = TileCfg<64, 64, 32, 2, 2>;
 using Cfg32x64 = TileCfg<32, 64, 16, 1, 2>;
-using Cfg64x64k32 = TileCfg<64, 64, 32, 2, 2>;
-using Cfg64x64k64 = TileCfg<64, 64, 64, 2, 2>;
-using Cfg64x128k32 = TileCfg<64, 128, 32, 2, 2>;
-using Cfg128x128k32 = TileCfg<128, 128, 32, 2, 2>;
 
 template <class Cfg>
-int launch_conv_cfg(const ConvParams &p, bool veca, hipStream_t stream) {
+int launch_pipe_cfg(const ConvParams &p, bool veca, hipStream_t stream) {
     dim3 grid((p.NPIX + Cfg::BN - 1) / Cfg::BN, (p.M + Cfg::BM - 1) / Cfg::BM, p.G);
     const bool is3d = p.T > 1 || p.KT > 1 || p.pt > 0 || p.st > 1;
-    static const bool pipe = !(getenv("PET_HIP_PIPE") && atoi(getenv("PET_HIP_PIPE")) == 0);
-    if (pipe) {
-        if (is3d) {
-            if (veca)
-                hipLaunchKernelGGL((conv_pipe_kernel<Cfg, true, true>), grid, dim3(Cfg::NT), 0,
-                                   stream, p);
-            else
-                hipLaunchKernelGGL((conv_pipe_kernel<Cfg, false, true>), grid, dim3(Cfg::NT), 0,
-                                   stream, p);
-        } else {
-            if (veca)
-                hipLaunchKernelGGL((conv_pipe_kernel<Cfg, true, false>), grid, dim3(Cfg::NT), 0,
-                                   stream, p);
-            else
-                hipLaunchKernelGGL((conv_pipe_kernel<Cfg, false, false>), grid, dim3(Cfg::NT), 0,
-                                   stream, p);
-        }
-        return check_launch("conv_pipe_kernel");
-    }
     if (is3d) {
         if (veca)
-            hipLaunchKernelGGL((conv_igemm_kernel<Cfg, true, true>), grid, dim3(Cfg::NT), 0,
-                               stream, p);
+            hipLaunchKernelGGL((conv_pipe_kernel<Cfg, true, true>), grid, dim3(Cfg::NT), 0, stream,
+                               p);
         else
-            hipLaunchKernelGGL((conv_igemm_kernel<Cfg, false, true>), grid, dim3(Cfg::NT), 0,
+            hipLaunchKernelGGL((conv_pipe_kernel<Cfg, false, true>), grid, dim3(Cfg::NT), 0,
                                stream, p);
     } else {
         if (veca)
-            hipLaunchKernelGGL((conv_igemm_kernel<Cfg, true, false>), grid, dim3(Cfg::NT), 0,
+            hipLaunchKernelGGL((conv_pipe_kernel<Cfg, true, false>), grid, dim3(Cfg::NT), 0,
                                stream, p);
         else
-            hipLaunchKernelGGL((conv_igemm_kernel<Cfg, false, false>), grid, dim3(Cfg::NT), 0,
+            hipLaunchKernelGGL((conv_pipe_kernel<Cfg, false, false>), grid, dim3(Cfg::NT), 0,
                                stream, p);
     }
-    return check_launch("conv_igemm_kernel");
+    return check_launch("conv_pipe_kernel");
 }
 
-long long tiles_for(int m, int n, int bm, int bn, int batch) {
-    return (long long)((m + bm - 1) / bm) * ((n + bn - 1) / bn) * batch;
-}
-
-// Tuning knob: PET_HIP_TILE=<0..3> forces a tile shape (read once).
-int forced_tile() {
-    static int v = [] {
-        const char *e = getenv("PET_HIP_TILE");
-        return e ? atoi(e) : -1;
-    }();
-    return v;
-}
-
-// 0: 128x128, 1: 64x128, 2: 64x64, 3: 32x64
+// Tile choice of the general kernel: the largest tile that still gives every
+// CU a workgroup. 0: 128x128, 1: 64x128, 2: 64x64, 3: 32x64.
 int pick_tile(int M, int N, int batch) {
     if (forced_tile() >= 0)
-        return forced_tile();
-    const long long want = 256; // one workgroup per CU at least
+        return forced_tile() & 3;
+    const long long want = 256;
     if (M >= 128 && tiles_for(M, N, 128, 128, batch) >= 2 * want)
         return 0;
     if (M >= 64 && tiles_for(M, N, 64, 128, batch) >= want)
         return 1;
-    if (M >= 64 && tiles_for(M, N, 64, 64, batch) >= want / 2)
-        return 2;
     if (M > 32)
         return 2;
     return 3;
@@ -1155,15 +638,23 @@ template <int RS, int CB>
 int launch_plane(const ConvParams &p, bool is3d, hipStream_t stream) {
     using C64x128 = PlaneCfg<64, 128, 2, 2, RS, CB>;
     using C64x64 = PlaneCfg<64, 64, 2, 2, RS, CB>;
-    const long long t128 = tiles_for(p.M, p.NPIX, 64, 128, p.G);
-    int tile = (p.M >= 64 && t128 >= 200) ? 0 : 1;
+    using C32x64 = PlaneCfg<32, 64, 1, 2, RS, CB>;
+    // the largest tile that still hands (nearly) every CU a workgroup
+    int tile = 2;
+    if (p.M > 32 && tiles_for(p.M, p.NPIX, 64, 64, p.G) >= 200)
+        tile = 1;
+    if (p.M > 32 && tiles_for(p.M, p.NPIX, 64, 128, p.G) >= 200)
+        tile = 0;
     if (forced_tile() >= 0)
-        tile = forced_tile() & 1;
+        tile = forced_tile() % 3;
     if (tile == 0)
         return is3d ? launch_plane_cfg<C64x128, true>(p, stream)
                     : launch_plane_cfg<C64x128, false>(p, stream);
-    return is3d ? launch_plane_cfg<C64x64, true>(p, stream)
-                : launch_plane_cfg<C64x64, false>(p, stream);
+    if (tile == 1)
+        return is3d ? launch_plane_cfg<C64x64, true>(p, stream)
+                    : launch_plane_cfg<C64x64, false>(p, stream);
+    return is3d ? launch_plane_cfg<C32x64, true>(p, stream)
+                : launch_plane_cfg<C32x64, false>(p, stream);
 }
 
 // Returns -1 when the plane kernel does not apply.
@@ -1190,48 +681,16 @@ int launch_conv(ConvParams &p, hipStream_t stream) {
     int rc = try_launch_plane(p, stream);
     if (rc >= 0)
         return rc;
-    bool veca = (p.K % 4 == 0) && (((uintptr_t)p.w & 15) == 0);
+    const bool veca = (p.K % 4 == 0) && (((uintptr_t)p.w & 15) == 0);
     switch (pick_tile(p.M, p.NPIX, p.G)) {
     case 0:
-        return launch_conv_cfg<Cfg128x128>(p, veca, stream);
+        return launch_pipe_cfg<Cfg128x128>(p, veca, stream);
     case 1:
-        return launch_conv_cfg<Cfg64x128>(p, veca, stream);
+        return launch_pipe_cfg<Cfg64x128>(p, veca, stream);
     case 2:
-        return launch_conv_cfg<Cfg64x64>(p, veca, stream);
-    case 4:
-        return launch_conv_cfg<Cfg64x64k32>(p, veca, stream);
-    case 5:
-        return launch_conv_cfg<Cfg64x64k64>(p, veca, stream);
-    case 6:
-        return launch_conv_cfg<Cfg64x128k32>(p, veca, stream);
-    case 7:
-        return launch_conv_cfg<Cfg128x128k32>(p, veca, stream);
+        return launch_pipe_cfg<Cfg64x64>(p, veca, stream);
     default:
-        return launch_conv_cfg<Cfg32x64>(p, veca, stream);
-    }
-}
-
-template <class Cfg, bool TA, bool TB>
-int launch_bmm_cfg(const GemmParams &p, int batch, bool vec, hipStream_t stream) {
-    dim3 grid((p.N + Cfg::BN - 1) / Cfg::BN, (p.M + Cfg::BM - 1) / Cfg::BM, batch);
-    if (vec)
-        hipLaunchKernelGGL((bmm_kernel<Cfg, TA, TB, true>), grid, dim3(Cfg::NT), 0, stream, p);
-    else
-        hipLaunchKernelGGL((bmm_kernel<Cfg, TA, TB, false>), grid, dim3(Cfg::NT), 0, stream, p);
-    return check_launch("bmm_kernel");
-}
-
-template <bool TA, bool TB>
-int launch_bmm_t(const GemmParams &p, int batch, bool vec, hipStream_t stream) {
-    switch (pick_tile(p.M, p.N, batch)) {
-    case 0:
-        return launch_bmm_cfg<Cfg128x128, TA, TB>(p, batch, vec, stream);
-    case 1:
-        return launch_bmm_cfg<Cfg64x128, TA, TB>(p, batch, vec, stream);
-    case 2:
-        return launch_bmm_cfg<Cfg64x64, TA, TB>(p, batch, vec, stream);
-    default:
-        return launch_bmm_cfg<Cfg32x64, TA, TB>(p, batch, vec, stream);
+        return launch_pipe_cfg<Cfg32x64>(p, veca, stream);
     }
 }
 
@@ -1327,55 +786,6 @@ int pet_hip_conv3d_f32(const float *x, const float *w, const float *bias, float 
     PET_REQUIRE_INIT();
     return conv_common(x, w, bias, y, n, c, t, h, wd, f, kt, r, s, pt, ph, pw, st, sh, sw, dt, dh,
                        dw, groups, act, as_stream(stream));
-}
-
-int pet_hip_bmm_f32(int transA, int transB, int b, int m, int n, int k, const float *A,
-                    const float *B, float *C, const float *bias, int act,
-                    pet_hip_stream_t stream) {
-    PET_REQUIRE_INIT();
-    if (b < 0 || m < 0 || n < 0 || k < 0)
-        return set_error(PET_HIP_ERR_INVALID, "negative matmul dims");
-    if (act < PET_HIP_ACT_NONE || act > PET_HIP_ACT_GELU)
-        return set_error(PET_HIP_ERR_INVALID, "unknown activation %d", act);
-    if ((long long)b * m * n == 0)
-        return PET_HIP_OK;
-    if (!C)
-        return set_error(PET_HIP_ERR_INVALID, "null tensor pointer");
-    if (k == 0) {
-        // empty contraction: C = act(bias)
-        int rc = pet_hip_fill_f32(C, 0.f, (size_t)b * m * n, stream);
-        if (rc == PET_HIP_OK && (bias || act != PET_HIP_ACT_NONE))
-            rc = pet_hip_bias_act(C, bias, C, (size_t)b * m, (size_t)n, 1, act, stream);
-        return rc;
-    }
-    if (!A || !B)
-        return set_error(PET_HIP_ERR_INVALID, "null tensor pointer");
-    if ((long long)m * k >= (1ll << 31) || (long long)k * n >= (1ll << 31) ||
-        (long long)m * n >= (1ll << 31) || b > 65535)
-        return set_error(PET_HIP_ERR_UNSUPPORTED, "matmul operand too large");
-    GemmParams p;
-    p.A = A;
-    p.B = B;
-    p.C = C;
-    p.bias = bias;
-    p.M = m;
-    p.N = n;
-    p.K = k;
-    p.sA = (long long)m * k;
-    p.sB = (long long)k * n;
-    p.sC = (long long)m * n;
-    p.act = act;
-    // float4 loads need every row start 16-byte aligned on both operands
-    long long lda = transA ? m : k, ldb = transB ? k : n;
-    bool vec = lda % 4 == 0 && ldb % 4 == 0 && p.sA % 4 == 0 && p.sB % 4 == 0 &&
-               (((uintptr_t)A | (uintptr_t)B) & 15) == 0 &&
-               (transA ? m % 4 == 0 : k % 4 == 0) && (transB ? k % 4 == 0 : n % 4 == 0);
-    hipStream_t s = as_stream(stream);
-    if (transA)
-        return transB ? launch_bmm_t<true, true>(p, b, vec, s)
-                      : launch_bmm_t<true, false>(p, b, vec, s);
-    return transB ? launch_bmm_t<false, true>(p, b, vec, s)
-                  : launch_bmm_t<false, false>(p, b, vec, s);
 }
 
 } // extern "C"
