@@ -1,0 +1,130 @@
+// Graph containers (role of the reference's include/graph.h): the builder API
+// the ONNX importer and the mutators call, connection inference, topological
+// execution on the device and the original-vs-mutant check.
+#pragma once
+#include "common.h"
+#include "operator.h"
+#include "tensor.h"
+#include <memory>
+
+namespace tpm {
+
+class GraphBase {
+  protected:
+    OpVec ops;
+    TensorVec tensors;
+    TensorVec inputs;
+    TensorVec outputs;
+
+  public:
+    GraphBase() {}
+    GraphBase(const GraphBase &) = delete;
+    virtual ~GraphBase(); // owns its operators and tensors
+
+    Tensor *tensor(const Dim &dims, Tensor::DataType dtype = Tensor::Float32);
+    Tensor *tensor(const Dim &dims, const std::string &dtype);
+    void addTensor(Tensor *t) { tensors.push_back(t); }
+    TensorVec &getTensors() { return tensors; }
+    OpVec &getOperators() { return ops; }
+    const OpVec &getOperators() const { return ops; }
+    TensorVec &getInputs() { return inputs; }
+    const TensorVec &getInputs() const { return inputs; }
+    TensorVec &getOutputs() { return outputs; }
+    const TensorVec &getOutputs() const { return outputs; }
+
+    // Fills inputOf / outputOf, predecessors / successors and the graph's
+    // input and output lists from the operators' tensor lists.
+    void updateConnection();
+    void removeOps(OpVec &removed);
+    // Operators in a topological order (Kahn, ties in insertion order).
+    bool topoOrder(OpVec &order) const;
+};
+
+class Graph : public GraphBase {
+  public:
+    Graph() {}
+
+    Operator *conv(Tensor *input, Tensor *weight, Tensor *output, int ph, int pw, int sh = 1,
+                   int sw = 1, int dh = 1, int dw = 1, Tensor *bias = nullptr);
+    Operator *conv(Tensor *input, Tensor *weight, int ph, int pw, int sh = 1, int sw = 1,
+                   int dh = 1, int dw = 1, Tensor *bias = nullptr);
+    Operator *conv(Tensor *input, Tensor *weight, Tensor *output, ConvOp::PaddingMode pm,
+                   int sh = 1, int sw = 1, int dh = 1, int dw = 1, Tensor *bias = nullptr);
+    Operator *conv(Tensor *input, Tensor *weight, ConvOp::PaddingMode pm, int sh = 1, int sw = 1,
+                   int dh = 1, int dw = 1, Tensor *bias = nullptr);
+    Operator *conv3d(Tensor *input, Tensor *weight, Tensor *output, const Dim &pad,
+                     const Dim &stride, const Dim &dilation, Tensor *bias = nullptr);
+    Operator *matmul(Tensor *A, Tensor *B, Tensor *C, bool transA = false, bool transB = false,
+                     Tensor *bias = nullptr);
+    Operator *matmul(Tensor *A, Tensor *B, bool transA = false, bool transB = false,
+                     Tensor *bias = nullptr);
+    Operator *pad(Tensor *input, Tensor *output, const Dim &begin, const Dim &end);
+    Operator *pad(Tensor *input, const Dim &begin, const Dim &end);
+    Operator *slice(Tensor *input, Tensor *output, const Dim &begin, const Dim &end);
+    Operator *slice(Tensor *input, const Dim &begin, const Dim &end);
+    Operator *concat(const TensorVec &inputs, Tensor *output, int dim);
+    Operator *concat(const TensorVec &inputs, int dim);
+    Operator *split(Tensor *input, const TensorVec &outputs, int dim, int num);
+    Operator *split(Tensor *input, int dim, int num);
+    Operator *split(Tensor *input, const TensorVec &outputs, int dim, std::vector<int> sizes);
+    Operator *split(Tensor *input, int dim, std::vector<int> sizes);
+    Operator *transpose(Tensor *input, Tensor *output, int split, const Perm &after,
+                        int factor = 2);
+    Operator *transpose(Tensor *input, int split, const Perm &after, int factor = 2);
+    Operator *flatten(Tensor *input, Tensor *output, int axis);
+    Operator *extend(Tensor *input, Tensor *output, int dim, int num);
+    Operator *extend(Tensor *input, int dim, int num);
+    Operator *maxpool(Tensor *input, Tensor *output, int kh, int kw, int dh, int dw, int ph,
+                      int pw, int sh, int sw);
+    Operator *avgpool(Tensor *input, Tensor *output, int kh, int kw, int ph, int pw, int sh,
+                      int sw);
+    Operator *avgpool(Tensor *input, Tensor *output); // global
+    Operator *add(const TensorVec &inputs, Tensor *output);
+    Operator *add(const TensorVec &inputs);
+    Operator *sub(Tensor *a, Tensor *b, Tensor *output);
+    Operator *mul(const TensorVec &inputs, Tensor *output);
+    Operator *mul(const TensorVec &inputs);
+    Operator *reshape(Tensor *input, Tensor *output);
+    Operator *identity(Tensor *input, Tensor *output);
+    Operator *relu(Tensor *input, Tensor *output);
+    Operator *relu(Tensor *input);
+    Operator *sigmoid(Tensor *input, Tensor *output);
+    Operator *tanh(Tensor *input, Tensor *output);
+    Operator *gelu(Tensor *input, Tensor *output);
+    Operator *softmax(Tensor *input, Tensor *output, int axis);
+    Operator *layernorm(Tensor *input, Tensor *output, Tensor *gamma, Tensor *beta,
+                        float eps = 1e-5f);
+
+    void setInputs(TensorVec v) { inputs = std::move(v); }
+    void setOutputs(TensorVec v) { outputs = std::move(v); }
+
+  private:
+    Operator *own(Operator *op);
+};
+
+class SubGraph : public GraphBase {
+    uint64_t hash = 2147483647;
+
+  public:
+    SubGraph() {}
+    // Clones the operators and their tensors (tensors are matched by hash).
+    explicit SubGraph(OpVec oplist);
+    SubGraph(const SubGraph &rhs) : SubGraph(rhs.ops) {}
+
+    // Runs every operator on the device in topological order.
+    bool compute();
+    // One output value; computes the graph if that has not happened yet.
+    const std::pair<bool, VType> compute(const Dim &point, size_t outputId = 0,
+                                         bool getAllPos = false);
+    // Seeds both graphs' inputs with the same data, runs both on the device
+    // and compares every output element for equality.
+    bool verification(SubGraph *mutant_graph, bool isFullComputing = true);
+    // Sum of op->perf() over the operators, in ms.
+    double perf(PerfEngine *pe, bool withPenalty = true);
+    uint64_t getHash();
+    int print();
+    int getComputeOps(OpVec &out);
+    void resetComputed();
+};
+
+} // namespace tpm

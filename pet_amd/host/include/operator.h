@@ -1,0 +1,654 @@
+// Operators of the PET graph on the MI355X backend (role of the reference's
+// include/operator.h). Same class names, constructor arguments and virtual
+// interface for the operators on the contraction / layout path, so the
+// mutators and the search engine can drive them unchanged; every compute()
+// and perf() runs HIP kernels through the C ABI (pet_hip.h), never the host.
+#pragma once
+#include "common.h"
+#include "perf.h"
+#include "tensor.h"
+#include "transpose.h"
+#include <sstream>
+
+namespace tpm {
+
+class PerfEngine;
+
+class Operator {
+  public:
+    // Numbering as in the reference (include/operator.h:19-51); the ops this
+    // backend does not execute are kept so type codes stay comparable.
+    enum OpType {
+        Unknown = 0,
+        Conv = 100,
+        Matmul,
+        ConvTrans,
+        G2BMM,
+        GBMML,
+        Pad,
+        Slice,
+        Concat,
+        Split,
+        Transpose,
+        Extend,
+        MaxPool,
+        AvgPool,
+        Add,
+        Sub,
+        Mul,
+        Div,
+        Pow,
+        Gather,
+        ReduceMean,
+        Reshape,
+        Identity,
+        BatchNorm = 200,
+        Softmax,
+        Activation,
+        Resize,
+        MemBound = 300,
+        Conv3d = 400, // not in the reference: ConvOp with a depth axis
+        LayerNorm,    // not in the reference
+    };
+    static std::string getOpName(OpType t);
+
+    enum ActType { None, Relu, Sigmoid, Tanh, Gelu /* Gelu is not in the reference */ };
+
+    Operator() : guid(generateGuid()), hash(generateHash()), type(Unknown) {}
+    explicit Operator(OpType type) : guid(generateGuid()), hash(generateHash()), type(type) {}
+    Operator(OpType type, TensorVec inputs, TensorVec outputs = {})
+        : guid(generateGuid()), hash(generateHash()), type(type), inputs(std::move(inputs)),
+          outputs(std::move(outputs)) {}
+    Operator(const Operator &rhs) : guid(generateGuid()), hash(rhs.hash), type(rhs.type) {}
+    virtual ~Operator() {}
+
+    bool isLinearOp() const { return type >= 100 && type < 200; }
+    bool isElementWiseOp() const { return type >= 200 && type < 300; }
+    bool isSplitOp() const { return type == Split; }
+    bool isConcatOp() const { return type == Concat; }
+    bool isComputeOp() const { return type == Conv || type == Matmul || type == Conv3d; }
+    bool isTransposeOp() const { return type == Transpose; }
+    bool isReshapeOp() const { return type == Reshape; }
+    bool isMemBoundOp() const { return type == MemBound || type == Activation || type == Transpose; }
+
+    bool isClear() const {
+        return inputs.empty() && outputs.empty() && successors.empty() && predecessors.empty();
+    }
+    void clear() {
+        inputs.clear();
+        outputs.clear();
+        successors.clear();
+        predecessors.clear();
+    }
+
+    void setSuccessors(OpVec v) { successors = std::move(v); }
+    void setPredecessors(OpVec v) { predecessors = std::move(v); }
+    void addSuccessors(Operator *op) { successors.push_back(op); }
+    void addPredecessors(Operator *op) { predecessors.push_back(op); }
+    OpVec &getSuccessors() { return successors; }
+    const OpVec &getSuccessors() const { return successors; }
+    OpVec &getPredecessors() { return predecessors; }
+    const OpVec &getPredecessors() const { return predecessors; }
+    Operator *getPredecessor() { return predecessors.size() == 1 ? predecessors[0] : nullptr; }
+
+    TensorVec &getInputs() { return inputs; }
+    const TensorVec &getInputs() const { return inputs; }
+    TensorVec &getOutputs() { return outputs; }
+    const TensorVec &getOutputs() const { return outputs; }
+    void setInputs(const TensorVec &v) { inputs = v; }
+    void setOutputs(const TensorVec &v) { outputs = v; }
+    Tensor *getInputs(size_t i) { return i < inputs.size() ? inputs[i] : nullptr; }
+    Tensor *getOutput() const { return isSplitOp() || outputs.empty() ? nullptr : outputs[0]; }
+    void addInput(Tensor *t) { inputs.push_back(t); }
+    void addOutput(Tensor *t) { outputs.push_back(t); }
+
+    // Time of one launch in ms on this GPU, hipEvent-timed on the backend
+    // stream and memoised in the PerfEngine; INFINITY if the backend rejects
+    // the shape.
+    virtual double perf(PerfEngine *pe, int rounds = 200, int warmupRounds = 200) = 0;
+    virtual Operator *clone() = 0;
+
+    // Computes the outputs on the device. nullptr when the operator rejects
+    // its shapes (same cases as the reference).
+    virtual Tensor *compute();
+    // Destination points -> (input ranges, closure that performs the
+    // computation). The closure always runs the whole operator on the device:
+    // there is no host arithmetic in this layer.
+    virtual std::pair<std::vector<DimRange>, std::function<bool()>> compute(DimRange dr);
+    virtual bool compute(const TensorVec &ins, const TensorVec &outs) {
+        return computeShape(ins, outs) && compute() != nullptr;
+    }
+
+    virtual Dim computeShape() = 0;
+    virtual bool computeShape(const TensorVec &ins, const TensorVec &outs);
+
+    virtual int numInputs() = 0;
+    virtual int numOutputs() = 0;
+    void print() const { std::cout << toString() << std::endl; }
+    virtual std::string toString() const = 0;
+    virtual std::string getName() const { return getOpName(type); }
+
+    size_t getGuid() const { return guid; }
+    uint64_t getHash() const { return hash; }
+    OpType getType() const { return type; }
+
+    virtual void inferSplittingPoints();
+    virtual void getOptypeAttr(std::string &optype, std::map<std::string, std::string> &attr,
+                               std::map<std::string, std::vector<int>> &extra) const;
+
+    // Issues the operator's kernels on `stream` with the tensors' device
+    // buffers (used by compute(), by perf() and by the graph runtime).
+    // Returns a pet_hip_status.
+    virtual int launch(pet_hip_stream_t stream) = 0;
+
+  protected:
+    virtual bool checkValid(const TensorVec &inputs) = 0;
+    virtual void initHash() = 0;
+    bool allocOutputs();
+    // hipEvent timing of `launch` on the backend stream.
+    double timeLaunches(int rounds, int warmupRounds);
+
+    const size_t guid;
+    uint64_t hash;
+    OpType type;
+    TensorVec inputs;
+    TensorVec outputs;
+    OpVec predecessors;
+    OpVec successors;
+};
+
+// ---- Conv ---------------------------------------------------------------------
+class ConvOp : public Operator {
+  public:
+    enum PaddingMode { Other, Same, Valid };
+
+    ConvOp(Tensor *input, Tensor *weight, Tensor *output, int ph, int pw, int sh = 1, int sw = 1,
+           int dh = 1, int dw = 1, Tensor *bias = nullptr, ActType act = None);
+    ConvOp(Tensor *input, Tensor *weight, int ph, int pw, int sh = 1, int sw = 1, int dh = 1,
+           int dw = 1, Tensor *bias = nullptr, ActType act = None);
+    ConvOp(int ph, int pw, int sh = 1, int sw = 1, int dh = 1, int dw = 1, Tensor *bias = nullptr,
+           ActType act = None);
+    ConvOp(Tensor *input, Tensor *weight, Tensor *output, PaddingMode pm = Same, int sh = 1,
+           int sw = 1, int dh = 1, int dw = 1, Tensor *bias = nullptr, ActType act = None);
+    ConvOp(Tensor *input, Tensor *weight, PaddingMode pm = Same, int sh = 1, int sw = 1,
+           int dh = 1, int dw = 1, Tensor *bias = nullptr, ActType act = None);
+    ConvOp(PaddingMode pm = Same, int sh = 1, int sw = 1, int dh = 1, int dw = 1,
+           Tensor *bias = nullptr, ActType act = None);
+    ConvOp(const ConvOp &rhs);
+    ConvOp *clone() override { return new ConvOp(*this); }
+
+    Dim computeShape() override;
+    Dim computeOutputPenalty(const Dim &p);
+    double perf(PerfEngine *pe, int rounds, int warmupRounds) override;
+    int launch(pet_hip_stream_t stream) override;
+    std::string toString() const override;
+    int numInputs() override { return 2; }
+    int numOutputs() override { return 1; }
+
+    Tensor *getBias() const { return bias; }
+    void setAct(ActType a) { act = a; }
+    ActType getAct() const { return act; }
+    bool same(const ConvOp &rhs);
+    PaddingMode getPaddingMode() { return padding; }
+    int getDh() const { return dh; }
+    int getDw() const { return dw; }
+    int getPh() const { return ph; }
+    int getPw() const { return pw; }
+    int getSh() const { return sh; }
+    int getSw() const { return sw; }
+    ConvArgs getArgs(int withPenalty) const;
+
+  private:
+    bool checkValid(const TensorVec &inputs) override;
+    void initHash() override;
+    void setPaddingMode();
+    // output extents for the current padding mode; updates ph / pw in the
+    // Same / Valid modes
+    void outputExtent(int h, int w, int r, int s, int &oh, int &ow);
+
+    int ph = 0, pw = 0, sh, sw, dh, dw;
+    Tensor *bias; // side pointer, not a graph edge
+    ActType act;
+    PaddingMode padding;
+};
+
+// ---- Conv3d (extension: the reference has no 3-D convolution) -----------------
+class Conv3dOp : public Operator {
+  public:
+    Conv3dOp(Tensor *input, Tensor *weight, Tensor *output, const Dim &pad, const Dim &stride,
+             const Dim &dilation, Tensor *bias = nullptr, ActType act = None);
+    Conv3dOp(const Conv3dOp &rhs);
+    Conv3dOp *clone() override { return new Conv3dOp(*this); }
+    Dim computeShape() override;
+    double perf(PerfEngine *pe, int rounds, int warmupRounds) override;
+    int launch(pet_hip_stream_t stream) override;
+    std::string toString() const override;
+    int numInputs() override { return 2; }
+    int numOutputs() override { return 1; }
+    void setAct(ActType a) { act = a; }
+    ActType getAct() const { return act; }
+    Tensor *getBias() const { return bias; }
+    const Dim &getPad() const { return pad; }
+    const Dim &getStride() const { return stride; }
+    const Dim &getDilation() const { return dilation; }
+
+  private:
+    bool checkValid(const TensorVec &inputs) override;
+    void initHash() override;
+    Dim pad, stride, dilation; // (t, h, w)
+    Tensor *bias;
+    ActType act;
+};
+
+// ---- Matmul -------------------------------------------------------------------
+class MatmulOp : public Operator {
+  public:
+    MatmulOp(Tensor *A, Tensor *B, Tensor *C, bool transA = false, bool transB = false,
+             Tensor *bias = nullptr, ActType act = None);
+    MatmulOp(Tensor *A, Tensor *B, bool transA = false, bool transB = false,
+             Tensor *bias = nullptr, ActType act = None);
+    MatmulOp(bool transA = false, bool transB = false, Tensor *bias = nullptr, ActType act = None);
+    MatmulOp(const MatmulOp &rhs)
+        : Operator(rhs), transA(rhs.transA), transB(rhs.transB), bias(rhs.bias), act(rhs.act) {}
+    MatmulOp *clone() override { return new MatmulOp(*this); }
+
+    Dim computeShape() override;
+    double perf(PerfEngine *pe, int rounds, int warmupRounds) override;
+    int launch(pet_hip_stream_t stream) override;
+    std::string toString() const override;
+    int numInputs() override { return 2; }
+    int numOutputs() override { return 1; }
+    Tensor *getBias() const { return bias; }
+    void setAct(ActType a) { act = a; }
+    ActType getAct() const { return act; }
+    bool getTransA() const { return transA; }
+    bool getTransB() const { return transB; }
+    MatmulArgs getArgs() const;
+    void dimExtend(Tensor *t); // 2-D tensors get a leading 1
+
+  private:
+    bool checkValid(const TensorVec &inputs) override;
+    void initHash() override;
+    void markWeight(Tensor *A, Tensor *B);
+    bool transA, transB;
+    Tensor *bias;
+    ActType act;
+};
+
+// ---- Pad / Slice --------------------------------------------------------------
+class PadOp : public Operator {
+  public:
+    PadOp(Tensor *input, Tensor *output, const Dim &begin, const Dim &end);
+    PadOp(Tensor *input, const Dim &begin, const Dim &end);
+    PadOp(const Dim &begin, const Dim &end);
+    PadOp(const PadOp &rhs) : Operator(rhs), begin(rhs.begin), end(rhs.end) {}
+    PadOp *clone() override { return new PadOp(*this); }
+    Dim computeShape() override;
+    double perf(PerfEngine *pe, int rounds, int warmupRounds) override;
+    int launch(pet_hip_stream_t stream) override;
+    std::string toString() const override;
+    int numInputs() override { return 1; }
+    int numOutputs() override { return 1; }
+    const Dim &getBegin() const { return begin; }
+    const Dim &getEnd() const { return end; }
+
+  private:
+    bool checkValid(const TensorVec &inputs) override;
+    void initHash() override;
+    Dim begin, end;
+};
+
+class SliceOp : public Operator {
+  public:
+    SliceOp(Tensor *input, Tensor *output, const Dim &begin, const Dim &end);
+    SliceOp(Tensor *input, const Dim &begin, const Dim &end);
+    SliceOp(const Dim &begin, const Dim &end);
+    SliceOp(const SliceOp &rhs) : Operator(rhs), begin(rhs.begin), end(rhs.end) {}
+    SliceOp *clone() override { return new SliceOp(*this); }
+    Dim computeShape() override;
+    double perf(PerfEngine *pe, int rounds, int warmupRounds) override;
+    int launch(pet_hip_stream_t stream) override;
+    std::string toString() const override;
+    int numInputs() override { return 1; }
+    int numOutputs() override { return 1; }
+    const Dim &getBegin() const { return begin; }
+    const Dim &getEnd() const { return end; }
+
+  private:
+    bool checkValid(const TensorVec &inputs) override;
+    void initHash() override;
+    Dim begin, end;
+};
+
+// ---- Concat / Split -------------------------------------------------------------
+class ConcatOp : public Operator {
+  public:
+    ConcatOp(TensorVec inputs, int dim);
+    ConcatOp(TensorVec inputs, Tensor *output, int dim);
+    explicit ConcatOp(int dim);
+    ConcatOp(const ConcatOp &rhs) : Operator(rhs), dim(rhs.dim) {}
+    ConcatOp *clone() override { return new ConcatOp(*this); }
+    Dim computeShape() override;
+    double perf(PerfEngine *pe, int rounds, int warmupRounds) override;
+    int launch(pet_hip_stream_t stream) override;
+    std::string toString() const override;
+    int numInputs() override { return (int)inputs.size(); }
+    int numOutputs() override { return 1; }
+    int getDim() const { return dim; }
+
+  private:
+    bool checkValid(const TensorVec &inputs) override;
+    void initHash() override;
+    int dim;
+};
+
+class SplitOp : public Operator {
+  public:
+    SplitOp(Tensor *input, int dim, int num);
+    SplitOp(Tensor *input, int dim, const std::vector<int> &sizes);
+    SplitOp(Tensor *input, const TensorVec &outputs, int dim, const std::vector<int> &sizes);
+    SplitOp(int dim, int num);
+    SplitOp(int dim, const std::vector<int> &sizes);
+    SplitOp(const SplitOp &rhs) : Operator(rhs), dim(rhs.dim), num(rhs.num), sizes(rhs.sizes) {}
+    SplitOp *clone() override { return new SplitOp(*this); }
+
+    Tensor *compute() override; // returns outputs[0] (the reference asserts here)
+    TensorVec computeV();
+    Dim computeShape() override;            // dims of output 0
+    std::vector<Dim> computeShapeV();       // ratio rule; empty when not divisible
+    bool computeShape(const TensorVec &ins, const TensorVec &outs) override;
+    double perf(PerfEngine *pe, int rounds, int warmupRounds) override;
+    int launch(pet_hip_stream_t stream) override;
+    std::string toString() const override;
+    int numInputs() override { return 1; }
+    int numOutputs() override { return (int)outputs.size(); }
+    int getDim() const { return dim; }
+    const std::vector<int> &getSizes() const { return sizes; }
+
+  private:
+    bool checkValid(const TensorVec &) override { return true; }
+    void initHash() override;
+    int dim, num;
+    std::vector<int> sizes; // ratios of the split dim
+};
+
+// ---- Transpose ------------------------------------------------------------------
+class PermItem {
+    friend class Perm;
+    std::vector<int> items;
+
+  public:
+    PermItem(int i) : items({i}) {}
+    PermItem(std::initializer_list<int> lst) : items(lst) {}
+    PermItem(const std::vector<int> &lst) : items(lst) {}
+    bool isSingle() const { return items.size() == 1; }
+    int getSingle() const { return items[0]; }
+    std::vector<int> &getVec() { return items; }
+    const std::vector<int> &getVec() const { return items; }
+    std::string toString() const;
+};
+
+class Perm {
+    std::vector<PermItem> perm;
+
+  public:
+    Perm(std::initializer_list<PermItem> perm) : perm(perm) {}
+    Perm(const std::vector<PermItem> &perm) : perm(perm) {}
+    std::vector<int> asVector() const;
+    std::vector<PermItem> &getPerm() { return perm; }
+    const std::vector<PermItem> &getPerm() const { return perm; }
+    PermItem &operator[](size_t i) { return perm[i]; }
+    const PermItem &operator[](size_t i) const { return perm[i]; }
+    size_t size() const { return perm.size(); }
+    std::string toString() const;
+};
+
+class TransposeOp : public Operator {
+  public:
+    enum TransType { NoneType, N2H, N2W, H2N, W2N, C2H, C2W, D2H, D2W };
+    enum TransPos { NonePos, Pre, Post };
+
+    TransposeOp(Tensor *input, Tensor *output, const Perm &before, const Perm &after,
+                int factor = 2, TransType trans_type = NoneType);
+    // In `after`, -1 names the dim the split introduces.
+    TransposeOp(Tensor *input, Tensor *output, int split, const Perm &after, int factor = 2,
+                TransType trans_type = NoneType);
+    TransposeOp(Tensor *input, int split, const Perm &after, int factor = 2,
+                TransType trans_type = NoneType);
+    TransposeOp(int split, const Perm &after, int factor = 2, TransType trans_type = NoneType);
+    TransposeOp(const TransposeOp &rhs);
+    TransposeOp *clone() override { return new TransposeOp(*this); }
+
+    Dim computeShape() override;
+    double perf(PerfEngine *pe, int rounds, int warmupRounds) override;
+    int launch(pet_hip_stream_t stream) override;
+    std::string toString() const override;
+    int numInputs() override { return 1; }
+    int numOutputs() override { return 1; }
+
+    // Micro-op lowering with the boundary-correction parameters: a Pre H2N/W2N
+    // split carries `padding` halo rows (copys), the matching Post fuse drops
+    // them (dels); a Pre N2H/N2W fuse inserts zero rows (pad), the Post split
+    // skips them (extr).
+    std::vector<std::shared_ptr<TransBasic>> getTTParam() const;
+
+    void setPos(TransPos pos) { trans_pos = pos; }
+    TransPos getPos() const { return trans_pos; }
+    void setType(TransType t) { trans_type = t; }
+    TransType getType() const { return trans_type; }
+    std::pair<int, int> getPaddingSize() const { return {padding_h, padding_w}; }
+    // With a non-zero padding size the operator runs its corrected form and
+    // its output shape changes accordingly.
+    void setPaddingSize(int h, int w) {
+        padding_h = h;
+        padding_w = w;
+    }
+    std::pair<Perm, Perm> getBeforeAndAfter() { return {before, after}; }
+    int getSplit() const { return split; }
+    int getFactor() const { return factor; }
+
+  private:
+    bool checkValid(const TensorVec &inputs) override;
+    void initHash() override;
+    void setParam(int dimSz);
+    bool flatDims(Dim &flat) const; // false when the split does not divide
+    bool corrected() const;
+
+    Perm before, after;
+    int split, factor;
+    TransType trans_type;
+    TransPos trans_pos = NonePos;
+    int padding_h = 0, padding_w = 0;
+};
+
+// ---- Extend ---------------------------------------------------------------------
+class ExtendOp : public Operator {
+  public:
+    ExtendOp(Tensor *input, Tensor *output, int dim, int num = 1);
+    ExtendOp(Tensor *input, int dim, int num);
+    ExtendOp(int dim, int num);
+    ExtendOp(const ExtendOp &rhs) : Operator(rhs), dim(rhs.dim), num(rhs.num) {}
+    ExtendOp *clone() override { return new ExtendOp(*this); }
+    Dim computeShape() override;
+    double perf(PerfEngine *pe, int rounds, int warmupRounds) override;
+    int launch(pet_hip_stream_t stream) override;
+    std::string toString() const override;
+    int numInputs() override { return 1; }
+    int numOutputs() override { return 1; }
+    int getDim() const { return dim; }
+    int getNum() const { return num; }
+
+  private:
+    bool checkValid(const TensorVec &) override { return true; }
+    void initHash() override;
+    int dim, num;
+};
+
+// ---- element-wise: Add / Sub / Mul (flat-modulo broadcast) ------------------------
+class EltwiseOp : public Operator {
+  public:
+    EltwiseOp(OpType type, TensorVec inputs, Tensor *output);
+    explicit EltwiseOp(OpType type) : Operator(type) { initHash(); }
+    EltwiseOp(const EltwiseOp &rhs) : Operator(rhs) {}
+    Dim computeShape() override;
+    double perf(PerfEngine *pe, int rounds, int warmupRounds) override;
+    int launch(pet_hip_stream_t stream) override;
+    std::string toString() const override;
+    int numInputs() override { return type == Sub ? 2 : (int)inputs.size(); }
+    int numOutputs() override { return 1; }
+    bool computeShape(const TensorVec &ins, const TensorVec &outs) override;
+
+  protected:
+    bool checkValid(const TensorVec &inputs) override;
+    void initHash() override;
+};
+
+class AddOp : public EltwiseOp {
+  public:
+    AddOp(TensorVec inputs, Tensor *output) : EltwiseOp(Add, std::move(inputs), output) {}
+    explicit AddOp(TensorVec inputs) : EltwiseOp(Add, std::move(inputs), nullptr) {}
+    AddOp() : EltwiseOp(Add) {}
+    AddOp *clone() override { return new AddOp(*this); }
+};
+
+class SubOp : public EltwiseOp {
+  public:
+    SubOp(Tensor *a, Tensor *b, Tensor *output = nullptr) : EltwiseOp(Sub, {a, b}, output) {}
+    SubOp() : EltwiseOp(Sub) {}
+    SubOp *clone() override { return new SubOp(*this); }
+};
+
+class MulOp : public EltwiseOp {
+  public:
+    MulOp(TensorVec inputs, Tensor *output) : EltwiseOp(Mul, std::move(inputs), output) {}
+    explicit MulOp(TensorVec inputs) : EltwiseOp(Mul, std::move(inputs), nullptr) {}
+    MulOp() : EltwiseOp(Mul) {}
+    MulOp *clone() override { return new MulOp(*this); }
+};
+
+// ---- single-input ops without a reference CPU compute ----------------------------
+class ActivationOp : public Operator {
+  public:
+    ActivationOp(Tensor *input, Tensor *output, ActType act);
+    ActivationOp(Tensor *input, ActType act);
+    explicit ActivationOp(ActType act);
+    ActivationOp(const ActivationOp &rhs) : Operator(rhs), actType(rhs.actType) {}
+    ActivationOp *clone() override { return new ActivationOp(*this); }
+    Dim computeShape() override;
+    double perf(PerfEngine *pe, int rounds, int warmupRounds) override;
+    int launch(pet_hip_stream_t stream) override;
+    std::string toString() const override;
+    int numInputs() override { return 1; }
+    int numOutputs() override { return 1; }
+    ActType getActType() const { return actType; }
+
+  private:
+    bool checkValid(const TensorVec &) override { return true; }
+    void initHash() override;
+    ActType actType;
+};
+
+// Max / average pooling (one class, as the two differ in one flag).
+class PoolOp : public Operator {
+  public:
+    PoolOp(OpType type, Tensor *input, Tensor *output, int kh, int kw, int dh, int dw, int ph,
+           int pw, int sh, int sw);
+    PoolOp(const PoolOp &rhs);
+    PoolOp *clone() override { return new PoolOp(*this); }
+    Dim computeShape() override;
+    double perf(PerfEngine *pe, int rounds, int warmupRounds) override;
+    int launch(pet_hip_stream_t stream) override;
+    std::string toString() const override;
+    int numInputs() override { return 1; }
+    int numOutputs() override { return 1; }
+    PoolArgs getArgs() const { return PoolArgs{kh, kw, ph, pw, sh, sw, dh, dw}; }
+
+  private:
+    bool checkValid(const TensorVec &inputs) override;
+    void initHash() override;
+    int kh, kw, dh, dw, ph, pw, sh, sw;
+};
+
+class MaxPoolOp : public PoolOp {
+  public:
+    MaxPoolOp(Tensor *input, Tensor *output, int kh, int kw, int dh, int dw, int ph, int pw,
+              int sh, int sw)
+        : PoolOp(MaxPool, input, output, kh, kw, dh, dw, ph, pw, sh, sw) {}
+};
+
+class AvgPoolOp : public PoolOp {
+  public:
+    AvgPoolOp(Tensor *input, Tensor *output, int kh, int kw, int ph, int pw, int sh, int sw)
+        : PoolOp(AvgPool, input, output, kh, kw, 1, 1, ph, pw, sh, sw) {}
+    // global average pool
+    AvgPoolOp(Tensor *input, Tensor *output);
+};
+
+class SoftmaxOp : public Operator {
+  public:
+    SoftmaxOp(Tensor *input, Tensor *output, int axis);
+    SoftmaxOp(const SoftmaxOp &rhs) : Operator(rhs), axis(rhs.axis) {}
+    SoftmaxOp *clone() override { return new SoftmaxOp(*this); }
+    Dim computeShape() override;
+    double perf(PerfEngine *pe, int rounds, int warmupRounds) override;
+    int launch(pet_hip_stream_t stream) override;
+    std::string toString() const override;
+    int numInputs() override { return 1; }
+    int numOutputs() override { return 1; }
+
+  private:
+    bool checkValid(const TensorVec &inputs) override;
+    void initHash() override;
+    int axis; // must be the last axis
+};
+
+class LayerNormOp : public Operator {
+  public:
+    LayerNormOp(Tensor *input, Tensor *output, Tensor *gamma, Tensor *beta, float eps = 1e-5f);
+    LayerNormOp(const LayerNormOp &rhs)
+        : Operator(rhs), gamma(rhs.gamma), beta(rhs.beta), eps(rhs.eps) {}
+    LayerNormOp *clone() override { return new LayerNormOp(*this); }
+    Dim computeShape() override;
+    double perf(PerfEngine *pe, int rounds, int warmupRounds) override;
+    int launch(pet_hip_stream_t stream) override;
+    std::string toString() const override;
+    int numInputs() override { return 1; }
+    int numOutputs() override { return 1; }
+    Tensor *getGamma() const { return gamma; }
+    Tensor *getBeta() const { return beta; }
+    float getEps() const { return eps; }
+
+  private:
+    bool checkValid(const TensorVec &) override { return true; }
+    void initHash() override;
+    Tensor *gamma, *beta; // side pointers like a conv bias
+    float eps;
+};
+
+// Reshape / Identity: a copy with the output's dims (element count must match).
+class ReshapeOp : public Operator {
+  public:
+    ReshapeOp(Tensor *input, Tensor *output);
+    ReshapeOp(const ReshapeOp &rhs) : Operator(rhs) {}
+    ReshapeOp *clone() override { return new ReshapeOp(*this); }
+    Dim computeShape() override;
+    double perf(PerfEngine *pe, int rounds, int warmupRounds) override;
+    int launch(pet_hip_stream_t stream) override;
+    std::string toString() const override;
+    int numInputs() override { return 1; }
+    int numOutputs() override { return 1; }
+
+  protected:
+    ReshapeOp(OpType type, Tensor *input, Tensor *output);
+    bool checkValid(const TensorVec &inputs) override;
+    void initHash() override;
+};
+
+class IdentityOp : public ReshapeOp {
+  public:
+    IdentityOp(Tensor *input, Tensor *output) : ReshapeOp(Identity, input, output) {}
+    IdentityOp *clone() override { return new IdentityOp(*this); }
+    Dim computeShape() override;
+};
+
+} // namespace tpm

@@ -1,0 +1,491 @@
+#include "code_engine.h"
+
+#include <algorithm>
+#include <fstream>
+#include <set>
+#include <sstream>
+#include <unordered_map>
+
+namespace tpm {
+
+// ---- GraphExec ----------------------------------------------------------------
+
+GraphExec::~GraphExec() {
+    if (graph) {
+        pet_hip_stream_sync(petStream());
+        pet_hip_graph_destroy(graph);
+    }
+}
+
+bool GraphExec::launch() {
+    return graph && petOk(pet_hip_graph_launch(graph, petStream()), "pet_hip_graph_launch");
+}
+
+bool GraphExec::sync() { return petOk(pet_hip_stream_sync(petStream()), "pet_hip_stream_sync"); }
+
+double GraphExec::time(int warmup, int rounds) {
+    for (int i = 0; i < warmup; ++i)
+        if (!launch())
+            return INFINITY;
+    pet_hip_event_t e0 = nullptr, e1 = nullptr;
+    pet_hip_event_create(&e0);
+    pet_hip_event_create(&e1);
+    pet_hip_event_record(e0, petStream());
+    for (int i = 0; i < rounds; ++i)
+        launch();
+    pet_hip_event_record(e1, petStream());
+    pet_hip_event_sync(e1);
+    float ms = 0.f;
+    pet_hip_event_elapsed_ms(&ms, e0, e1);
+    pet_hip_event_destroy(e0);
+    pet_hip_event_destroy(e1);
+    return rounds > 0 ? (double)ms / rounds : 0.0;
+}
+
+namespace {
+
+// Which operators need no kernel because their tensors can share storage.
+struct AliasPlan {
+    std::set<const Operator *> skipped;
+};
+
+bool weightOnly(const Operator *op) {
+    if (op->getInputs().empty())
+        return false;
+    for (auto t : op->getInputs())
+        if (t->getType() != Tensor::Weight)
+            return false;
+    return true;
+}
+
+size_t elems(const Tensor *t) { return t->size(); }
+
+} // namespace
+
+// Storage sharing, decided before anything is captured:
+//  * Split on dim 0: every output is a slab of the input buffer.
+//  * Concat on dim 0: every input that an operator of this graph produces (and
+//    that is used nowhere else in a conflicting way) is produced directly
+//    into its slab of the output buffer.
+//  * Reshape: the output is the input buffer.
+static AliasPlan planAliases(const OpVec &order) {
+    AliasPlan plan;
+    std::set<const Tensor *> aliased;
+    for (auto op : order) {
+        if (op->getType() == Operator::Split && static_cast<SplitOp *>(op)->getDim() == 0) {
+            Tensor *in = op->getInputs()[0];
+            float *base = in->devicePtr();
+            size_t off = 0;
+            for (auto out : op->getOutputs()) {
+                out->aliasDevice(base + off);
+                aliased.insert(out);
+                off += elems(out);
+            }
+            plan.skipped.insert(op);
+        } else if (op->getType() == Operator::Reshape) {
+            Tensor *in = op->getInputs()[0], *out = op->getOutputs()[0];
+            if (elems(in) == elems(out)) {
+                out->aliasDevice(in->devicePtr());
+                aliased.insert(out);
+                plan.skipped.insert(op);
+            }
+        }
+    }
+    // Concat: the output buffer must exist before its producers' buffers are
+    // redirected, and a part can only live in one place.
+    for (auto op : order) {
+        if (op->getType() != Operator::Concat || static_cast<ConcatOp *>(op)->getDim() != 0)
+            continue;
+        bool ok = true;
+        std::set<const Tensor *> seen;
+        for (auto in : op->getInputs()) {
+            Operator *prod = in->getOutputOf();
+            if (prod == nullptr || aliased.count(in) || !seen.insert(in).second ||
+                plan.skipped.count(prod))
+                ok = false;
+        }
+        if (!ok)
+            continue;
+        Tensor *out = op->getOutputs()[0];
+        float *base = out->devicePtr();
+        size_t off = 0;
+        for (auto in : op->getInputs()) {
+            in->aliasDevice(base + off);
+            aliased.insert(in);
+            off += elems(in);
+        }
+        plan.skipped.insert(op);
+    }
+    return plan;
+}
+
+std::unique_ptr<GraphExec> CodeEngine::instantiate(std::shared_ptr<SubGraph> &graph) {
+    if (!petInit())
+        return nullptr;
+    OpVec order;
+    if (!graph->topoOrder(order)) {
+        std::fprintf(stderr, "[pet] graph has a cycle\n");
+        return nullptr;
+    }
+    // settle every buffer (allocation + upload of host-side data) before capture
+    for (auto t : graph->getTensors())
+        if (!t->isValid() || t->devicePtr() == nullptr)
+            return nullptr;
+    for (auto op : order) {
+        if (auto conv = dynamic_cast<ConvOp *>(op))
+            if (conv->getBias())
+                conv->getBias()->devicePtr();
+        if (auto mm = dynamic_cast<MatmulOp *>(op))
+            if (mm->getBias())
+                mm->getBias()->devicePtr();
+        if (auto c3 = dynamic_cast<Conv3dOp *>(op))
+            if (c3->getBias())
+                c3->getBias()->devicePtr();
+        if (auto ln = dynamic_cast<LayerNormOp *>(op))
+            for (Tensor *t : {ln->getGamma(), ln->getBeta()})
+                if (t)
+                    t->devicePtr();
+    }
+    AliasPlan plan = planAliases(order);
+
+    std::unique_ptr<GraphExec> exec(new GraphExec());
+    pet_hip_stream_t s = petStream();
+    // operators that only touch weights run once, outside the replayed graph
+    // (the reference's "Preprocess operators for weights" block,
+    // src/Graph/code_engine.cc:183-190)
+    for (auto op : order)
+        if (weightOnly(op) && !plan.skipped.count(op)) {
+            if (op->launch(s) != PET_HIP_OK)
+                return nullptr;
+            for (auto t : op->getOutputs())
+                t->deviceWritten();
+        }
+    if (!petOk(pet_hip_stream_sync(s), "pet_hip_stream_sync"))
+        return nullptr;
+    if (!petOk(pet_hip_graph_begin_capture(s), "pet_hip_graph_begin_capture"))
+        return nullptr;
+    bool ok = true;
+    for (auto op : order) {
+        if (plan.skipped.count(op)) {
+            exec->nAliasOps++;
+            continue;
+        }
+        if (weightOnly(op))
+            continue;
+        if (op->launch(s) != PET_HIP_OK) {
+            std::fprintf(stderr, "[pet] capture of %s failed: %s\n", op->toString().c_str(),
+                         pet_hip_last_error());
+            ok = false;
+            break;
+        }
+        exec->nLaunchOps++;
+    }
+    pet_hip_graph_t g = nullptr;
+    if (!petOk(pet_hip_graph_end_capture(s, &g), "pet_hip_graph_end_capture") || !ok) {
+        if (g)
+            pet_hip_graph_destroy(g);
+        return nullptr;
+    }
+    exec->graph = g;
+    for (auto t : graph->getTensors())
+        if (t->getOutputOf() != nullptr) {
+            t->deviceWritten();
+            t->setComputed();
+        }
+    return exec;
+}
+
+// ---- emitted program ------------------------------------------------------------
+
+namespace {
+
+struct Emitter {
+    std::ostringstream os;
+    std::unordered_map<const Tensor *, std::string> names;
+    int counter = 0;
+
+    std::string name(const Tensor *t) {
+        auto it = names.find(t);
+        if (it != names.end())
+            return it->second;
+        std::string n = "t" + std::to_string(counter++);
+        names.emplace(t, n);
+        return n;
+    }
+    std::string ints(const std::vector<int> &v) {
+        std::string s = "{";
+        for (size_t i = 0; i < v.size(); ++i)
+            s += (i ? ", " : "") + std::to_string(v[i]);
+        return s + "}";
+    }
+    void line(const std::string &l) { os << l << "\n"; }
+};
+
+std::string nullable(Emitter &e, Tensor *t) { return t ? e.name(t) : std::string("nullptr"); }
+
+} // namespace
+
+std::string CodeEngine::genCode(std::shared_ptr<SubGraph> &graph) {
+    OpVec order;
+    if (!graph->topoOrder(order))
+        return "";
+    Emitter e;
+    e.line("// Generated by tpm::CodeEngine for the MI355X backend.");
+    e.line("// Build: hipcc -O2 prog.cpp -I<repo>/include -L<repo>/pet_amd/lib -lpet_hip "
+           "-Wl,-rpath,<repo>/pet_amd/lib -o prog");
+    e.line("#include <cstdio>");
+    e.line("#include <cstdlib>");
+    e.line("#include \"pet_hip.h\"");
+    e.line("#define CHECK(x) do { int _s = (x); if (_s) { std::fprintf(stderr, \"%s: %s\\n\", #x, "
+           "pet_hip_last_error()); std::exit(1); } } while (0)");
+    e.line("int main() {");
+    e.line("    CHECK(pet_hip_init(0));");
+    e.line("    pet_hip_stream_t s; CHECK(pet_hip_stream_create(&s));");
+    // tensors (bias side pointers included)
+    std::vector<Tensor *> all(graph->getTensors().begin(), graph->getTensors().end());
+    for (auto op : order) {
+        if (auto conv = dynamic_cast<ConvOp *>(op))
+            if (conv->getBias())
+                all.push_back(conv->getBias());
+        if (auto mm = dynamic_cast<MatmulOp *>(op))
+            if (mm->getBias())
+                all.push_back(mm->getBias());
+        if (auto c3 = dynamic_cast<Conv3dOp *>(op))
+            if (c3->getBias())
+                all.push_back(c3->getBias());
+        if (auto ln = dynamic_cast<LayerNormOp *>(op))
+            for (Tensor *t : {ln->getGamma(), ln->getBeta()})
+                if (t)
+                    all.push_back(t);
+    }
+    std::set<const Tensor *> viewOf;
+    std::set<const Operator *> skipped;
+    // storage sharing, mirrored from instantiate(): split / concat on dim 0, reshape
+    std::vector<std::string> aliasLines;
+    for (auto op : order) {
+        if (op->getType() == Operator::Split && static_cast<SplitOp *>(op)->getDim() == 0) {
+            size_t off = 0;
+            for (auto out : op->getOutputs()) {
+                aliasLines.push_back("    float *" + e.name(out) + " = " +
+                                     e.name(op->getInputs()[0]) + " + " + std::to_string(off) + ";");
+                viewOf.insert(out);
+                off += out->size();
+            }
+            skipped.insert(op);
+        } else if (op->getType() == Operator::Reshape) {
+            aliasLines.push_back("    float *" + e.name(op->getOutputs()[0]) + " = " +
+                                 e.name(op->getInputs()[0]) + ";");
+            viewOf.insert(op->getOutputs()[0]);
+            skipped.insert(op);
+        }
+    }
+    for (auto op : order) {
+        if (op->getType() != Operator::Concat || static_cast<ConcatOp *>(op)->getDim() != 0)
+            continue;
+        bool ok = true;
+        std::set<const Tensor *> seen;
+        for (auto in : op->getInputs())
+            if (in->getOutputOf() == nullptr || viewOf.count(in) || !seen.insert(in).second ||
+                skipped.count(in->getOutputOf()))
+                ok = false;
+        if (!ok)
+            continue;
+        size_t off = 0;
+        for (auto in : op->getInputs()) {
+            aliasLines.push_back("    float *" + e.name(in) + " = " + e.name(op->getOutputs()[0]) +
+                                 " + " + std::to_string(off) + ";");
+            viewOf.insert(in);
+            off += in->size();
+        }
+        skipped.insert(op);
+    }
+    uint64_t seed = 1;
+    for (auto t : all) {
+        if (viewOf.count(t))
+            continue;
+        std::string n = e.name(t);
+        e.line("    float *" + n + "; CHECK(pet_hip_malloc((void **)&" + n + ", " +
+               std::to_string(std::max<size_t>(t->size(), 1)) + " * sizeof(float)));");
+        // inputs and weights get uniform noise, as the reference's emitted
+        // program does with cuRAND (src/Graph/code_engine.cc:582-583)
+        if (t->getOutputOf() == nullptr)
+            e.line("    CHECK(pet_hip_rand_uniform_f32(" + n + ", " + std::to_string(t->size()) +
+                   ", " + std::to_string(seed++) + "ull, -1.f, 1.f, s));");
+    }
+    for (auto &l : aliasLines)
+        e.line(l);
+
+    auto emitOp = [&](Operator *op) -> bool {
+        std::ostringstream c;
+        auto in = [&](size_t i) { return e.name(op->getInputs()[i]); };
+        auto out = [&](size_t i) { return e.name(op->getOutputs()[i]); };
+        if (auto conv = dynamic_cast<ConvOp *>(op)) {
+            auto d = op->getInputs()[0]->getDims(), w = op->getInputs()[1]->getDims();
+            c << "pet_hip_conv2d_f32(" << in(0) << ", " << in(1) << ", "
+              << nullable(e, conv->getBias()) << ", " << out(0) << ", " << d[0] << ", " << d[1]
+              << ", " << d[2] << ", " << d[3] << ", " << w[0] << ", " << w[2] << ", " << w[3]
+              << ", " << conv->getPh() << ", " << conv->getPw() << ", " << conv->getSh() << ", "
+              << conv->getSw() << ", " << conv->getDh() << ", " << conv->getDw() << ", "
+              << d[1] / w[1] << ", " << (int)conv->getAct() << ", s)";
+        } else if (auto c3 = dynamic_cast<Conv3dOp *>(op)) {
+            auto d = op->getInputs()[0]->getDims(), w = op->getInputs()[1]->getDims();
+            c << "pet_hip_conv3d_f32(" << in(0) << ", " << in(1) << ", "
+              << nullable(e, c3->getBias()) << ", " << out(0);
+            for (int v : {d[0], d[1], d[2], d[3], d[4], w[0], w[2], w[3], w[4]})
+                c << ", " << v;
+            for (const Dim *v : {&c3->getPad(), &c3->getStride(), &c3->getDilation()})
+                for (int x : *v)
+                    c << ", " << x;
+            c << ", " << d[1] / w[1] << ", " << (int)c3->getAct() << ", s)";
+        } else if (auto ln = dynamic_cast<LayerNormOp *>(op)) {
+            size_t cols = (size_t)op->getInputs()[0]->getDims().back();
+            c << "pet_hip_layernorm(" << in(0) << ", " << nullable(e, ln->getGamma()) << ", "
+              << nullable(e, ln->getBeta()) << ", " << out(0) << ", "
+              << op->getInputs()[0]->size() / cols << ", " << cols << ", " << ln->getEps()
+              << "f, s)";
+        } else if (auto mm = dynamic_cast<MatmulOp *>(op)) {
+            bool ta, tb;
+            int b, m, n, k;
+            std::tie(ta, tb, b, m, n, k) = mm->getArgs();
+            c << "pet_hip_bmm_f32(" << ta << ", " << tb << ", " << b << ", " << m << ", " << n
+              << ", " << k << ", " << in(0) << ", " << in(1) << ", " << out(0) << ", "
+              << nullable(e, mm->getBias()) << ", " << (int)mm->getAct() << ", s)";
+        } else if (auto tr = dynamic_cast<TransposeOp *>(op)) {
+            TransProgram prog;
+            if (!TransposeEngine::getInstance().lower(tr->getTTParam(),
+                                                      op->getInputs()[0]->getDims(), prog))
+                return false;
+            std::string id = std::to_string(op->getGuid());
+            e.line("    static const int tin" + id + "[] = " + e.ints(prog.inDims) + ", tops" + id +
+                   "[] = " + e.ints(prog.ops) + ", tperm" + id + "[] = " + e.ints(prog.perms) + ";");
+            e.line("    // " + TransposeEngine::getInstance().describe(prog));
+            c << "pet_hip_trans_chain(" << in(0) << ", " << out(0) << ", tin" << id << ", "
+              << prog.inDims.size() << ", tops" << id << ", " << prog.nops << ", tperm" << id
+              << ", odims, &orank, s)";
+        } else if (auto sp = dynamic_cast<SplitOp *>(op)) {
+            std::string id = std::to_string(op->getGuid());
+            std::string ptrs = "{";
+            std::vector<int> sizes;
+            for (size_t i = 0; i < op->getOutputs().size(); ++i) {
+                ptrs += (i ? ", " : "") + out(i);
+                sizes.push_back(op->getOutputs()[i]->getDims()[sp->getDim()]);
+            }
+            e.line("    float *souts" + id + "[] = " + ptrs + "}; static const int sdims" + id +
+                   "[] = " + e.ints(op->getInputs()[0]->getDims()) + ", ssz" + id +
+                   "[] = " + e.ints(sizes) + ";");
+            c << "pet_hip_split(" << in(0) << ", souts" << id << ", " << sizes.size() << ", sdims"
+              << id << ", " << op->getInputs()[0]->getDims().size() << ", " << sp->getDim()
+              << ", ssz" << id << ", s)";
+        } else if (auto cc = dynamic_cast<ConcatOp *>(op)) {
+            std::string id = std::to_string(op->getGuid());
+            std::string ptrs = "{";
+            std::vector<int> sizes;
+            for (size_t i = 0; i < op->getInputs().size(); ++i) {
+                ptrs += (i ? ", " : "") + in(i);
+                sizes.push_back(op->getInputs()[i]->getDims()[cc->getDim()]);
+            }
+            e.line("    const float *cins" + id + "[] = " + ptrs + "}; static const int cdims" + id +
+                   "[] = " + e.ints(op->getOutputs()[0]->getDims()) + ", csz" + id +
+                   "[] = " + e.ints(sizes) + ";");
+            c << "pet_hip_concat(cins" << id << ", " << sizes.size() << ", " << out(0) << ", cdims"
+              << id << ", " << op->getOutputs()[0]->getDims().size() << ", " << cc->getDim()
+              << ", csz" << id << ", s)";
+        } else if (auto pd = dynamic_cast<PadOp *>(op)) {
+            std::string id = std::to_string(op->getGuid());
+            e.line("    static const int pdims" + id + "[] = " +
+                   e.ints(op->getInputs()[0]->getDims()) + ", pb" + id + "[] = " +
+                   e.ints(pd->getBegin()) + ", pe" + id + "[] = " + e.ints(pd->getEnd()) + ";");
+            c << "pet_hip_pad(" << in(0) << ", " << out(0) << ", pdims" << id << ", pb" << id
+              << ", pe" << id << ", " << pd->getBegin().size() << ", s)";
+        } else if (auto sl = dynamic_cast<SliceOp *>(op)) {
+            std::string id = std::to_string(op->getGuid());
+            e.line("    static const int ldims" + id + "[] = " +
+                   e.ints(op->getInputs()[0]->getDims()) + ", lb" + id + "[] = " +
+                   e.ints(sl->getBegin()) + ", le" + id + "[] = " + e.ints(sl->getEnd()) + ";");
+            c << "pet_hip_slice(" << in(0) << ", " << out(0) << ", ldims" << id << ", lb" << id
+              << ", le" << id << ", " << sl->getBegin().size() << ", s)";
+        } else if (auto ex = dynamic_cast<ExtendOp *>(op)) {
+            std::string id = std::to_string(op->getGuid());
+            e.line("    static const int edims" + id + "[] = " +
+                   e.ints(op->getInputs()[0]->getDims()) + ";");
+            c << "pet_hip_extend(" << in(0) << ", " << out(0) << ", edims" << id << ", "
+              << op->getInputs()[0]->getDims().size() << ", " << ex->getDim() << ", "
+              << ex->getNum() << ", s)";
+        } else if (dynamic_cast<EltwiseOp *>(op)) {
+            std::string id = std::to_string(op->getGuid());
+            std::string ptrs = "{", sizes = "{";
+            for (size_t i = 0; i < op->getInputs().size(); ++i) {
+                ptrs += (i ? ", " : "") + in(i);
+                sizes += (i ? ", " : "") + std::to_string(op->getInputs()[i]->size());
+            }
+            e.line("    const float *eins" + id + "[] = " + ptrs + "}; static const size_t esz" + id +
+                   "[] = " + sizes + "};");
+            int code = op->getType() == Operator::Add ? 0 : (op->getType() == Operator::Sub ? 1 : 2);
+            c << "pet_hip_eltwise(" << code << ", eins" << id << ", esz" << id << ", "
+              << op->getInputs().size() << ", " << out(0) << ", " << op->getOutputs()[0]->size()
+              << ", s)";
+        } else if (auto act = dynamic_cast<ActivationOp *>(op)) {
+            c << "pet_hip_activation(" << in(0) << ", " << out(0) << ", "
+              << op->getInputs()[0]->size() << ", " << (int)act->getActType() << ", s)";
+        } else if (auto pool = dynamic_cast<PoolOp *>(op)) {
+            int kh, kw, ph, pw, sh, sw, dh, dw;
+            std::tie(kh, kw, ph, pw, sh, sw, dh, dw) = pool->getArgs();
+            auto d = op->getInputs()[0]->getDims();
+            c << "pet_hip_pool2d(" << in(0) << ", " << out(0) << ", " << d[0] << ", " << d[1]
+              << ", " << d[2] << ", " << d[3] << ", " << kh << ", " << kw << ", " << ph << ", "
+              << pw << ", " << sh << ", " << sw << ", " << dh << ", " << dw << ", "
+              << (op->getType() == Operator::MaxPool ? 0 : 1) << ", s)";
+        } else if (dynamic_cast<SoftmaxOp *>(op)) {
+            size_t cols = (size_t)op->getInputs()[0]->getDims().back();
+            c << "pet_hip_softmax(" << in(0) << ", " << out(0) << ", "
+              << op->getInputs()[0]->size() / cols << ", " << cols << ", s)";
+        } else if (dynamic_cast<ReshapeOp *>(op)) {
+            c << "pet_hip_memcpy_d2d(" << out(0) << ", " << in(0) << ", "
+              << op->getInputs()[0]->size() << " * sizeof(float), s)";
+        } else {
+            return false;
+        }
+        e.line("    CHECK(" + c.str() + "); // " + op->toString());
+        return true;
+    };
+
+    e.line("    int odims[PET_HIP_MAX_RANK], orank = 0; (void)odims; (void)orank;");
+    e.line("    // operators that only touch weights run once");
+    for (auto op : order)
+        if (weightOnly(op) && !skipped.count(op) && !emitOp(op))
+            return "";
+    e.line("    CHECK(pet_hip_stream_sync(s));");
+    e.line("    // the rest is captured once and replayed as a HIP graph");
+    e.line("    CHECK(pet_hip_graph_begin_capture(s));");
+    for (auto op : order)
+        if (!weightOnly(op) && !skipped.count(op) && !emitOp(op))
+            return "";
+    e.line("    pet_hip_graph_t g; CHECK(pet_hip_graph_end_capture(s, &g));");
+    e.line("    pet_hip_event_t st, ed; CHECK(pet_hip_event_create(&st)); "
+           "CHECK(pet_hip_event_create(&ed));");
+    e.line("    int warmup = 100, rounds = 1000;");
+    e.line("    for (int i = 0; i < warmup + rounds; i++) {");
+    e.line("        if (i == warmup) CHECK(pet_hip_event_record(st, s));");
+    e.line("        CHECK(pet_hip_graph_launch(g, s));");
+    e.line("    }");
+    e.line("    CHECK(pet_hip_event_record(ed, s));");
+    e.line("    CHECK(pet_hip_event_sync(ed));");
+    e.line("    float duration; CHECK(pet_hip_event_elapsed_ms(&duration, st, ed));");
+    e.line("    std::printf(\" Time(ms) : %f\\n\", duration / rounds);");
+    e.line("    return 0;");
+    e.line("}");
+    return e.os.str();
+}
+
+int CodeEngine::genCode(std::shared_ptr<SubGraph> &graph, const std::string &filename) {
+    std::string code = genCode(graph);
+    if (code.empty())
+        return 1;
+    std::ofstream f(filename);
+    if (!f)
+        return 1;
+    f << code;
+    return 0;
+}
+
+} // namespace tpm

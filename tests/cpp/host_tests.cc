@@ -1,0 +1,397 @@
+// Test driver for the C++ host layer (tpm::Graph / Operator / PerfEngine /
+// CodeEngine on the MI355X backend). Cases follow the reference's own test
+// programs (src/Test/*.cc): device results are checked against the CPU oracle
+// (linked only into this binary) or against each other where the reference
+// tests an identity. Usage: pet_host_tests [case-name]; exit code 0 = pass.
+#include <cmath>
+#include <cstring>
+#include <fstream>
+#include <functional>
+#include <string>
+
+#include "code_engine.h"
+#include "graph.h"
+#include "perf_engine.h"
+
+using namespace tpm;
+
+extern "C" {
+int oracle_conv2d_f32(const float *x, const float *w, float *y, int n, int c, int h, int wd, int f,
+                      int cpg, int r, int s, int ph, int pw, int sh, int sw, int dh, int dw,
+                      int oh, int ow);
+int oracle_matmul_f32(const float *A, const float *B, float *C, int b, int m, int n, int k,
+                      int transA, int transB);
+int oracle_transpose_f32(const float *x, float *y, const int *flatDim, const int *after, int nflat);
+int oracle_conv_out_dim(int i, int k, int p, int s, int d);
+}
+
+#define EXPECT(cond)                                                                           \
+    do {                                                                                       \
+        if (!(cond)) {                                                                         \
+            std::printf("  FAILED %s:%d: %s\n", __FILE__, __LINE__, #cond);                    \
+            return false;                                                                      \
+        }                                                                                      \
+    } while (0)
+
+static void fillSmall(Tensor *t, int seed) { t->dataRand(seed); }
+
+static bool equalArrays(const float *a, const float *b, size_t n) {
+    for (size_t i = 0; i < n; ++i)
+        if (a[i] != b[i]) {
+            std::printf("  mismatch at %zu: %g vs %g\n", i, (double)a[i], (double)b[i]);
+            return false;
+        }
+    return true;
+}
+
+// src/Test/conv_test_3.cc: a 3x3 convolution on iota-like data; here the full
+// device result is checked against the oracle instead of point-wise compute.
+static bool test_conv_vs_oracle() {
+    const int n = 2, c = 16, h = 14, w = 14, f = 32, r = 3, s = 3;
+    Tensor i0({n, c, h, w}), w0({f, c, r, s}), o0;
+    fillSmall(&i0, 1);
+    fillSmall(&w0, 2);
+    ConvOp conv(&i0, &w0, &o0, 1, 1, 1, 1, 1, 1);
+    EXPECT(o0.getDims() == (Dim{n, f, h, w}));
+    EXPECT(conv.compute() != nullptr);
+    std::vector<float> ref(o0.size());
+    oracle_conv2d_f32(i0.getDataPtr(), w0.getDataPtr(), ref.data(), n, c, h, w, f, c, r, s, 1, 1,
+                      1, 1, 1, 1, h, w);
+    EXPECT(equalArrays(o0.getDataPtr(), ref.data(), ref.size()));
+    // shape rules: Same mode derives the padding, the d>1 & s>1 quirk is kept
+    Tensor i1({1, 4, 16, 16}), w1({4, 4, 3, 3}), o1;
+    ConvOp same(&i1, &w1, &o1, ConvOp::Same, 1, 1, 2, 2);
+    EXPECT(same.getPh() == 2 && o1.getDims() == (Dim{1, 4, 16, 16}));
+    Tensor o2;
+    ConvOp quirk(&i1, &w1, &o2, 0, 0, 2, 2, 2, 2);
+    EXPECT(o2.getDims()[2] == oracle_conv_out_dim(16, 3, 0, 2, 2) && o2.getDims()[2] == 7);
+    return true;
+}
+
+// f % groups != 0 -> compute() returns nullptr (src/Graph/operator.cc:108-109)
+static bool test_conv_invalid_groups() {
+    Tensor i0({1, 4, 5, 5}), w0({3, 2, 3, 3}), o0;
+    i0.dataRand(1);
+    w0.dataRand(2);
+    ConvOp conv(&i0, &w0, &o0, 1, 1);
+    EXPECT(conv.compute() == nullptr);
+    return true;
+}
+
+// src/Test/transpose_test_1.cc / transpose_test_2.cc: N2H and its inverse.
+static bool test_transpose_n2h_h2n() {
+    const int n = 4, c = 6, h = 8, w = 10;
+    Tensor x({n, c, h, w}), y, z;
+    fillSmall(&x, 3);
+    TransposeOp n2h(&x, &y, 0, {0, 1, {-1, 2}, 3}, 2, TransposeOp::N2H);
+    EXPECT(y.getDims() == (Dim{n / 2, c, 2 * h, w}));
+    EXPECT(n2h.compute() != nullptr);
+    int flat[5] = {n / 2, 2, c, h, w}, after[5] = {0, 2, 1, 3, 4};
+    std::vector<float> ref(x.size());
+    oracle_transpose_f32(x.getDataPtr(), ref.data(), flat, after, 5);
+    EXPECT(equalArrays(y.getDataPtr(), ref.data(), ref.size()));
+    TransposeOp h2n(&y, &z, 2, {{0, 2}, 1, -1, 3}, -2, TransposeOp::H2N);
+    EXPECT(z.getDims() == x.getDims());
+    EXPECT(h2n.compute() != nullptr);
+    EXPECT(equalArrays(z.getDataPtr(), x.getDataPtr(), x.size()));
+    // a split that does not divide is rejected
+    Tensor odd({3, 2, 4, 4}), bad;
+    odd.dataRand(1);
+    TransposeOp t(&odd, &bad, 0, {0, 1, {-1, 2}, 3}, 2);
+    EXPECT(!bad.isValid());
+    EXPECT(t.compute() == nullptr);
+    return true;
+}
+
+// src/Test/batch_gemm_test.cc: concat lhs, concat rhs, bmm, split == two matmuls.
+static bool test_batch_gemm_merge() {
+    const int m = 8, n = 8, k = 4;
+    Graph g1;
+    auto i0 = g1.tensor({1, m, k}), w0 = g1.tensor({1, k, n}), w1 = g1.tensor({1, k, n});
+    auto op0 = g1.matmul(i0, w0), op1 = g1.matmul(i0, w1);
+    g1.updateConnection();
+    std::vector<float> a(m * k), b0(k * n), b1(k * n);
+    for (size_t i = 0; i < a.size(); ++i)
+        a[i] = (float)i;
+    for (size_t i = 0; i < b0.size(); ++i) {
+        b0[i] = 3.f * i;
+        b1[i] = 7.f * i;
+    }
+    i0->setData(a.data());
+    w0->setData(b0.data());
+    w1->setData(b1.data());
+    EXPECT(op0->compute() && op1->compute());
+    auto o0 = op0->getOutputs()[0], o1 = op1->getOutputs()[0];
+    EXPECT(o0->getData({0, 0, 0}) == 336.f);
+
+    Graph g2;
+    auto l0 = g2.tensor({1, m, k}), r0 = g2.tensor({1, k, n}), r1 = g2.tensor({1, k, n});
+    auto c0 = g2.concat({l0, l0}, 0), c1 = g2.concat({r0, r1}, 0);
+    auto mm = g2.matmul(c0->getOutputs()[0], c1->getOutputs()[0]);
+    auto sp = g2.split(mm->getOutputs()[0], 0, std::vector<int>{1, 1});
+    g2.updateConnection();
+    l0->setData(a.data());
+    r0->setData(b0.data());
+    r1->setData(b1.data());
+    OpVec order;
+    EXPECT(g2.topoOrder(order) && order.size() == 4);
+    for (auto op : order)
+        EXPECT(op->compute() != nullptr);
+    EXPECT(equalArrays(sp->getOutputs()[0]->getDataPtr(), o0->getDataPtr(), o0->size()));
+    EXPECT(equalArrays(sp->getOutputs()[1]->getDataPtr(), o1->getDataPtr(), o1->size()));
+    return true;
+}
+
+// src/Test/pad_slice_test.cc: pad -> conv -> slice equals conv, checked with
+// SubGraph::verification (exact equality of all outputs on shared random data).
+static bool test_pad_conv_slice_verification() {
+    Graph g1, g2;
+    auto x1 = g1.tensor({1, 8, 7, 7}), w1 = g1.tensor({8, 8, 3, 3});
+    g1.conv(x1, w1, 1, 1);
+    g1.updateConnection();
+    auto x2 = g2.tensor({1, 8, 7, 7}), w2 = g2.tensor({8, 8, 3, 3});
+    auto p = g2.pad(x2, {0, 0, 0, 0}, {0, 0, 1, 1});
+    auto cv = g2.conv(p->getOutputs()[0], w2, 1, 1);
+    g2.slice(cv->getOutputs()[0], {0, 0, 0, 0}, {0, 0, 1, 1});
+    g2.updateConnection();
+    SubGraph s1(g1.getOperators()), s2(g2.getOperators());
+    EXPECT(s1.getInputs().size() == 2 && s2.getInputs().size() == 2);
+    EXPECT(s1.verification(&s2, true));
+    return true;
+}
+
+// BASELINE config 1, small: conv == H2N (halo) -> conv -> N2H (drop). Without
+// the correction the two programs differ at the seam.
+static bool test_corrected_h2n_program() {
+    const int c = 8, h = 12, w = 10, f = 8;
+    auto build = [&](Graph &g, bool corrected) {
+        auto x = g.tensor({1, c, h, w}), wt = g.tensor({f, c, 3, 3});
+        auto pre = static_cast<TransposeOp *>(g.transpose(x, 2, {{0, 2}, 1, -1, 3}, -2));
+        pre->setType(TransposeOp::H2N);
+        if (corrected) {
+            pre->setPos(TransposeOp::Pre);
+            pre->setPaddingSize(1, 1);
+            pre->computeShape();
+        }
+        auto cv = g.conv(pre->getOutputs()[0], wt, 1, 1);
+        auto post = static_cast<TransposeOp *>(
+            g.transpose(cv->getOutputs()[0], 0, {0, 1, {-1, 2}, 3}, 2));
+        post->setType(TransposeOp::N2H);
+        if (corrected) {
+            post->setPos(TransposeOp::Post);
+            post->setPaddingSize(1, 1);
+            post->computeShape();
+        }
+        g.updateConnection();
+        return post->getOutputs()[0];
+    };
+    Graph g0, g1, g2;
+    auto x0 = g0.tensor({1, c, h, w}), w0 = g0.tensor({f, c, 3, 3});
+    g0.conv(x0, w0, 1, 1);
+    g0.updateConnection();
+    Tensor *outC = build(g1, true);
+    Tensor *outP = build(g2, false);
+    EXPECT(outC->getDims() == (Dim{1, f, h, w}));
+    EXPECT(outP->getDims() == (Dim{1, f, h, w}));
+    SubGraph s0(g0.getOperators()), s1(g1.getOperators()), s2(g2.getOperators());
+    EXPECT(s0.verification(&s1, true));
+    EXPECT(!s0.verification(&s2, true)); // partially equivalent only
+    return true;
+}
+
+// Dilated conv == D2H, D2W (rows / columns de-interleaved into the batch) ->
+// dense conv -> inverse; two chained TransposeOps on each side.
+static bool test_dilated_space_to_batch_program() {
+    const int c = 8, hw = 16, f = 8;
+    Graph g0, g1;
+    auto x0 = g0.tensor({1, c, hw, hw}), w0 = g0.tensor({f, c, 3, 3});
+    g0.conv(x0, w0, 2, 2, 1, 1, 2, 2);
+    g0.updateConnection();
+    auto x1 = g1.tensor({1, c, hw, hw}), w1 = g1.tensor({f, c, 3, 3});
+    // H: [N,C,H/2,2,W] -> [(2,N),C,H/2,W]; then W likewise
+    auto th = g1.transpose(x1, 2, {{-1, 0}, 1, 2, 3}, 2);
+    auto tw = g1.transpose(th->getOutputs()[0], 3, {{-1, 0}, 1, 2, 3}, 2);
+    EXPECT(tw->getOutputs()[0]->getDims() == (Dim{4, c, hw / 2, hw / 2}));
+    auto cv = g1.conv(tw->getOutputs()[0], w1, 1, 1);
+    // inverse: batch (2, N') -> W interleave, then batch (2, N) -> H interleave
+    // (with factor -2 on dim 0 the flat dims are (2, N'), index 0 is the phase
+    // and -1 the remaining batch)
+    auto iw = g1.transpose(cv->getOutputs()[0], 0, {-1, 1, 2, {3, 0}}, -2);
+    auto ih = g1.transpose(iw->getOutputs()[0], 0, {-1, 1, {2, 0}, 3}, -2);
+    EXPECT(ih->getOutputs()[0]->getDims() == (Dim{1, f, hw, hw}));
+    g1.updateConnection();
+    SubGraph s0(g0.getOperators()), s1(g1.getOperators());
+    EXPECT(s0.verification(&s1, true));
+    return true;
+}
+
+// CodeEngine: the captured HIP graph reproduces SubGraph::compute, dim-0 split
+// and concat cost no kernel, and the emitted program names the same calls.
+static bool test_code_engine_graph_runtime() {
+    const int m = 16, n = 32, k = 8;
+    auto build = [&](Graph &g) {
+        auto a = g.tensor({1, m, k}), b0 = g.tensor({1, k, n}), b1 = g.tensor({1, k, n});
+        auto la = g.concat({a, a}, 0);
+        auto m0 = g.relu(b0), m1 = g.relu(b1); // producers inside the graph -> concat can alias
+        auto rb = g.concat({m0->getOutputs()[0], m1->getOutputs()[0]}, 0);
+        auto mm = g.matmul(la->getOutputs()[0], rb->getOutputs()[0]);
+        auto sp = g.split(mm->getOutputs()[0], 0, 2);
+        g.add({sp->getOutputs()[0], sp->getOutputs()[1]});
+        g.updateConnection();
+    };
+    Graph g;
+    build(g);
+    auto s1 = std::make_shared<SubGraph>(g.getOperators());
+    auto s2 = std::make_shared<SubGraph>(g.getOperators());
+    for (size_t i = 0; i < s1->getInputs().size(); ++i) {
+        s1->getInputs()[i]->dataRand((int)i + 5);
+        s2->getInputs()[i]->setData(s1->getInputs()[i]->getDataPtr());
+    }
+    EXPECT(s1->compute());
+    CodeEngine ce;
+    auto exec = ce.instantiate(s2);
+    EXPECT(exec != nullptr);
+    EXPECT(exec->numAliasedOps() == 2); // rhs concat and the split; lhs concat repeats `a`
+    for (int rep = 0; rep < 3; ++rep) {
+        EXPECT(exec->launch() && exec->sync());
+        Tensor *o1 = s1->getOutputs()[0], *o2 = s2->getOutputs()[0];
+        o2->deviceWritten();
+        EXPECT(equalArrays(o1->getDataPtr(), o2->getDataPtr(), o1->size()));
+    }
+    double ms = exec->time(5, 20);
+    EXPECT(std::isfinite(ms) && ms > 0.0);
+    std::string code = ce.genCode(s2);
+    EXPECT(code.find("pet_hip_bmm_f32(") != std::string::npos);
+    EXPECT(code.find("pet_hip_graph_begin_capture") != std::string::npos);
+    EXPECT(code.find("pet_hip_concat(") != std::string::npos); // the repeated-input concat
+    EXPECT(code.find("pet_hip_split(") == std::string::npos);  // aliased away
+    return true;
+}
+
+// Writes the emitted program of the config-1 transformed graph to argv[2]; the
+// python test compiles and runs it.
+static std::string g_emit_path;
+static bool test_emit_program() {
+    Graph g;
+    auto x = g.tensor({1, 16, 24, 20}), wt = g.tensor({16, 16, 3, 3});
+    auto pre = static_cast<TransposeOp *>(g.transpose(x, 2, {{0, 2}, 1, -1, 3}, -2));
+    pre->setType(TransposeOp::H2N);
+    pre->setPos(TransposeOp::Pre);
+    pre->setPaddingSize(1, 1);
+    pre->computeShape();
+    auto cv = static_cast<ConvOp *>(g.conv(pre->getOutputs()[0], wt, 1, 1));
+    cv->setAct(Operator::Relu);
+    auto post = static_cast<TransposeOp *>(g.transpose(cv->getOutputs()[0], 0, {0, 1, {-1, 2}, 3}, 2));
+    post->setType(TransposeOp::N2H);
+    post->setPos(TransposeOp::Post);
+    post->setPaddingSize(1, 1);
+    post->computeShape();
+    g.updateConnection();
+    auto sg = std::make_shared<SubGraph>(g.getOperators());
+    CodeEngine ce;
+    std::string path = g_emit_path.empty() ? "/tmp/pet_emitted.cpp" : g_emit_path;
+    EXPECT(ce.genCode(sg, path) == 0);
+    std::ifstream f(path);
+    std::string text((std::istreambuf_iterator<char>(f)), std::istreambuf_iterator<char>());
+    EXPECT(text.find("pet_hip_trans_chain(") != std::string::npos);
+    EXPECT(text.find("pet_hip_conv2d_f32(") != std::string::npos);
+    EXPECT(text.find("Time(ms)") != std::string::npos);
+    return true;
+}
+
+// Operator::perf: hipEvent timing, memoised per argument tuple.
+static bool test_perf_engine_memo() {
+    PerfEngine pe;
+    Tensor i0({1, 64, 28, 28}), w0({64, 64, 3, 3}), o0;
+    ConvOp conv(&i0, &w0, &o0, 1, 1);
+    double t1 = conv.perf(&pe, 20, 5);
+    EXPECT(std::isfinite(t1) && t1 > 0.0);
+    EXPECT(pe.checkOpPerf(Operator::Conv, conv.getArgs(pe.withPenalty())));
+    double t2 = conv.perf(&pe, 20, 5);
+    EXPECT(t1 == t2); // memo hit
+    // penalty rows change the key and the measured shape
+    i0.addPenalty(2, 1);
+    double t3 = conv.perf(&pe, 20, 5);
+    EXPECT(std::isfinite(t3) && std::get<2>(conv.getArgs(1)) == 29);
+    pe.setPenalty(0);
+    EXPECT(conv.perf(&pe, 20, 5) == t1);
+    Tensor a({3, 128, 768}), b({3, 768, 768}), c;
+    MatmulOp mm(&a, &b, &c);
+    double tm = mm.perf(&pe, 20, 5);
+    EXPECT(std::isfinite(tm) && tm > 0.0 && mm.perf(&pe, 20, 5) == tm);
+    // weight-side transposes are free, activation-side ones are timed
+    Tensor wt({64, 64, 3, 3}, Tensor::Weight), wtT;
+    TransposeOp tw(&wt, &wtT, -1, {0, 1, 3, 2});
+    EXPECT(tw.perf(&pe, 20, 5) == 0.0);
+    Tensor act({1, 64, 56, 56}), actT;
+    TransposeOp ta(&act, &actT, 2, {{0, 2}, 1, -1, 3}, -2);
+    double tt = ta.perf(&pe, 20, 5);
+    EXPECT(std::isfinite(tt) && tt > 0.0);
+    double bw = pe.layoutBandwidthGiBs();
+    EXPECT(bw > 100.0);
+    std::printf("  conv %.4f ms, conv+penalty %.4f ms, bmm %.4f ms, H2N %.4f ms, copy %.0f GiB/s\n",
+                t1, t3, tm, tt, bw);
+    return true;
+}
+
+// Split ratio rule and eltwise broadcast through the operator classes.
+static bool test_split_ratio_and_eltwise() {
+    Tensor x({2, 6, 4}), bias({4});
+    x.dataRand(1);
+    bias.dataRand(2);
+    SplitOp sp(&x, 1, std::vector<int>{1, 2});
+    EXPECT(sp.getOutputs()[0]->getDims() == (Dim{2, 2, 4}));
+    EXPECT(sp.getOutputs()[1]->getDims() == (Dim{2, 4, 4}));
+    EXPECT(!sp.computeV().empty());
+    EXPECT(sp.getOutputs()[1]->getData({1, 3, 2}) == x.getData({1, 5, 2}));
+    SplitOp bad(&x, 1, std::vector<int>{1, 3});
+    EXPECT(!bad.getOutputs()[0]->isValid());
+    EXPECT(bad.computeV().empty());
+    Tensor y;
+    AddOp add({&x, &bias}, &y);
+    EXPECT(add.compute() != nullptr);
+    for (size_t i = 0; i < x.size(); ++i)
+        EXPECT(y.getData(i) == x.getData(i) + bias.getData(i % 4));
+    for (auto t : sp.getOutputs())
+        delete t;
+    for (auto t : bad.getOutputs())
+        delete t;
+    return true;
+}
+
+int main(int argc, char **argv) {
+    std::vector<std::pair<std::string, std::function<bool()>>> cases = {
+        {"conv_vs_oracle", test_conv_vs_oracle},
+        {"conv_invalid_groups", test_conv_invalid_groups},
+        {"transpose_n2h_h2n", test_transpose_n2h_h2n},
+        {"batch_gemm_merge", test_batch_gemm_merge},
+        {"pad_conv_slice_verification", test_pad_conv_slice_verification},
+        {"corrected_h2n_program", test_corrected_h2n_program},
+        {"dilated_space_to_batch_program", test_dilated_space_to_batch_program},
+        {"code_engine_graph_runtime", test_code_engine_graph_runtime},
+        {"emit_program", test_emit_program},
+        {"perf_engine_memo", test_perf_engine_memo},
+        {"split_ratio_and_eltwise", test_split_ratio_and_eltwise},
+    };
+    std::string only = argc > 1 ? argv[1] : "";
+    if (argc > 2)
+        g_emit_path = argv[2];
+    if (!petInit()) {
+        std::printf("no gfx950 device: %s\n", pet_hip_last_error());
+        return 2;
+    }
+    int failed = 0, ran = 0;
+    for (auto &c : cases) {
+        if (!only.empty() && only != c.first)
+            continue;
+        std::printf("[ RUN ] %s\n", c.first.c_str());
+        std::fflush(stdout);
+        bool ok = c.second();
+        std::printf("[ %s ] %s\n", ok ? " OK " : "FAIL", c.first.c_str());
+        std::fflush(stdout);
+        failed += !ok;
+        ran++;
+    }
+    std::printf("%d run, %d failed\n", ran, failed);
+    return failed ? 1 : (ran ? 0 : 3);
+}
