@@ -31,6 +31,8 @@ struct ConvParams {
     int NPIX; // N * OT * OH * OW
     int OPIX; // OT * OH * OW
     int act;
+    int bias_mode; // 1: bias[f] per output channel, 2: bias[pixel] per output column
+    int splitk;    // plane kernel: K steps are dealt to this many workgroups per tile
     FastDiv fd_krs, fd_rs, fd_s;     // k -> (c, kt, r, s)
     FastDiv fd_opix, fd_ohw, fd_ow;  // pixel -> (n, ot, oh, ow)
     int tiles_n;                     // pixel tiles (for the workgroup swizzle)
@@ -326,7 +328,8 @@ __global__ __launch_bounds__(Cfg::NT) void conv_plane_kernel(ConvParams p) {
     const int wm0 = (wave / Cfg::WGN) * Cfg::WM;
     const int wn0 = (wave % Cfg::WGN) * Cfg::WN;
     const int l32 = lane & 31, hk = lane >> 5;
-    const int g = blockIdx.z;
+    const int g = blockIdx.z / p.splitk;
+    const int ks = blockIdx.z - g * p.splitk; // which share of the K steps
     const int m0 = blockIdx.y * Cfg::BM;
     const int n0 = blockIdx.x * Cfg::BN;
 
@@ -415,11 +418,14 @@ __global__ __launch_bounds__(Cfg::NT) void conv_plane_kernel(ConvParams p) {
 
     // step counters of the prefetch stream: channel block and kt slice
     const int ncb = p.cpg / CB;
-    const int nit = ncb * p.KT;
-    int pcb = 0, pq = 0;
+    const int nit_all = ncb * p.KT;
+    const int it_begin = (int)((long long)ks * nit_all / p.splitk);
+    const int it_end = (int)((long long)(ks + 1) * nit_all / p.splitk);
+    const int nit = it_end - it_begin;
+    int pcb = it_begin / p.KT, pq = it_begin - pcb * p.KT;
     auto advance_prefetch = [&]() __attribute__((always_inline)) {
         // stays on the last step once the end is reached (harmless re-load)
-        if (pcb * p.KT + pq + 1 < nit) {
+        if (pcb * p.KT + pq + 1 < it_end) {
             if (++pq == p.KT) {
                 pq = 0;
                 ++pcb;
@@ -559,7 +565,9 @@ __global__ __launch_bounds__(Cfg::NT) void conv_plane_kernel(ConvParams p) {
         unsigned n = fd_div(pix, p.fd_opix);
         unsigned rem = pix - n * p.OPIX;
         float *__restrict__ yb = p.y + (((long long)n * p.F + (long long)g * p.M) * p.OPIX + rem);
-        const float *__restrict__ bias = p.bias ? p.bias + g * p.M : nullptr;
+        const float *__restrict__ bias =
+            (p.bias && p.bias_mode == 1) ? p.bias + g * p.M : nullptr;
+        const float colbias = (p.bias && p.bias_mode == 2) ? p.bias[rem] : 0.f;
 #pragma unroll
         for (int tm = 0; tm < TM; ++tm) {
 #pragma unroll
@@ -567,9 +575,16 @@ __global__ __launch_bounds__(Cfg::NT) void conv_plane_kernel(ConvParams p) {
                 int f = m0 + wm0 + tm * 32 + (r / 4) * 8 + hk * 4 + (r % 4);
                 if (f < p.M) {
                     float v = acc[tm][tn][r];
-                    if (bias)
-                        v += bias[f];
-                    yb[(unsigned)f * (unsigned)p.OPIX] = apply_act(v, p.act);
+                    float *dst = yb + (unsigned)f * (unsigned)p.OPIX;
+                    if (p.splitk > 1) {
+                        // partial sum: the output was initialised with the bias
+                        // by the host; the activation runs afterwards
+                        unsafeAtomicAdd(dst, v);
+                    } else {
+                        if (bias)
+                            v += bias[f];
+                        *dst = apply_act(v + colbias, p.act);
+                    }
                 }
             }
         }
@@ -618,8 +633,27 @@ int pick_tile(int M, int N, int batch) {
     return 3;
 }
 
+// Output initialisation for split-K launches: y = bias (per channel or per
+// column) or 0; the partial sums are then added atomically.
+__global__ __launch_bounds__(256) void splitk_init_kernel(float *__restrict__ y,
+                                                          const float *__restrict__ bias,
+                                                          int bias_mode, unsigned F, unsigned OPIX,
+                                                          size_t total) {
+    size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+    const size_t step = (size_t)gridDim.x * 256;
+    for (; i < total; i += step) {
+        float v = 0.f;
+        if (bias) {
+            unsigned pix = (unsigned)(i % OPIX);
+            unsigned f = (unsigned)((i / OPIX) % F);
+            v = bias_mode == 2 ? bias[pix] : bias[f];
+        }
+        y[i] = v;
+    }
+}
+
 template <class Cfg, bool IS3D>
-int launch_plane_cfg(const ConvParams &p, hipStream_t stream) {
+int launch_plane_cfg(ConvParams p, hipStream_t stream) {
     const size_t lds_bytes = 2 * (size_t)Cfg::STAGE * sizeof(float);
     static int attr_status = [&] {
         hipError_t e = hipFuncSetAttribute(
@@ -629,9 +663,36 @@ int launch_plane_cfg(const ConvParams &p, hipStream_t stream) {
     }();
     if (attr_status)
         return -1; // caller falls back to the general kernel
-    dim3 grid((p.NPIX + Cfg::BN - 1) / Cfg::BN, (p.M + Cfg::BM - 1) / Cfg::BM, p.G);
+    const long long tiles = tiles_for(p.M, p.NPIX, Cfg::BM, Cfg::BN, p.G);
+    const int nit = (p.cpg / Cfg::CB) * p.KT;
+    // Split K when the tiles alone leave most CUs idle: each workgroup keeps at
+    // least two K steps, and about 256 workgroups are aimed for.
+    int splitk = 1;
+    if (tiles < 160 && nit >= 4) {
+        splitk = (int)std::min<long long>(nit / 2, (256 + tiles - 1) / tiles);
+        splitk = std::max(1, std::min(splitk, 64));
+    }
+    static const int forced = getenv("PET_HIP_SPLITK") ? atoi(getenv("PET_HIP_SPLITK")) : 0;
+    if (forced > 0)
+        splitk = std::min(forced, nit);
+    if ((long long)p.G * splitk > 65535)
+        splitk = 1;
+    p.splitk = splitk;
+    if (splitk > 1) {
+        const size_t total = (size_t)p.NPIX * p.F;
+        unsigned grid = (unsigned)std::min<size_t>((total + 255) / 256, 4096);
+        hipLaunchKernelGGL(splitk_init_kernel, dim3(grid), dim3(256), 0, stream, p.y, p.bias,
+                           p.bias_mode, (unsigned)p.F, (unsigned)p.OPIX, total);
+        int rc = check_launch("splitk_init_kernel");
+        if (rc)
+            return rc;
+    }
+    dim3 grid((p.NPIX + Cfg::BN - 1) / Cfg::BN, (p.M + Cfg::BM - 1) / Cfg::BM, p.G * splitk);
     hipLaunchKernelGGL((conv_plane_kernel<Cfg, IS3D>), grid, dim3(Cfg::NT), lds_bytes, stream, p);
-    return check_launch("conv_plane_kernel");
+    int rc = check_launch("conv_plane_kernel");
+    if (rc == PET_HIP_OK && splitk > 1 && p.act != PET_HIP_ACT_NONE)
+        rc = pet_hip_activation(p.y, p.y, (size_t)p.NPIX * p.F, p.act, (pet_hip_stream_t)stream);
+    return rc;
 }
 
 template <int RS, int CB>
@@ -639,10 +700,9 @@ int launch_plane(const ConvParams &p, bool is3d, hipStream_t stream) {
     using C64x128 = PlaneCfg<64, 128, 2, 2, RS, CB>;
     using C64x64 = PlaneCfg<64, 64, 2, 2, RS, CB>;
     using C32x64 = PlaneCfg<32, 64, 1, 2, RS, CB>;
-    // the largest tile that still hands (nearly) every CU a workgroup
-    int tile = 2;
-    if (p.M > 32 && tiles_for(p.M, p.NPIX, 64, 64, p.G) >= 200)
-        tile = 1;
+    // 64x128 when it alone fills the GPU; otherwise 64x64 (two workgroups fit a
+    // CU, and split-K supplies the missing parallelism); 32x64 for M <= 32
+    int tile = p.M > 32 ? 1 : 2;
     if (p.M > 32 && tiles_for(p.M, p.NPIX, 64, 128, p.G) >= 200)
         tile = 0;
     if (forced_tile() >= 0)
@@ -756,6 +816,8 @@ int conv_common(const float *x, const float *w, const float *bias, float *y, int
     p.NPIX = (int)npix;
     p.OPIX = (int)opix;
     p.act = act;
+    p.bias_mode = 1;
+    p.splitk = 1;
     p.fd_krs = make_fastdiv((unsigned)(kt * r * s));
     p.fd_rs = make_fastdiv((unsigned)(r * s));
     p.fd_s = make_fastdiv((unsigned)s);
@@ -768,6 +830,54 @@ int conv_common(const float *x, const float *w, const float *bias, float *y, int
 }
 
 } // namespace
+
+namespace pet {
+namespace mfma {
+
+// Batched row-major matmul without transposes is a grouped 1x1 convolution:
+// the batch is the group, B[b] ([k][n]) is that group's k-channel "image" of n
+// pixels, A[b] ([m][k]) its filters. Returns -1 when the plane kernel does not
+// apply (k not a multiple of 32, operands above 2 GiB, misaligned A).
+int bmm_as_grouped_1x1(const float *A, const float *B, float *C, const float *bias, int b, int m,
+                       int n, int k, int act, hipStream_t stream) {
+    if (k % 32 != 0 || b > 65535)
+        return -1;
+    ConvParams p;
+    memset(&p, 0, sizeof(p));
+    p.x = B;
+    p.w = A;
+    p.bias = bias;
+    p.y = C;
+    p.N = 1;
+    p.C = b * k;
+    p.T = 1;
+    p.H = 1;
+    p.W = n;
+    p.F = b * m;
+    p.KT = p.R = p.S = 1;
+    p.st = p.sh = p.sw = p.dt = p.dh = p.dw = 1;
+    p.G = b;
+    p.cpg = k;
+    p.OT = p.OH = 1;
+    p.OW = n;
+    p.M = m;
+    p.K = k;
+    p.NPIX = n;
+    p.OPIX = n;
+    p.act = act;
+    p.bias_mode = 2;
+    p.splitk = 1;
+    p.fd_krs = make_fastdiv(1);
+    p.fd_rs = make_fastdiv(1);
+    p.fd_s = make_fastdiv(1);
+    p.fd_opix = make_fastdiv((unsigned)n);
+    p.fd_ohw = make_fastdiv((unsigned)n);
+    p.fd_ow = make_fastdiv((unsigned)n);
+    return try_launch_plane(p, stream);
+}
+
+} // namespace mfma
+} // namespace pet
 
 extern "C" {
 

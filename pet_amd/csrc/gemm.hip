@@ -188,6 +188,11 @@ int pet_hip_bmm_f32(int transA, int transB, int b, int m, int n, int k, const fl
     p.sB = (long long)k * n;
     p.sC = (long long)m * n;
     p.act = act;
+    if (!transA && !transB) {
+        int rc = bmm_as_grouped_1x1(A, B, C, bias, b, m, n, k, act, as_stream(stream));
+        if (rc >= 0)
+            return rc;
+    }
     // float4 loads need every row start 16-byte aligned on both operands
     long long lda = transA ? m : k, ldb = transB ? k : n;
     bool vec = lda % 4 == 0 && ldb % 4 == 0 && p.sA % 4 == 0 && p.sB % 4 == 0 &&
