@@ -42,6 +42,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--cpu-seconds", type=float, default=15.0)
+    ap.add_argument("--no-configs", action="store_true",
+                    help="skip the latency table of the other four configurations")
     ap.add_argument("--dominant-only", type=int, default=0, metavar="N",
                     help="launch only the dominant kernel N times and exit (for rocprofv3)")
     args = ap.parse_args()
@@ -177,6 +179,42 @@ def main():
                    "GB/s": big_bytes / ms / 1e6, "frac_hbm": big_bytes / ms / 1e6 / HBM_PEAK_GBS})
     del big, big_out
 
+    # ---- the other configurations: batch-1 latency of the original network and of
+    # its PET-transformed program, each replayed as one HIP graph
+    other = {}
+    if not args.no_configs:
+        from pet_amd import programs
+        specs = [("c1_conv_56x56", programs.run_c1, programs.params_c1(0), 0.2312),
+                 ("c3_resnet18", programs.run_c3, programs.params_c3(0), 3.628),
+                 ("c4_bert_base_seq128", programs.run_c4, programs.params_c4(0), 22.347),
+                 ("c5_resnet3d18", programs.run_c5, programs.params_c5(0), 81.393)]
+        for name, run, params, gflop in specs:
+            entry = {"GFLOP": gflop}
+            for label, transformed in (("original_ms", False), ("pet_ms", True)):
+                try:
+                    ns = programs.GpuNS(keep=True)
+                    table = {}
+                    with torch.cuda.stream(stream):
+                        run(ns, params, transformed, T=table)  # uploads, weight-side ops
+                        stream.synchronize()
+                        ns.kept.clear()  # back to the allocator's pool for the captured run
+                        abi.call("pet_hip_graph_begin_capture", sp)
+                        try:
+                            run(ns, params, transformed, T=table)
+                        finally:
+                            gh = ctypes.c_void_p(0)
+                            abi.call("pet_hip_graph_end_capture", sp, ctypes.byref(gh))
+                    reps = max(10, args.steps // 10)
+                    entry[label] = time_graph(gh, reps, 3)
+                    abi.call("pet_hip_graph_destroy", gh)
+                    del ns, table
+                except Exception as exc:  # report, do not lose the main measurement
+                    entry[label] = None
+                    entry[label + "_error"] = str(exc)[:200]
+            if entry.get("pet_ms"):
+                entry["pet_TFLOP/s"] = gflop / entry["pet_ms"]
+            other[name] = entry
+
     dom_flop = conv_flop(DIL * DIL, 512, hs, hs, 512, 3, 3)
     dom_ms = conv_ms[0]
     achieved = dom_flop / dom_ms / 1e9
@@ -234,6 +272,7 @@ def main():
         "roofline": roofline,
         "cpu_baseline": cpu,
         "per_op": per_op,
+        "configs": other,
     }
     print(json.dumps(out))
 

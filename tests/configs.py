@@ -1,15 +1,11 @@
-"""The five benchmark configurations as programs over an operator namespace.
-
-Each ``run_*`` function is written once against a small namespace ``ns`` and is
-executed twice by the tests: with ``GpuNS`` (every call is one C-ABI call on
-device tensors) and with ``OracleNS`` (the CPU oracle on numpy arrays). The
-``transformed`` variants are the PET programs: the same network after the
-mutator's rewrites (src/Mutant/generator.cc, src/nnet/nmutator.cc).
-"""
+"""Test-side view of the configuration programs: everything from
+``pet_amd.programs`` plus ``OracleNS``, the same operator namespace on numpy
+arrays backed by the CPU oracle."""
 import numpy as np
 
+from pet_amd.programs import *  # noqa: F401,F403
+from pet_amd.programs import GpuNS  # noqa: F401
 
-# --------------------------------------------------------------------- namespaces
 
 class OracleNS:
     """numpy + CPU oracle."""
@@ -80,318 +76,3 @@ class OracleNS:
 
     def reshape(self, x, shape):
         return x.reshape(shape)
-
-
-class GpuNS:
-    """torch device tensors, every operator through the C ABI."""
-
-    def __init__(self):
-        import torch
-        from pet_amd import ops
-        self.t = torch
-        self.ops = ops
-
-    def tensor(self, a):
-        return self.t.from_numpy(np.ascontiguousarray(a, dtype=np.float32)).cuda()
-
-    def numpy(self, t):
-        self.t.cuda.synchronize()
-        return t.cpu().numpy()
-
-    def conv2d(self, x, w, ph, pw, sh=1, sw=1, dh=1, dw=1, bias=None, act="none"):
-        return self.ops.conv2d(x, w, ph, pw, sh, sw, dh, dw, bias=bias, act=act)
-
-    def conv3d(self, x, w, pad, stride=(1, 1, 1), dil=(1, 1, 1), bias=None, act="none"):
-        return self.ops.conv3d(x, w, pad, stride, dil, bias=bias, act=act)
-
-    def matmul(self, A, B, transA=False, transB=False, bias=None, act="none"):
-        return self.ops.matmul(A, B, transA, transB, bias=bias, act=act)
-
-    def permute_flat(self, x, flat, perm):
-        return self.ops.permute_flat(x, flat, perm)
-
-    def transpose(self, x, split, after, factor=2):
-        return self.ops.transpose(x, split, after, factor)
-
-    def trans_chain(self, x, chain):
-        return self.ops.trans_chain(x, chain)
-
-    def split(self, x, dim, sizes=None, num=None):
-        return self.ops.split(x, dim, sizes, num)
-
-    def concat(self, xs, dim):
-        return self.ops.concat(xs, dim)
-
-    def pad(self, x, b, e):
-        return self.ops.pad(x, b, e)
-
-    def slice(self, x, b, e):
-        return self.ops.slice_(x, b, e)
-
-    def extend(self, x, dim, num):
-        return self.ops.extend(x, dim, num)
-
-    def add(self, xs, shape=None):
-        return self.ops.eltwise("add", xs, shape or tuple(xs[0].shape))
-
-    def mul(self, xs, shape=None):
-        return self.ops.eltwise("mul", xs, shape or tuple(xs[0].shape))
-
-    def act(self, x, act):
-        return self.ops.activation(x, act)
-
-    def pool2d(self, x, kh, kw, ph, pw, sh, sw, mode="max"):
-        return self.ops.pool2d(x, kh, kw, ph, pw, sh, sw, mode=mode)
-
-    def softmax(self, x):
-        return self.ops.softmax(x)
-
-    def layernorm(self, x, g, b):
-        return self.ops.layernorm(x, g, b)
-
-    def reshape(self, x, shape):
-        return x.view(shape)
-
-
-# -------------------------------------------------------------- config 1: one conv
-
-def params_c1(seed=0, c=64, hw=56):
-    rng = np.random.default_rng(seed)
-    x = rng.uniform(-1, 1, (1, c, hw, hw)).astype(np.float32)
-    w = rng.uniform(-1, 1, (c, c, 3, 3)).astype(np.float32)
-    return {"x": x, "w": w}
-
-
-def run_c1(ns, p, transformed=False):
-    x, w = ns.tensor(p["x"]), ns.tensor(p["w"])
-    if not transformed:
-        return ns.conv2d(x, w, 1, 1)
-    half = p["x"].shape[2] // 2
-    xs = ns.trans_chain(x, [("split", 2, half, 0, 1), ("reorder", [0, 2, 1, 3, 4]),
-                            ("fuse", 0, 0, 0)])
-    y = ns.conv2d(xs, w, 1, 1)
-    return ns.trans_chain(y, [("split", 0, 2, 0, 0), ("reorder", [0, 2, 1, 3, 4]),
-                              ("fuse", 2, 0, 1)])
-
-
-# ------------------------------------------------- config 2: dilated conv block
-
-C2_CHANNELS = [512, 512, 512, 512, 256, 128, 64]
-
-
-def params_c2(seed=0, channels=None, hw=64):
-    ch = channels or C2_CHANNELS
-    rng = np.random.default_rng(seed)
-    x = rng.standard_normal((1, ch[0], hw, hw)).astype(np.float32)
-    ws = [(0.01 * rng.standard_normal((ch[i + 1], ch[i], 3, 3))).astype(np.float32)
-          for i in range(len(ch) - 1)]
-    return {"x": x, "ws": ws}
-
-
-def run_c2(ns, p, transformed=False, d=2):
-    x = ns.tensor(p["x"])
-    ws = [ns.tensor(w) for w in p["ws"]]
-    if not transformed:
-        for w in ws:
-            x = ns.conv2d(x, w, d, d, 1, 1, d, d, act="relu")
-        return x
-    _, c, h, wd = p["x"].shape
-    x = ns.reshape(ns.permute_flat(x, [1, c, h // d, d, wd // d, d], [3, 5, 0, 1, 2, 4]),
-                   (d * d, c, h // d, wd // d))
-    for w in ws:
-        x = ns.conv2d(x, w, 1, 1, act="relu")
-    f = p["ws"][-1].shape[0]
-    y = ns.permute_flat(x, [d, d, 1, f, h // d, wd // d], [2, 3, 4, 0, 5, 1])
-    return ns.reshape(y, (1, f, h, wd))
-
-
-# ------------------------------------------------------------ config 3: ResNet-18
-
-def _kaiming(rng, shape):
-    fan_in = int(np.prod(shape[1:]))
-    return (rng.standard_normal(shape) * np.sqrt(2.0 / fan_in)).astype(np.float32)
-
-
-def params_c3(seed=0, hw=224, width=64, classes=1000):
-    """Weights with BatchNorm already folded: every conv carries a bias."""
-    rng = np.random.default_rng(seed)
-    p = {"x": rng.standard_normal((1, 3, hw, hw)).astype(np.float32)}
-
-    def conv(name, f, c, k):
-        p[name + ".w"] = _kaiming(rng, (f, c, k, k))
-        p[name + ".b"] = (0.1 * rng.standard_normal(f)).astype(np.float32)
-
-    conv("stem", width, 3, 7)
-    cin = width
-    for li, mult in enumerate([1, 2, 4, 8]):
-        cout = width * mult
-        for bi in range(2):
-            pre = "l%d.b%d" % (li + 1, bi)
-            conv(pre + ".c1", cout, cin if bi == 0 else cout, 3)
-            conv(pre + ".c2", cout, cout, 3)
-            if bi == 0 and li > 0:
-                conv(pre + ".ds", cout, cin, 1)
-        cin = cout
-    p["fc.w"] = (rng.standard_normal((1, cin, classes)) / np.sqrt(cin)).astype(np.float32)
-    p["fc.b"] = (0.1 * rng.standard_normal(classes)).astype(np.float32)
-    return p
-
-
-def run_c3(ns, p, transformed=False):
-    T = {k: ns.tensor(v) for k, v in p.items()}
-    x = ns.conv2d(T["x"], T["stem.w"], 3, 3, 2, 2, bias=T["stem.b"], act="relu")
-    x = ns.pool2d(x, 3, 3, 1, 1, 2, 2, mode="max")
-    for li in range(4):
-        for bi in range(2):
-            pre = "l%d.b%d" % (li + 1, bi)
-            stride = 2 if (bi == 0 and li > 0) else 1
-            has_ds = (pre + ".ds.w") in p
-            if has_ds and transformed:
-                # PET merge of the two convs that read the same tensor
-                # (generator.cc:1236-1325, MAX variant): the 1x1/s2 filter is
-                # zero-padded to 3x3 (its tap at the centre equals 1x1 with pad 0),
-                # weights are concatenated on dim 0, one conv, split on dim 1.
-                w1 = p[pre + ".c1.w"]
-                wd = p[pre + ".ds.w"]
-                wpad = np.zeros((wd.shape[0], wd.shape[1], 3, 3), np.float32)
-                wpad[:, :, 1, 1] = wd[:, :, 0, 0]
-                wm = ns.concat([T[pre + ".c1.w"], ns.tensor(wpad)], 0)
-                bm = ns.concat([T[pre + ".c1.b"], T[pre + ".ds.b"]], 0)
-                ym = ns.conv2d(x, wm, 1, 1, stride, stride, bias=bm)
-                y, idn = ns.split(ym, 1, sizes=[w1.shape[0], wd.shape[0]])
-                y = ns.act(y, "relu")
-            else:
-                y = ns.conv2d(x, T[pre + ".c1.w"], 1, 1, stride, stride,
-                              bias=T[pre + ".c1.b"], act="relu")
-                idn = x
-                if has_ds:
-                    idn = ns.conv2d(x, T[pre + ".ds.w"], 0, 0, 2, 2, bias=T[pre + ".ds.b"])
-            y = ns.conv2d(y, T[pre + ".c2.w"], 1, 1, bias=T[pre + ".c2.b"])
-            x = ns.act(ns.add([y, idn]), "relu")
-    n, c, h, w = tuple(x.shape)
-    x = ns.pool2d(x, h, w, 0, 0, 1, 1, mode="avg")
-    x = ns.reshape(x, (1, 1, c))
-    return ns.matmul(x, T["fc.w"], bias=T["fc.b"])
-
-
-# -------------------------------------------------- config 4: BERT-base-shaped encoder
-
-def params_c4(seed=0, layers=12, seq=128, hidden=768, heads=12, ffn=3072):
-    rng = np.random.default_rng(seed)
-    p = {"x": rng.standard_normal((1, seq, hidden)).astype(np.float32),
-         "meta": (layers, seq, hidden, heads, ffn)}
-
-    def lin(name, k, n):
-        p[name + ".w"] = (0.02 * rng.standard_normal((1, k, n))).astype(np.float32)
-        p[name + ".b"] = (0.02 * rng.standard_normal(n)).astype(np.float32)
-
-    for l in range(layers):
-        for nm in ("q", "k", "v", "o"):
-            lin("L%d.%s" % (l, nm), hidden, hidden)
-        lin("L%d.f1" % l, hidden, ffn)
-        lin("L%d.f2" % l, ffn, hidden)
-        for nm in ("ln1", "ln2"):
-            p["L%d.%s.g" % (l, nm)] = (1 + 0.1 * rng.standard_normal(hidden)).astype(np.float32)
-            p["L%d.%s.b" % (l, nm)] = (0.1 * rng.standard_normal(hidden)).astype(np.float32)
-    return p
-
-
-def run_c4(ns, p, transformed=False):
-    layers, seq, hidden, heads, ffn = p["meta"]
-    dh = hidden // heads
-    T = {k: ns.tensor(v) for k, v in p.items() if k != "meta"}
-    scale = ns.tensor(np.array([1.0 / np.sqrt(dh)], np.float32))
-    x = T["x"]
-
-    def to_heads(t):  # [1, seq, hidden] -> [heads, seq, dh]
-        return ns.transpose(ns.reshape(t, (seq, hidden)), 1, [1, 0, -1], dh)
-
-    for l in range(layers):
-        pre = "L%d." % l
-        if transformed:
-            # PET batch-matmul merge (generator.cc:1495-1552): the three projections
-            # become one b=3 BatchMatmul; the lhs is repeated along dim 0, the
-            # weights are concatenated on dim 0, the result is split on dim 0.
-            xa = ns.extend(x, 0, 2)
-            wqkv = ns.concat([T[pre + "q.w"], T[pre + "k.w"], T[pre + "v.w"]], 0)
-            qkv = ns.matmul(xa, wqkv)
-            q, k, v = ns.split(qkv, 0, num=3)
-            q = ns.add([q, T[pre + "q.b"]])
-            k = ns.add([k, T[pre + "k.b"]])
-            v = ns.add([v, T[pre + "v.b"]])
-        else:
-            q = ns.matmul(x, T[pre + "q.w"], bias=T[pre + "q.b"])
-            k = ns.matmul(x, T[pre + "k.w"], bias=T[pre + "k.b"])
-            v = ns.matmul(x, T[pre + "v.w"], bias=T[pre + "v.b"])
-        qh, kh, vh = to_heads(q), to_heads(k), to_heads(v)
-        s = ns.matmul(qh, kh, transB=True)                 # [heads, seq, seq]
-        s = ns.softmax(ns.mul([s, scale]))
-        ctx = ns.matmul(s, vh)                             # [heads, seq, dh]
-        ctx = ns.reshape(ns.transpose(ctx, -1, [1, 0, 2]), (1, seq, hidden))
-        att = ns.matmul(ctx, T[pre + "o.w"], bias=T[pre + "o.b"])
-        x = ns.layernorm(ns.add([x, att]), T[pre + "ln1.g"], T[pre + "ln1.b"])
-        h = ns.matmul(x, T[pre + "f1.w"], bias=T[pre + "f1.b"], act="gelu")
-        h = ns.matmul(h, T[pre + "f2.w"], bias=T[pre + "f2.b"])
-        x = ns.layernorm(ns.add([x, h]), T[pre + "ln2.g"], T[pre + "ln2.b"])
-    return x
-
-
-# -------------------------------------------------------- config 5: ResNet3D-18
-
-def params_c5(seed=0, t=16, hw=112, width=64, classes=400):
-    rng = np.random.default_rng(seed)
-    p = {"x": rng.standard_normal((1, 3, t, hw, hw)).astype(np.float32)}
-
-    def conv(name, f, c, k):
-        fan_in = c * int(np.prod(k))
-        p[name + ".w"] = (rng.standard_normal((f, c) + tuple(k)) *
-                          np.sqrt(2.0 / fan_in)).astype(np.float32)
-        p[name + ".b"] = (0.1 * rng.standard_normal(f)).astype(np.float32)
-
-    conv("stem", width, 3, (3, 7, 7))
-    cin = width
-    for li, mult in enumerate([1, 2, 4, 8]):
-        cout = width * mult
-        for bi in range(2):
-            pre = "l%d.b%d" % (li + 1, bi)
-            conv(pre + ".c1", cout, cin if bi == 0 else cout, (3, 3, 3))
-            conv(pre + ".c2", cout, cout, (3, 3, 3))
-            if bi == 0 and li > 0:
-                conv(pre + ".ds", cout, cin, (1, 1, 1))
-        cin = cout
-    p["fc.w"] = (rng.standard_normal((1, cin, classes)) / np.sqrt(cin)).astype(np.float32)
-    p["fc.b"] = (0.1 * rng.standard_normal(classes)).astype(np.float32)
-    return p
-
-
-def run_c5(ns, p, transformed=False):
-    T = {k: ns.tensor(v) for k, v in p.items()}
-    x = ns.conv3d(T["x"], T["stem.w"], (1, 3, 3), (1, 2, 2), bias=T["stem.b"], act="relu")
-    for li in range(4):
-        for bi in range(2):
-            pre = "l%d.b%d" % (li + 1, bi)
-            st = (2, 2, 2) if (bi == 0 and li > 0) else (1, 1, 1)
-            y = ns.conv3d(x, T[pre + ".c1.w"], (1, 1, 1), st, bias=T[pre + ".c1.b"], act="relu")
-            idn = x
-            if (pre + ".ds.w") in p:
-                idn = ns.conv3d(x, T[pre + ".ds.w"], (0, 0, 0), (2, 2, 2), bias=T[pre + ".ds.b"])
-            if transformed and st == (1, 1, 1):
-                # T2N: the clip is cut in two along time with a one-frame halo, the two
-                # halves run as a batch of 2, and the seam frames are dropped afterwards
-                # (the 5-D form of the H2N / N2H correction).
-                tt = y.shape[2]
-                if tt % 2 == 0 and tt >= 4:
-                    ys = ns.trans_chain(y, [("split", 2, tt // 2, 0, 1),
-                                            ("reorder", [0, 2, 1, 3, 4, 5]), ("fuse", 0, 0, 0)])
-                    z = ns.conv3d(ys, T[pre + ".c2.w"], (1, 1, 1), bias=T[pre + ".c2.b"])
-                    y = ns.trans_chain(z, [("split", 0, 2, 0, 0),
-                                           ("reorder", [0, 2, 1, 3, 4, 5]), ("fuse", 2, 0, 1)])
-                else:
-                    y = ns.conv3d(y, T[pre + ".c2.w"], (1, 1, 1), bias=T[pre + ".c2.b"])
-            else:
-                y = ns.conv3d(y, T[pre + ".c2.w"], (1, 1, 1), bias=T[pre + ".c2.b"])
-            x = ns.act(ns.add([y, idn]), "relu")
-    n, c, t, h, w = tuple(x.shape)
-    x = ns.pool2d(ns.reshape(x, (1, c, t, h * w)), t, h * w, 0, 0, 1, 1, mode="avg")
-    x = ns.reshape(x, (1, 1, c))
-    return ns.matmul(x, T["fc.w"], bias=T["fc.b"])
