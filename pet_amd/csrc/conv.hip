@@ -33,6 +33,8 @@ struct ConvParams {
     int act;
     int bias_mode; // 1: bias[f] per output channel, 2: bias[pixel] per output column
     int splitk;    // plane kernel: K steps are dealt to this many workgroups per tile
+    float *ws;     // split-K: partial tiles, [tile][split][register][thread]
+    int *cnt;      // split-K: arrival counter per tile, zero between launches
     FastDiv fd_krs, fd_rs, fd_s;     // k -> (c, kt, r, s)
     FastDiv fd_opix, fd_ohw, fd_ow;  // pixel -> (n, ot, oh, ow)
     int tiles_n;                     // pixel tiles (for the workgroup swizzle)
@@ -556,6 +558,59 @@ __global__ __launch_bounds__(Cfg::NT) void conv_plane_kernel(ConvParams p) {
     if (kt < nit)
         step(std::integral_constant<int, 0>{});
 
+    // split-K: park the partial tile, and let the workgroup that arrives last add
+    // the S partials in a fixed order (the result does not depend on timing).
+    // Partials travel as device-scope relaxed atomic stores and loads, which go
+    // through to the level where all XCDs agree; the wait below keeps them ahead
+    // of the arrival count. Full device fences would also write back and
+    // invalidate everything else the L2s hold, which costs tens of microseconds.
+    if (p.splitk > 1) {
+        const int S = p.splitk;
+        const unsigned tile_id = (g * gridDim.y + blockIdx.y) * gridDim.x + blockIdx.x;
+        constexpr int NREG = TM * TN * 16;
+        float *mine = p.ws + ((size_t)tile_id * S + ks) * NREG * NT + tid;
+#pragma unroll
+        for (int tm = 0; tm < TM; ++tm)
+#pragma unroll
+            for (int tn = 0; tn < TN; ++tn)
+#pragma unroll
+                for (int r = 0; r < 16; ++r)
+                    __hip_atomic_store(mine + ((tm * TN + tn) * 16 + r) * NT, acc[tm][tn][r],
+                                       __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); // this lane's partials have landed
+        __syncthreads();                                 // ... and every lane's
+        int *flag = reinterpret_cast<int *>(lds);
+        if (tid == 0)
+            *flag = __hip_atomic_fetch_add(&p.cnt[tile_id], 1, __ATOMIC_RELAXED,
+                                           __HIP_MEMORY_SCOPE_AGENT) == S - 1;
+        __syncthreads();
+        if (!*flag)
+            return;
+        const float *all = p.ws + (size_t)tile_id * S * NREG * NT + tid;
+#pragma unroll
+        for (int tm = 0; tm < TM; ++tm)
+#pragma unroll
+            for (int tn = 0; tn < TN; ++tn)
+#pragma unroll
+                for (int r = 0; r < 16; ++r)
+                    acc[tm][tn][r] = 0.f;
+        for (int s2 = 0; s2 < S; ++s2) {
+            const float *part = all + (size_t)s2 * NREG * NT;
+#pragma unroll
+            for (int tm = 0; tm < TM; ++tm)
+#pragma unroll
+                for (int tn = 0; tn < TN; ++tn)
+#pragma unroll
+                    for (int r = 0; r < 16; ++r)
+                        acc[tm][tn][r] +=
+                            __hip_atomic_load(part + ((tm * TN + tn) * 16 + r) * NT,
+                                              __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+        if (tid == 0)
+            __hip_atomic_store(&p.cnt[tile_id], 0, __ATOMIC_RELAXED,
+                               __HIP_MEMORY_SCOPE_AGENT); // ready for the next launch
+    }
+
     // epilogue: bias + activation, NC(T)HW store
 #pragma unroll
     for (int tn = 0; tn < TN; ++tn) {
@@ -575,16 +630,9 @@ __global__ __launch_bounds__(Cfg::NT) void conv_plane_kernel(ConvParams p) {
                 int f = m0 + wm0 + tm * 32 + (r / 4) * 8 + hk * 4 + (r % 4);
                 if (f < p.M) {
                     float v = acc[tm][tn][r];
-                    float *dst = yb + (unsigned)f * (unsigned)p.OPIX;
-                    if (p.splitk > 1) {
-                        // partial sum: the output was initialised with the bias
-                        // by the host; the activation runs afterwards
-                        unsafeAtomicAdd(dst, v);
-                    } else {
-                        if (bias)
-                            v += bias[f];
-                        *dst = apply_act(v + colbias, p.act);
-                    }
+                    if (bias)
+                        v += bias[f];
+                    yb[(unsigned)f * (unsigned)p.OPIX] = apply_act(v + colbias, p.act);
                 }
             }
         }
@@ -633,25 +681,6 @@ int pick_tile(int M, int N, int batch) {
     return 3;
 }
 
-// Output initialisation for split-K launches: y = bias (per channel or per
-// column) or 0; the partial sums are then added atomically.
-__global__ __launch_bounds__(256) void splitk_init_kernel(float *__restrict__ y,
-                                                          const float *__restrict__ bias,
-                                                          int bias_mode, unsigned F, unsigned OPIX,
-                                                          size_t total) {
-    size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
-    const size_t step = (size_t)gridDim.x * 256;
-    for (; i < total; i += step) {
-        float v = 0.f;
-        if (bias) {
-            unsigned pix = (unsigned)(i % OPIX);
-            unsigned f = (unsigned)((i / OPIX) % F);
-            v = bias_mode == 2 ? bias[pix] : bias[f];
-        }
-        y[i] = v;
-    }
-}
-
 template <class Cfg, bool IS3D>
 int launch_plane_cfg(ConvParams p, hipStream_t stream) {
     const size_t lds_bytes = 2 * (size_t)Cfg::STAGE * sizeof(float);
@@ -677,22 +706,23 @@ int launch_plane_cfg(ConvParams p, hipStream_t stream) {
         splitk = std::min(forced, nit);
     if ((long long)p.G * splitk > 65535)
         splitk = 1;
-    p.splitk = splitk;
     if (splitk > 1) {
-        const size_t total = (size_t)p.NPIX * p.F;
-        unsigned grid = (unsigned)std::min<size_t>((total + 255) / 256, 4096);
-        hipLaunchKernelGGL(splitk_init_kernel, dim3(grid), dim3(256), 0, stream, p.y, p.bias,
-                           p.bias_mode, (unsigned)p.F, (unsigned)p.OPIX, total);
-        int rc = check_launch("splitk_init_kernel");
-        if (rc)
-            return rc;
+        // the partial tiles and arrival counters live in the library's scratch
+        size_t ws_elems;
+        int ncnt;
+        splitk_workspace(&p.ws, &ws_elems, &p.cnt, &ncnt);
+        const size_t per_split = (size_t)tiles * Cfg::BM * Cfg::BN;
+        if (tiles > ncnt || per_split == 0)
+            splitk = 1;
+        else
+            splitk = (int)std::min<size_t>(splitk, ws_elems / per_split);
+        if (splitk < 2)
+            splitk = 1;
     }
+    p.splitk = splitk;
     dim3 grid((p.NPIX + Cfg::BN - 1) / Cfg::BN, (p.M + Cfg::BM - 1) / Cfg::BM, p.G * splitk);
     hipLaunchKernelGGL((conv_plane_kernel<Cfg, IS3D>), grid, dim3(Cfg::NT), lds_bytes, stream, p);
-    int rc = check_launch("conv_plane_kernel");
-    if (rc == PET_HIP_OK && splitk > 1 && p.act != PET_HIP_ACT_NONE)
-        rc = pet_hip_activation(p.y, p.y, (size_t)p.NPIX * p.F, p.act, (pet_hip_stream_t)stream);
-    return rc;
+    return check_launch("conv_plane_kernel");
 }
 
 template <int RS, int CB>

@@ -23,6 +23,22 @@ int set_error(int status, const char *fmt, ...) {
 
 bool initialised() { return g_init.load(); }
 
+// Library-owned scratch for split-K contractions: partial tiles and one arrival
+// counter per output tile. Allocated once in pet_hip_init (the reference's
+// PerfEngine likewise owns its cuDNN workspace, src/Graph/perf_engine.cc:31-42).
+// Launches that use it must not overlap on different streams.
+static float *g_ws = nullptr;
+static int *g_cnt = nullptr;
+constexpr size_t kWsElems = (size_t)16 << 20; // 64 MiB of floats
+constexpr int kNumCounters = 16384;
+
+void splitk_workspace(float **ws, size_t *ws_elems, int **counters, int *num_counters) {
+    *ws = g_ws;
+    *ws_elems = g_ws ? kWsElems : 0;
+    *counters = g_cnt;
+    *num_counters = g_cnt ? kNumCounters : 0;
+}
+
 __global__ void fill_kernel(float *dst, float v, size_t n) {
     size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
     size_t stride = (size_t)gridDim.x * blockDim.x;
@@ -74,6 +90,12 @@ int pet_hip_init(int device) {
         return set_error(PET_HIP_ERR_UNSUPPORTED,
                          "this library is built for gfx950 only, device is %s",
                          prop.gcnArchName);
+    if (!g_ws) {
+        PET_HIP_CHECK(hipMalloc((void **)&g_ws, kWsElems * sizeof(float)));
+        PET_HIP_CHECK(hipMalloc((void **)&g_cnt, kNumCounters * sizeof(int)));
+        PET_HIP_CHECK(hipMemset(g_cnt, 0, kNumCounters * sizeof(int)));
+        PET_HIP_CHECK(hipDeviceSynchronize());
+    }
     g_device = device;
     g_init.store(true);
     err_buf()[0] = 0;
@@ -84,6 +106,12 @@ int pet_hip_shutdown(void) {
     if (!g_init.load())
         return PET_HIP_OK;
     PET_HIP_CHECK(hipDeviceSynchronize());
+    if (g_ws) {
+        PET_HIP_CHECK(hipFree(g_ws));
+        PET_HIP_CHECK(hipFree(g_cnt));
+        g_ws = nullptr;
+        g_cnt = nullptr;
+    }
     g_init.store(false);
     return PET_HIP_OK;
 }
