@@ -35,6 +35,14 @@ def conv_flop(n, f, oh, ow, c, r, s):
     return 2.0 * n * f * oh * ow * c * r * s
 
 
+# HBM-side bytes one launch of the dominant kernel moves, from rocprofv3 --pmc runs of
+# `bench.py --dominant-only 20`: FETCH_SIZE 25974.0 KiB per dispatch scaled by 1.9986
+# (what a 256 MiB plain copy reads on that counter), WRITE_SIZE 8192.0 KiB scaled by 1.0.
+# A counter cannot be read from inside this process; the summary is
+# profiles/conv_plane_64x128_rs9_c2_layer_512to512.txt.
+DOMINANT_TRAFFIC_BYTES = int((25974.0 * 1.9986 + 8192.0) * 1024)
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -95,6 +103,11 @@ def main():
 
     if args.dominant_only:
         # profiling aid: the 512->512 layer of the optimised program, nothing else
+        # plus one plain copy of 256 MiB (a pad by zero) that calibrates the
+        # FETCH_SIZE / WRITE_SIZE counters
+        cal = torch.zeros((64, 1024, 1024), device=dev)
+        cal_out = torch.empty_like(cal)
+        ops.pad(cal, [0, 0, 0], [0, 0, 0], out=cal_out)
         ops.permute_flat(x, s2b_flat, s2b_perm, out=t_s2b)
         for _ in range(args.dominant_only):
             ops.conv2d(t_s2b, ws[0], 1, 1, act="relu", out=t_act[0])
@@ -220,7 +233,8 @@ def main():
     achieved = dom_flop / dom_ms / 1e9
     roofline = {"bound": "mfma", "kernel": "conv_plane_kernel<64x128, RS=9, CB=8> (512->512, 4x32x32, 3x3, ReLU)",
                 "achieved": achieved, "peak": MFMA_FP32_PEAK_TFLOPS, "unit": "TFLOP/s",
-                "frac": achieved / MFMA_FP32_PEAK_TFLOPS, "traffic": None,
+                "frac": achieved / MFMA_FP32_PEAK_TFLOPS,
+                "traffic": DOMINANT_TRAFFIC_BYTES, "traffic_unit": "bytes per launch",
                 "flop_per_launch": dom_flop, "avg_launch_ms": dom_ms}
 
     total_flop = sum(conv_flop(1, CHANNELS[i + 1], HW, HW, CHANNELS[i], 3, 3) for i in range(6))

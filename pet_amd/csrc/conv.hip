@@ -33,6 +33,8 @@ struct ConvParams {
     int act;
     int bias_mode; // 1: bias[f] per output channel, 2: bias[pixel] per output column
     int splitk;    // plane kernel: K steps are dealt to this many workgroups per tile
+    int xcd_chunk; // plane kernel: tiles per XCD when the tile grid is dealt in bands (0: off)
+    int xcd_mg;    // ... and how many M tiles wide a band is
     float *ws;     // split-K: partial tiles, [tile][split][register][thread]
     int *cnt;      // split-K: arrival counter per tile, zero between launches
     FastDiv fd_krs, fd_rs, fd_s;     // k -> (c, kt, r, s)
@@ -332,8 +334,22 @@ __global__ __launch_bounds__(Cfg::NT) void conv_plane_kernel(ConvParams p) {
     const int l32 = lane & 31, hk = lane >> 5;
     const int g = blockIdx.z / p.splitk;
     const int ks = blockIdx.z - g * p.splitk; // which share of the K steps
-    const int m0 = blockIdx.y * Cfg::BM;
-    const int n0 = blockIdx.x * Cfg::BN;
+    // Workgroups are handed to the 8 XCDs round-robin in launch order, and each
+    // XCD has its own L2. Renumber so that an XCD owns one compact band of tiles
+    // (xcd_mg M tiles wide) instead of every eighth tile: its L2 then holds
+    // 1/8th of the operands rather than all the filters.
+    unsigned bx = blockIdx.x, by = blockIdx.y;
+    if (p.xcd_chunk) {
+        const unsigned L = bx + gridDim.x * by;
+        const unsigned Lp = (L & 7) * p.xcd_chunk + (L >> 3);
+        const unsigned mg = p.xcd_mg;
+        const unsigned band = Lp / (mg * gridDim.x);
+        const unsigned in_band = Lp - band * mg * gridDim.x;
+        by = band * mg + in_band % mg;
+        bx = in_band / mg;
+    }
+    const int m0 = by * Cfg::BM;
+    const int n0 = bx * Cfg::BN;
 
     const int THW = p.T * p.H * p.W, HW = p.H * p.W;
     const int KRS = p.KT * RS; // weights per (f, c)
@@ -566,7 +582,7 @@ __global__ __launch_bounds__(Cfg::NT) void conv_plane_kernel(ConvParams p) {
     // invalidate everything else the L2s hold, which costs tens of microseconds.
     if (p.splitk > 1) {
         const int S = p.splitk;
-        const unsigned tile_id = (g * gridDim.y + blockIdx.y) * gridDim.x + blockIdx.x;
+        const unsigned tile_id = (g * gridDim.y + by) * gridDim.x + bx;
         constexpr int NREG = TM * TN * 16;
         float *mine = p.ws + ((size_t)tile_id * S + ks) * NREG * NT + tid;
 #pragma unroll
@@ -721,6 +737,27 @@ int launch_plane_cfg(ConvParams p, hipStream_t stream) {
     }
     p.splitk = splitk;
     dim3 grid((p.NPIX + Cfg::BN - 1) / Cfg::BN, (p.M + Cfg::BM - 1) / Cfg::BM, p.G * splitk);
+    // XCD bands: only when every z plane starts on XCD 0 and has several tiles per XCD
+    p.xcd_chunk = 0;
+    p.xcd_mg = 1;
+    static const bool xcd_off = getenv("PET_HIP_XCD") && atoi(getenv("PET_HIP_XCD")) == 0;
+    const unsigned plane_tiles = grid.x * grid.y;
+    if (!xcd_off && plane_tiles % 8 == 0 && plane_tiles >= 64) {
+        const unsigned chunk = plane_tiles / 8;
+        // bytes an XCD pulls for a band mg tiles wide: its filters + its pixels
+        double best = 0;
+        for (unsigned mg = 1; mg <= grid.y; mg *= 2) {
+            if (grid.y % mg || chunk % mg)
+                continue;
+            const double cost = (double)mg * Cfg::BM * p.K +
+                                (double)(chunk / mg) * Cfg::BN * p.cpg * p.st * p.sh * p.sw;
+            if (best == 0 || cost < best) {
+                best = cost;
+                p.xcd_mg = (int)mg;
+            }
+        }
+        p.xcd_chunk = (int)chunk;
+    }
     hipLaunchKernelGGL((conv_plane_kernel<Cfg, IS3D>), grid, dim3(Cfg::NT), lds_bytes, stream, p);
     return check_launch("conv_plane_kernel");
 }
