@@ -3,6 +3,8 @@
 #include "view.h"
 
 #include <algorithm>
+#include <cstdlib>
+#include <cstring>
 #include <vector>
 
 namespace pet {
@@ -46,19 +48,43 @@ struct DirectParams {
     unsigned total; // number of work items (elements / VEC)
 };
 
+typedef float vf4 __attribute__((ext_vector_type(4)));
+
+// Streaming (non-temporal) accesses for tensors too large to stay in cache.
+template <bool NT>
+__device__ __forceinline__ vf4 ld4(const float *p) {
+    const vf4 *q = reinterpret_cast<const vf4 *>(p);
+    return NT ? __builtin_nontemporal_load(q) : *q;
+}
+template <bool NT>
+__device__ __forceinline__ void st4(float *p, vf4 v) {
+    vf4 *q = reinterpret_cast<vf4 *>(p);
+    if (NT)
+        __builtin_nontemporal_store(v, q);
+    else
+        *q = v;
+}
+
 // One work item = VEC consecutive elements of the innermost iteration dim.
 // With VEC == 4 the host has checked that the four elements are contiguous and
-// 16-byte aligned on both sides and share one validity result.
-template <int VEC>
+// 16-byte aligned on both sides and share one validity result. A thread takes
+// UN items 256 apart and issues all its loads before its stores, so UN 16-byte
+// requests per lane are in flight.
+template <int VEC, int UN, bool NT>
 __global__ __launch_bounds__(256) void view_direct_kernel(const float *__restrict__ x,
                                                           float *__restrict__ y,
                                                           DirectParams p) {
-    unsigned t = blockIdx.x * 256u + threadIdx.x;
-    const unsigned step = gridDim.x * 256u;
-    for (; t < p.total; t += step) {
-        unsigned rem = t;
-        long long io = p.ibase, oo = p.obase;
-        bool ok = true;
+    const unsigned base = blockIdx.x * (256u * UN) + threadIdx.x;
+    long long io[UN], oo[UN];
+    bool ok[UN], live[UN];
+#pragma unroll
+    for (int u = 0; u < UN; ++u) {
+        const unsigned t = base + u * 256u;
+        live[u] = t < p.total;
+        unsigned rem = live[u] ? t : 0u;
+        io[u] = p.ibase;
+        oo[u] = p.obase;
+        ok[u] = live[u];
 #pragma unroll
         for (int d = PET_HIP_MAX_RANK - 1; d >= 0; --d) {
             if (d < p.rank) {
@@ -67,25 +93,230 @@ __global__ __launch_bounds__(256) void view_direct_kernel(const float *__restric
                 rem = q;
                 if (d == p.rank - 1)
                     idx *= VEC;
-                oo += (long long)idx * p.os[d];
+                oo[u] += (long long)idx * p.os[d];
                 unsigned r = idx;
                 if (p.has_div[d]) {
                     unsigned qq = fd_div(idx, p.m[d]);
                     r = idx - qq * p.m[d].d;
-                    io += (long long)qq * p.sq[d];
+                    io[u] += (long long)qq * p.sq[d];
                 }
-                io += (long long)r * p.sr[d];
-                ok = ok && ((int)r >= p.lo[d]) && ((int)r < p.hi[d]);
+                io[u] += (long long)r * p.sr[d];
+                ok[u] = ok[u] && ((int)r >= p.lo[d]) && ((int)r < p.hi[d]);
             }
         }
-        if (VEC == 4) {
-            float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
-            if (ok)
-                v = *reinterpret_cast<const float4 *>(x + io);
-            *reinterpret_cast<float4 *>(y + oo) = v;
-        } else {
-            y[oo] = ok ? x[io] : 0.f;
+    }
+    if (VEC == 4) {
+        vf4 v[UN];
+#pragma unroll
+        for (int u = 0; u < UN; ++u) {
+            v[u] = (vf4){0.f, 0.f, 0.f, 0.f};
+            if (ok[u])
+                v[u] = ld4<NT>(x + io[u]);
         }
+#pragma unroll
+        for (int u = 0; u < UN; ++u)
+            if (live[u])
+                st4<NT>(y + oo[u], v[u]);
+    } else {
+        float v[UN];
+#pragma unroll
+        for (int u = 0; u < UN; ++u)
+            v[u] = ok[u] ? x[io[u]] : 0.f;
+#pragma unroll
+        for (int u = 0; u < UN; ++u)
+            if (live[u])
+                y[oo[u]] = v[u];
+    }
+}
+
+// Index of one element of the iteration space -> input offset and validity.
+// 32-bit wrap-around arithmetic: both buffers hold fewer than 2^31 elements, so
+// the offset of every valid element is exact modulo 2^32.
+__device__ __forceinline__ void decode_in(const DirectParams &p, unsigned e, unsigned &io,
+                                          bool &ok) {
+    io = (unsigned)p.ibase;
+#pragma unroll
+    for (int d = PET_HIP_MAX_RANK - 1; d >= 0; --d) {
+        if (d < p.rank) {
+            unsigned q = fd_div(e, p.ext[d]);
+            unsigned r = e - q * p.ext[d].d;
+            e = q;
+            if (p.has_div[d]) {
+                unsigned qq = fd_div(r, p.m[d]);
+                r -= qq * p.m[d].d;
+                io += qq * (unsigned)p.sq[d];
+            }
+            io += r * (unsigned)p.sr[d];
+            ok = ok && ((int)r >= p.lo[d]) && ((int)r < p.hi[d]);
+        }
+    }
+}
+
+// Dense, 16-byte aligned output but an input side that cannot be vectorised (an
+// innermost extent that is not a multiple of 4, a window that cuts through
+// it): a thread gathers 4 consecutive output elements one by one and stores
+// them as one 16-byte word. p.total counts the 4-element groups; the output
+// offset of group t is obase + 4t.
+template <bool NT>
+__global__ __launch_bounds__(256) void view_gather4_kernel(const float *__restrict__ x,
+                                                           float *__restrict__ y,
+                                                           DirectParams p) {
+    constexpr int UN = 2;
+    const unsigned base = blockIdx.x * (256u * UN) + threadIdx.x;
+    float v[UN][4];
+#pragma unroll
+    for (int u = 0; u < UN; ++u) {
+        const unsigned t = base + u * 256u;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            unsigned io;
+            bool ok = t < p.total;
+            decode_in(p, ok ? t * 4u + j : 0u, io, ok);
+            v[u][j] = 0.f;
+            if (ok)
+                v[u][j] = NT ? __builtin_nontemporal_load(x + io) : x[io];
+        }
+    }
+#pragma unroll
+    for (int u = 0; u < UN; ++u) {
+        const unsigned t = base + u * 256u;
+        if (t < p.total)
+            st4<NT>(y + p.obase + 4ll * t, (vf4){v[u][0], v[u][1], v[u][2], v[u][3]});
+    }
+}
+
+// Interleave kernels for the space-to-batch family: a dim of extent E (2 or 4)
+// that is innermost on one side sits next to the dim that is innermost on the
+// other side. Each thread moves a 4 x E block through registers, with 16-byte
+// accesses on both sides and no LDS.
+struct InterleaveParams {
+    DirectParams dp;   // the iteration space without the E dim; innermost dim in units of 4
+    long long e_stride; // stride of the E dim on the side where it is not innermost
+};
+
+// DEINT: input holds (w, e) pairs with e innermost; output has w innermost and
+// e far away (space-to-batch). Otherwise the reverse (batch-to-space).
+template <int E, bool DEINT, bool NT>
+__global__ __launch_bounds__(256) void view_interleave_kernel(const float *__restrict__ x,
+                                                              float *__restrict__ y,
+                                                              InterleaveParams ip) {
+    const DirectParams &p = ip.dp;
+    constexpr int UN = 1;
+    const unsigned base = blockIdx.x * (256u * UN) + threadIdx.x;
+    unsigned io[UN], oo[UN];
+    bool live[UN];
+    vf4 a[UN][E];
+#pragma unroll
+    for (int u = 0; u < UN; ++u) {
+        const unsigned t = base + u * 256u;
+        live[u] = t < p.total;
+        unsigned rem = live[u] ? t : 0u;
+        io[u] = (unsigned)p.ibase;
+        oo[u] = (unsigned)p.obase;
+#pragma unroll
+        for (int d = PET_HIP_MAX_RANK - 1; d >= 0; --d) {
+            if (d < p.rank) {
+                unsigned q = fd_div(rem, p.ext[d]);
+                unsigned idx = rem - q * p.ext[d].d;
+                rem = q;
+                if (d == p.rank - 1)
+                    idx *= 4;
+                oo[u] += idx * (unsigned)p.os[d];
+                io[u] += idx * (unsigned)p.sr[d];
+            }
+        }
+        if (live[u]) {
+#pragma unroll
+            for (int e = 0; e < E; ++e)
+                a[u][e] = ld4<NT>(x + io[u] + (DEINT ? 4u * e : (unsigned)ip.e_stride * e));
+        }
+    }
+#pragma unroll
+    for (int u = 0; u < UN; ++u) {
+        if (!live[u])
+            continue;
+        float m[4 * E];
+#pragma unroll
+        for (int e = 0; e < E; ++e) {
+            m[4 * e + 0] = a[u][e].x;
+            m[4 * e + 1] = a[u][e].y;
+            m[4 * e + 2] = a[u][e].z;
+            m[4 * e + 3] = a[u][e].w;
+        }
+#pragma unroll
+        for (int e = 0; e < E; ++e) {
+            vf4 o;
+            if (DEINT) // m is [w][e]: pick plane e
+                o = (vf4){m[0 * E + e], m[1 * E + e], m[2 * E + e], m[3 * E + e]};
+            else       // m is [e][w]: output word e holds flat positions 4e .. 4e+3 of [w][e]
+                o = (vf4){m[((4 * e + 0) % E) * 4 + (4 * e + 0) / E],
+                          m[((4 * e + 1) % E) * 4 + (4 * e + 1) / E],
+                          m[((4 * e + 2) % E) * 4 + (4 * e + 2) / E],
+                          m[((4 * e + 3) % E) * 4 + (4 * e + 3) / E]};
+            st4<NT>(y + oo[u] + (DEINT ? (unsigned)ip.e_stride * e : 4u * e), o);
+        }
+    }
+}
+
+// The 2-wide case moves whole cache lines on both sides: a lane handles one
+// 16-byte word of the interleaved side and, with its neighbour (lane ^ 1),
+// one word of each of the two planes; the pair swaps two floats each through a
+// lane shuffle. p's last dim counts the interleaved row in 16-byte words.
+template <bool DEINT, bool NT>
+__global__ __launch_bounds__(256) void view_interleave2_kernel(const float *__restrict__ x,
+                                                               float *__restrict__ y,
+                                                               InterleaveParams ip) {
+    const DirectParams &p = ip.dp;
+    constexpr int UN = 4;
+    const unsigned base = blockIdx.x * (256u * UN) + threadIdx.x;
+    const bool odd = threadIdx.x & 1;
+    unsigned io[UN], oo[UN];
+    bool live[UN];
+    vf4 a[UN];
+#pragma unroll
+    for (int u = 0; u < UN; ++u) {
+        const unsigned t = base + u * 256u;
+        live[u] = t < p.total; // the same for both lanes of a pair: total is even
+        unsigned rem = live[u] ? t : 0u;
+        io[u] = (unsigned)p.ibase;
+        oo[u] = (unsigned)p.obase;
+#pragma unroll
+        for (int d = PET_HIP_MAX_RANK - 1; d >= 0; --d) {
+            if (d < p.rank) {
+                unsigned q = fd_div(rem, p.ext[d]);
+                unsigned idx = rem - q * p.ext[d].d;
+                rem = q;
+                if (d == p.rank - 1) {
+                    // word idx of the interleaved row <-> word idx/2 of plane idx%2
+                    const unsigned planar = 4u * (idx >> 1) + (idx & 1) * (unsigned)ip.e_stride;
+                    io[u] += DEINT ? 4u * idx : planar;
+                    oo[u] += DEINT ? planar : 4u * idx;
+                } else {
+                    oo[u] += idx * (unsigned)p.os[d];
+                    io[u] += idx * (unsigned)p.sr[d];
+                }
+            }
+        }
+        a[u] = (vf4){0.f, 0.f, 0.f, 0.f};
+        if (live[u])
+            a[u] = ld4<NT>(x + io[u]);
+    }
+#pragma unroll
+    for (int u = 0; u < UN; ++u) {
+        const vf4 v = a[u];
+        vf4 o;
+        if (DEINT) {
+            // even lane keeps plane 0 (x, z) and wants the neighbour's; odd likewise for plane 1
+            const float r0 = __shfl_xor(odd ? v.x : v.y, 1);
+            const float r1 = __shfl_xor(odd ? v.z : v.w, 1);
+            o = odd ? (vf4){r0, r1, v.y, v.w} : (vf4){v.x, v.z, r0, r1};
+        } else {
+            const float r0 = __shfl_xor(odd ? v.x : v.z, 1);
+            const float r1 = __shfl_xor(odd ? v.y : v.w, 1);
+            o = odd ? (vf4){r0, v.z, r1, v.w} : (vf4){v.x, r0, v.y, r1};
+        }
+        if (live[u])
+            st4<NT>(y + oo[u], o);
     }
 }
 
@@ -94,7 +325,6 @@ __global__ __launch_bounds__(256) void view_direct_kernel(const float *__restric
 // "input order" (tile dims sorted by input stride, so consecutive lanes read
 // consecutive addresses), parked in LDS, and written in "output order" (sorted
 // by output stride). Dims outside the tile are handled by the grid.
-constexpr int kTileMax = 4096;
 constexpr int kTileDims = 4;
 
 struct TiledParams {
@@ -121,10 +351,15 @@ struct TiledParams {
     int tile_elems;
 };
 
+// VIN / VOUT: the host has checked that four consecutive elements in input
+// (output) order are contiguous, 16-byte aligned and valid together, so the
+// global side moves 16 bytes per lane. Loads of a pass are all issued before the
+// LDS writes (four requests per lane in flight).
+template <bool VIN, bool VOUT, bool NT>
 __global__ __launch_bounds__(256) void view_tiled_kernel(const float *__restrict__ x,
                                                          float *__restrict__ y,
                                                          TiledParams p) {
-    __shared__ float lds[kTileMax + kTileMax / 32];
+    extern __shared__ float lds[]; // tile_elems * 33 / 32 floats
     const unsigned wg = blockIdx.x;
     long long ibase = p.ibase, obase = p.obase;
     bool wg_ok = true;
@@ -155,47 +390,107 @@ __global__ __launch_bounds__(256) void view_tiled_kernel(const float *__restrict
             org_out[i] = (int)((q - fd_div(q, p.out_nt[i]) * p.out_nt[i].d) << p.out_shift[i]);
         }
     }
+    constexpr int UN = 4;
     // load phase: consecutive lanes walk the tile in input order
-    for (int t = threadIdx.x; t < p.tile_elems; t += 256) {
-        int remt = t;
-        long long io = ibase;
-        bool ok = wg_ok;
+    {
+        constexpr int W = VIN ? 4 : 1;
+        const int items = p.tile_elems / W;
+        for (int b = 0; b < items; b += 256 * UN) {
+            vf4 v[UN];
 #pragma unroll
-        for (int i = 0; i < kTileDims; ++i) {
-            if (i < p.ntd) {
-                int c = remt & ((1 << p.in_shift[i]) - 1);
-                remt >>= p.in_shift[i];
-                int idx = org_in[i] + c;
-                ok = ok && idx < p.in_ext[i];
-                io += (long long)idx * p.in_sr[i];
+            for (int u = 0; u < UN; ++u) {
+                const int t = b + u * 256 + (int)threadIdx.x;
+                int remt = t * W;
+                long long io = ibase;
+                bool ok = wg_ok && t < items;
+#pragma unroll
+                for (int i = 0; i < kTileDims; ++i) {
+                    if (i < p.ntd) {
+                        int c = remt & ((1 << p.in_shift[i]) - 1);
+                        remt >>= p.in_shift[i];
+                        int idx = org_in[i] + c;
+                        ok = ok && idx < p.in_ext[i];
+                        io += (long long)idx * p.in_sr[i];
+                    }
+                }
+                v[u] = (vf4){0.f, 0.f, 0.f, 0.f};
+                if (ok) {
+                    if (VIN)
+                        v[u] = ld4<NT>(x + io);
+                    else
+                        v[u].x = NT ? __builtin_nontemporal_load(x + io) : x[io];
+                }
+            }
+#pragma unroll
+            for (int u = 0; u < UN; ++u) {
+                const int t = b + u * 256 + (int)threadIdx.x;
+                if (t < items) {
+                    if (VIN) {
+                        const int e = t * 4, pad = e >> 5; // 4 | 32: one pad for all four
+                        lds[e + pad] = v[u].x;
+                        lds[e + 1 + pad] = v[u].y;
+                        lds[e + 2 + pad] = v[u].z;
+                        lds[e + 3 + pad] = v[u].w;
+                    } else {
+                        lds[t + (t >> 5)] = v[u].x;
+                    }
+                }
             }
         }
-        float v = 0.f;
-        if (ok)
-            v = x[io];
-        lds[t + (t >> 5)] = v;
     }
     __syncthreads();
     // store phase: consecutive lanes walk the tile in output order
-    for (int t = threadIdx.x; t < p.tile_elems; t += 256) {
-        int remt = t;
-        long long oo = obase;
-        int lin = 0;
-        bool ok = true;
+    {
+        constexpr int W = VOUT ? 4 : 1;
+        const int items = p.tile_elems / W;
+        for (int t = threadIdx.x; t < items; t += 256) {
+            int remt = t * W;
+            long long oo = obase;
+            bool ok = true;
 #pragma unroll
-        for (int i = 0; i < kTileDims; ++i) {
-            if (i < p.ntd) {
-                int c = remt & ((1 << p.out_shift[i]) - 1);
-                remt >>= p.out_shift[i];
-                int idx = org_out[i] + c;
-                ok = ok && idx < p.out_ext[i];
-                oo += (long long)idx * p.out_os[i];
-                lin += c << p.out_to_in_pos[i];
+            for (int i = 0; i < kTileDims; ++i) {
+                if (i < p.ntd) {
+                    int c = remt & ((1 << p.out_shift[i]) - 1);
+                    remt >>= p.out_shift[i];
+                    int idx = org_out[i] + c;
+                    ok = ok && idx < p.out_ext[i];
+                    oo += (long long)idx * p.out_os[i];
+                }
+            }
+            if (!ok)
+                continue;
+            float r[W];
+#pragma unroll
+            for (int j = 0; j < W; ++j) {
+                int e = t * W + j, lin = 0;
+#pragma unroll
+                for (int i = 0; i < kTileDims; ++i) {
+                    if (i < p.ntd) {
+                        lin += (e & ((1 << p.out_shift[i]) - 1)) << p.out_to_in_pos[i];
+                        e >>= p.out_shift[i];
+                    }
+                }
+                r[j] = lds[lin + (lin >> 5)];
+            }
+            if (VOUT) {
+                st4<NT>(y + oo, (vf4){r[0], r[W > 1 ? 1 : 0], r[W > 2 ? 2 : 0], r[W > 3 ? 3 : 0]});
+            } else {
+                if (NT)
+                    __builtin_nontemporal_store(r[0], y + oo);
+                else
+                    y[oo] = r[0];
             }
         }
-        if (ok)
-            y[oo] = lds[lin + (lin >> 5)];
     }
+}
+
+// Tensors beyond this many elements (256 MiB in + out) cannot stay in the
+// last-level cache between kernels: stream them with non-temporal accesses.
+static inline bool stream_sized(long long total) {
+    static const long long thr = getenv("PET_HIP_VIEW_NT")
+                                     ? atoll(getenv("PET_HIP_VIEW_NT"))
+                                     : (32ll << 20);
+    return total >= thr;
 }
 
 static inline bool plain(const ViewDim &d) {
@@ -313,6 +608,98 @@ int launch_view_copy(const float *x, float *y, ViewDesc v, long long in_elems,
     bool inner_coalesced_out = inner.os == 1;
     bool inner_coalesced_in = plain(inner) ? inner.sr == 1 : (inner.sr == 1);
 
+    // ---- interleave path: a 2- or 4-wide dim innermost on one side, adjacent to
+    // the dim that is innermost on the other side (space-to-batch and its inverse)
+    {
+        const bool aligned = c.ibase % 4 == 0 && c.obase % 4 == 0 && (uintptr_t)x % 16 == 0 &&
+                             (uintptr_t)y % 16 == 0;
+        int kE = -1, kW = -1;
+        bool deint = false;
+        if (aligned && plain(inner) && inner.os == 1 && (inner.sr == 2 || inner.sr == 4) &&
+            inner.ext % 4 == 0) {
+            // output innermost = w; look for the E dim (input innermost)
+            for (int i = 0; i < L; ++i)
+                if (plain(c.d[i]) && c.d[i].sr == 1 && c.d[i].ext == inner.sr && c.d[i].os % 4 == 0)
+                    kE = i;
+            kW = L;
+            deint = true;
+        } else if (aligned && plain(inner) && inner.os == 1 && (inner.ext == 2 || inner.ext == 4) &&
+                   inner.sr % 4 == 0) {
+            // output innermost = the E dim; look for w (input innermost)
+            for (int i = 0; i < L; ++i)
+                if (plain(c.d[i]) && c.d[i].sr == 1 && c.d[i].os == inner.ext &&
+                    c.d[i].ext % 4 == 0)
+                    kW = i;
+            kE = L;
+        }
+        bool ok = kE >= 0 && kW >= 0 && kE != kW;
+        for (int i = 0; ok && i < c.rank; ++i) {
+            if (i == kE || i == kW)
+                continue;
+            const ViewDim &d = c.d[i];
+            if (!plain(d) || d.os % 4 || d.sr % 4)
+                ok = false;
+        }
+        if (ok) {
+            InterleaveParams ip;
+            memset(&ip, 0, sizeof(ip));
+            DirectParams &p = ip.dp;
+            p.ibase = c.ibase;
+            p.obase = c.obase;
+            int r = 0;
+            auto put = [&](const ViewDim &d, int ext) {
+                p.ext[r] = make_fastdiv((unsigned)ext);
+                p.os[r] = d.os;
+                p.sr[r] = d.sr;
+                ++r;
+            };
+            for (int i = 0; i < c.rank; ++i)
+                if (i != kE && i != kW)
+                    put(c.d[i], c.d[i].ext);
+            const int E = c.d[kE].ext;
+            // E == 2: the last dim counts 16-byte words of the interleaved row
+            put(c.d[kW], E == 2 ? c.d[kW].ext / 2 : c.d[kW].ext / 4);
+            p.rank = r;
+            ip.e_stride = deint ? c.d[kE].os : c.d[kE].sr;
+            const long long items = E == 2 ? total / 4 : total / (4 * E);
+            p.total = (unsigned)items;
+            const bool nt = stream_sized(total);
+            const unsigned per_wg = 256u * (E == 2 ? 4 : 1);
+            const dim3 grid((unsigned)((items + per_wg - 1) / per_wg)), block(256);
+            if (E == 2) {
+                if (deint && nt)
+                    hipLaunchKernelGGL((view_interleave2_kernel<true, true>), grid, block, 0,
+                                       stream, x, y, ip);
+                else if (deint)
+                    hipLaunchKernelGGL((view_interleave2_kernel<true, false>), grid, block, 0,
+                                       stream, x, y, ip);
+                else if (nt)
+                    hipLaunchKernelGGL((view_interleave2_kernel<false, true>), grid, block, 0,
+                                       stream, x, y, ip);
+                else
+                    hipLaunchKernelGGL((view_interleave2_kernel<false, false>), grid, block, 0,
+                                       stream, x, y, ip);
+                return check_launch("view_interleave2_kernel");
+            }
+#define PET_IL(EE, DI, NTF)                                                                       \
+    hipLaunchKernelGGL((view_interleave_kernel<EE, DI, NTF>), grid, block, 0, stream, x, y, ip)
+#define PET_IL_NT(EE, DI)                                                                         \
+    do {                                                                                          \
+        if (nt)                                                                                   \
+            PET_IL(EE, DI, true);                                                                 \
+        else                                                                                      \
+            PET_IL(EE, DI, false);                                                                \
+    } while (0)
+            if (deint)
+                PET_IL_NT(4, true);
+            else
+                PET_IL_NT(4, false);
+#undef PET_IL_NT
+#undef PET_IL
+            return check_launch("view_interleave_kernel");
+        }
+    }
+
     // ---- tiled path: output-innermost dim is not the input-innermost one
     if (inner_coalesced_out && plain(inner) && inner.sr != 1 && total >= 4096) {
         // find the plain dim with the smallest positive input stride
@@ -360,15 +747,19 @@ int launch_view_copy(const float *x, float *y, ViewDesc v, long long in_elems,
                     acc += tsh[d];
                 }
             };
-            run(by_in, 6);
-            run(by_out, 6);
-            // grow towards 4096 elements: alternate between the two orders
+            static const int tl_env =
+                getenv("PET_HIP_VIEW_TILELOG") ? atoi(getenv("PET_HIP_VIEW_TILELOG")) : 0;
+            const int TL = tl_env ? tl_env : 12;
+            const int RL = TL / 2;
+            run(by_in, RL);
+            run(by_out, RL);
+            // grow towards 2^TL elements: alternate between the two orders
             bool grew = true;
-            while (tile_log() < 12 && grew) {
+            while (tile_log() < TL && grew) {
                 grew = false;
                 for (const std::vector<int> *ord : {&by_out, &by_in}) {
                     for (int d : *ord) {
-                        if (tile_log() >= 12)
+                        if (tile_log() >= TL)
                             break;
                         if (tsh[d] < ceil_log2(c.d[d].ext) &&
                             (tsh[d] > 0 || tile_dims() < kTileDims)) {
@@ -379,7 +770,7 @@ int launch_view_copy(const float *x, float *y, ViewDesc v, long long in_elems,
                     }
                 }
             }
-            if (tile_log() <= 12 && tile_dims() >= 2 && tile_dims() <= kTileDims) {
+            if (tile_log() <= TL && tile_dims() >= 2 && tile_dims() <= kTileDims) {
                 TiledParams p;
                 memset(&p, 0, sizeof(p));
                 p.rank = c.rank;
@@ -439,8 +830,60 @@ int launch_view_copy(const float *x, float *y, ViewDesc v, long long in_elems,
                 }
                 p.tile_elems = 1 << pos;
                 if (ngroups < (1ll << 31)) {
-                    hipLaunchKernelGGL(view_tiled_kernel, dim3((unsigned)ngroups), dim3(256), 0,
-                                       stream, x, y, p);
+                    // can the global side move 16 bytes per lane?
+                    auto vec_ok = [&](const std::vector<int> &ord, bool in_side) {
+                        auto stride = [&](int d) { return in_side ? c.d[d].sr : c.d[d].os; };
+                        const int d0 = ord[0];
+                        size_t first_free = 1;
+                        if (stride(d0) != 1)
+                            return false;
+                        if (tsh[d0] >= 2) {
+                            if (c.d[d0].ext % 4)
+                                return false;
+                        } else {
+                            // a 2-wide innermost dim: the next one must continue the run
+                            if (c.d[d0].ext != 2 || ord.size() < 2 || stride(ord[1]) != 2 ||
+                                c.d[ord[1]].ext % 2)
+                                return false;
+                            first_free = 2;
+                        }
+                        for (size_t i = first_free; i < ord.size(); ++i)
+                            if (stride(ord[i]) % 4)
+                                return false;
+                        for (int i = 0; i < c.rank; ++i) {
+                            if (tsh[i] > 0)
+                                continue;
+                            if (stride(i) % 4 || (in_side && c.d[i].m < c.d[i].ext && c.d[i].sq % 4))
+                                return false;
+                        }
+                        const long long base = in_side ? c.ibase : c.obase;
+                        const uintptr_t ptr = in_side ? (uintptr_t)x : (uintptr_t)y;
+                        return base % 4 == 0 && ptr % 16 == 0;
+                    };
+                    const bool vin = vec_ok(tin, true), vout = vec_ok(tout, false);
+                    const bool nt = stream_sized(total);
+                    const dim3 grid((unsigned)ngroups), block(256);
+                    const size_t lds_bytes =
+                        (size_t)(p.tile_elems + p.tile_elems / 32 + 1) * sizeof(float);
+#define PET_TILED(VI, VO, NTF)                                                                    \
+    hipLaunchKernelGGL((view_tiled_kernel<VI, VO, NTF>), grid, block, lds_bytes, stream, x, y, p)
+#define PET_TILED_NT(VI, VO)                                                                      \
+    do {                                                                                          \
+        if (nt)                                                                                   \
+            PET_TILED(VI, VO, true);                                                              \
+        else                                                                                      \
+            PET_TILED(VI, VO, false);                                                             \
+    } while (0)
+                    if (vin && vout)
+                        PET_TILED_NT(true, true);
+                    else if (vin)
+                        PET_TILED_NT(true, false);
+                    else if (vout)
+                        PET_TILED_NT(false, true);
+                    else
+                        PET_TILED_NT(false, false);
+#undef PET_TILED_NT
+#undef PET_TILED
                     return check_launch("view_tiled_kernel");
                 }
             }
@@ -481,13 +924,51 @@ int launch_view_copy(const float *x, float *y, ViewDesc v, long long in_elems,
         p.lo[L] = c.d[L].lo;
         p.hi[L] = c.d[L].hi;
     }
+    if (!vec && total % 4 == 0 && total >= 4096 && c.obase % 4 == 0 && (uintptr_t)y % 16 == 0) {
+        // is the output dense (row-major over the iteration dims)?
+        bool dense = true;
+        long long expect = 1;
+        for (int i = c.rank - 1; i >= 0; --i) {
+            if (c.d[i].os != expect)
+                dense = false;
+            expect *= c.d[i].ext;
+        }
+        if (dense) {
+            p.total = (unsigned)(total / 4);
+            const bool nt = stream_sized(total);
+            const dim3 grid((unsigned)((p.total + 511) / 512)), block(256);
+            if (nt)
+                hipLaunchKernelGGL(view_gather4_kernel<true>, grid, block, 0, stream, x, y, p);
+            else
+                hipLaunchKernelGGL(view_gather4_kernel<false>, grid, block, 0, stream, x, y, p);
+            return check_launch("view_gather4_kernel");
+        }
+    }
     long long items = vec ? total / 4 : total;
     p.total = (unsigned)items;
-    unsigned grid = (unsigned)std::min<long long>((items + 255) / 256, 1 << 20);
-    if (vec)
-        hipLaunchKernelGGL(view_direct_kernel<4>, dim3(grid), dim3(256), 0, stream, x, y, p);
-    else
-        hipLaunchKernelGGL(view_direct_kernel<1>, dim3(grid), dim3(256), 0, stream, x, y, p);
+    // four items per thread once that still leaves every CU several workgroups
+    const bool un4 = items >= 256ll * 4 * 2048;
+    const bool nt = stream_sized(total);
+    const unsigned per_wg = 256u * (un4 ? 4 : 1);
+    const dim3 grid((unsigned)((items + per_wg - 1) / per_wg)), block(256);
+#define PET_DIRECT(V, U, NTF)                                                                     \
+    hipLaunchKernelGGL((view_direct_kernel<V, U, NTF>), grid, block, 0, stream, x, y, p)
+    if (vec) {
+        if (un4 && nt)
+            PET_DIRECT(4, 4, true);
+        else if (un4)
+            PET_DIRECT(4, 4, false);
+        else
+            PET_DIRECT(4, 1, false);
+    } else {
+        if (un4 && nt)
+            PET_DIRECT(1, 4, true);
+        else if (un4)
+            PET_DIRECT(1, 4, false);
+        else
+            PET_DIRECT(1, 1, false);
+    }
+#undef PET_DIRECT
     return check_launch("view_direct_kernel");
 }
 
