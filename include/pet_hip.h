@@ -66,6 +66,14 @@ PET_HIP_API int pet_hip_shutdown(void);
 PET_HIP_API const char *pet_hip_last_error(void);
 /* name of the device's architecture ("gfx950") and number of compute units */
 PET_HIP_API int pet_hip_device_info(char *arch, size_t arch_len, int *num_cu);
+/* on != 0: contractions whose K loop is split over workgroups add their partial
+ * sums in a fixed order (one launch, partial tiles in library scratch), so equal
+ * inputs give bit-equal outputs from run to run. Off (the default) they use float
+ * atomics, which is faster and exact only up to summation order. The reference
+ * leaves this to the cuDNN algorithm it picks per convolution
+ * (src/Graph/operator.cc:296-515 loops over the algorithms). Environment variable
+ * PET_HIP_DETERMINISTIC=1 sets the initial value. */
+PET_HIP_API int pet_hip_set_deterministic(int on);
 
 /* ---- memory (cudaMalloc / cudaMemcpy / cudaFree call sites,
  * src/Graph/perf_engine.cc:31-47, src/Graph/code_engine.cc:560-643) ---------- */

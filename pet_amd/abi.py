@@ -23,6 +23,7 @@ SIGNATURES = {
     "pet_hip_init": [_i],
     "pet_hip_shutdown": [],
     "pet_hip_device_info": [ctypes.c_char_p, _sz, _c_int_p],
+    "pet_hip_set_deterministic": [ctypes.c_int],
     "pet_hip_malloc": [ctypes.POINTER(_vp), _sz],
     "pet_hip_free": [_vp],
     "pet_hip_memcpy_h2d": [_vp, _vp, _sz, _vp],

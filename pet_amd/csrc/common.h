@@ -14,6 +14,8 @@ namespace pet {
 char *err_buf();
 int set_error(int status, const char *fmt, ...);
 bool initialised();
+// Whether split contractions must add their partial sums in a fixed order.
+bool deterministic();
 // Split-K scratch owned by the library (see runtime.hip).
 void splitk_workspace(float **ws, size_t *ws_elems, int **counters, int *num_counters);
 

@@ -24,13 +24,25 @@ int set_error(int status, const char *fmt, ...) {
 bool initialised() { return g_init.load(); }
 
 // Library-owned scratch for split-K contractions: partial tiles and one arrival
-// counter per output tile. Allocated once in pet_hip_init (the reference's
+// counter per output tile (zero between launches). Allocated once in pet_hip_init (the reference's
 // PerfEngine likewise owns its cuDNN workspace, src/Graph/perf_engine.cc:31-42).
 // Launches that use it must not overlap on different streams.
 static float *g_ws = nullptr;
 static int *g_cnt = nullptr;
-constexpr size_t kWsElems = (size_t)16 << 20; // 64 MiB of floats
+constexpr size_t kWsElems = (size_t)8 << 20; // 32 MiB of floats
 constexpr int kNumCounters = 16384;
+
+static std::atomic<int> g_deterministic{-1};
+
+bool deterministic() {
+    int v = g_deterministic.load();
+    if (v < 0) {
+        const char *e = getenv("PET_HIP_DETERMINISTIC");
+        v = e && atoi(e) != 0;
+        g_deterministic.store(v);
+    }
+    return v != 0;
+}
 
 void splitk_workspace(float **ws, size_t *ws_elems, int **counters, int *num_counters) {
     *ws = g_ws;
@@ -117,6 +129,11 @@ int pet_hip_shutdown(void) {
 }
 
 const char *pet_hip_last_error(void) { return err_buf(); }
+
+int pet_hip_set_deterministic(int on) {
+    pet::g_deterministic.store(on != 0);
+    return PET_HIP_OK;
+}
 
 int pet_hip_device_info(char *arch, size_t arch_len, int *num_cu) {
     PET_REQUIRE_INIT();

@@ -129,16 +129,21 @@ __global__ __launch_bounds__(256) void view_direct_kernel(const float *__restric
     }
 }
 
-// Index of one element of the iteration space -> input offset and validity.
-// 32-bit wrap-around arithmetic: both buffers hold fewer than 2^31 elements, so
-// the offset of every valid element is exact modulo 2^32.
-__device__ __forceinline__ void decode_in(const DirectParams &p, unsigned e, unsigned &io,
-                                          bool &ok) {
+// Index of one element of the iteration space -> input offset and validity,
+// split into the innermost dim and the rest so that neighbours along a row reuse
+// the outer part. 32-bit wrap-around arithmetic: both buffers hold fewer than
+// 2^31 elements, so the offset of every valid element is exact modulo 2^32.
+__device__ __forceinline__ void decode_outer(const DirectParams &p, unsigned e, unsigned &inner,
+                                             unsigned &io, bool &ok) {
     io = (unsigned)p.ibase;
+    const int L = p.rank - 1;
+    unsigned q = fd_div(e, p.ext[L]);
+    inner = e - q * p.ext[L].d;
+    e = q;
 #pragma unroll
-    for (int d = PET_HIP_MAX_RANK - 1; d >= 0; --d) {
-        if (d < p.rank) {
-            unsigned q = fd_div(e, p.ext[d]);
+    for (int d = PET_HIP_MAX_RANK - 2; d >= 0; --d) {
+        if (d < L) {
+            q = fd_div(e, p.ext[d]);
             unsigned r = e - q * p.ext[d].d;
             e = q;
             if (p.has_div[d]) {
@@ -152,6 +157,18 @@ __device__ __forceinline__ void decode_in(const DirectParams &p, unsigned e, uns
     }
 }
 
+__device__ __forceinline__ void eval_inner(const DirectParams &p, unsigned r, unsigned &io,
+                                           bool &ok) {
+    const int L = p.rank - 1;
+    if (p.has_div[L]) {
+        unsigned qq = fd_div(r, p.m[L]);
+        r -= qq * p.m[L].d;
+        io += qq * (unsigned)p.sq[L];
+    }
+    io += r * (unsigned)p.sr[L];
+    ok = ok && ((int)r >= p.lo[L]) && ((int)r < p.hi[L]);
+}
+
 // Dense, 16-byte aligned output but an input side that cannot be vectorised (an
 // innermost extent that is not a multiple of 4, a window that cuts through
 // it): a thread gathers 4 consecutive output elements one by one and stores
@@ -161,17 +178,27 @@ template <bool NT>
 __global__ __launch_bounds__(256) void view_gather4_kernel(const float *__restrict__ x,
                                                            float *__restrict__ y,
                                                            DirectParams p) {
-    constexpr int UN = 2;
+    constexpr int UN = 4;
     const unsigned base = blockIdx.x * (256u * UN) + threadIdx.x;
+    const unsigned ext_inner = p.ext[p.rank - 1].d;
     float v[UN][4];
 #pragma unroll
     for (int u = 0; u < UN; ++u) {
         const unsigned t = base + u * 256u;
+        const bool live = t < p.total;
+        const unsigned e0 = live ? t * 4u : 0u;
+        unsigned inner, io_outer;
+        bool ok_outer = live;
+        decode_outer(p, e0, inner, io_outer, ok_outer);
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
-            unsigned io;
-            bool ok = t < p.total;
-            decode_in(p, ok ? t * 4u + j : 0u, io, ok);
+            if (j > 0 && ++inner == ext_inner) { // next row: decode afresh
+                ok_outer = live;
+                decode_outer(p, e0 + j, inner, io_outer, ok_outer);
+            }
+            unsigned io = io_outer;
+            bool ok = ok_outer;
+            eval_inner(p, inner, io, ok);
             v[u][j] = 0.f;
             if (ok)
                 v[u][j] = NT ? __builtin_nontemporal_load(x + io) : x[io];
@@ -187,76 +214,13 @@ __global__ __launch_bounds__(256) void view_gather4_kernel(const float *__restri
 
 // Interleave kernels for the space-to-batch family: a dim of extent E (2 or 4)
 // that is innermost on one side sits next to the dim that is innermost on the
-// other side. Each thread moves a 4 x E block through registers, with 16-byte
-// accesses on both sides and no LDS.
+// other side. DEINT: the input holds (w, e) with e innermost and the output has
+// w innermost with the planes e far apart (space-to-batch); otherwise the
+// reverse (batch-to-space). 16-byte accesses on both sides, no LDS.
 struct InterleaveParams {
     DirectParams dp;   // the iteration space without the E dim; innermost dim in units of 4
     long long e_stride; // stride of the E dim on the side where it is not innermost
 };
-
-// DEINT: input holds (w, e) pairs with e innermost; output has w innermost and
-// e far away (space-to-batch). Otherwise the reverse (batch-to-space).
-template <int E, bool DEINT, bool NT>
-__global__ __launch_bounds__(256) void view_interleave_kernel(const float *__restrict__ x,
-                                                              float *__restrict__ y,
-                                                              InterleaveParams ip) {
-    const DirectParams &p = ip.dp;
-    constexpr int UN = 1;
-    const unsigned base = blockIdx.x * (256u * UN) + threadIdx.x;
-    unsigned io[UN], oo[UN];
-    bool live[UN];
-    vf4 a[UN][E];
-#pragma unroll
-    for (int u = 0; u < UN; ++u) {
-        const unsigned t = base + u * 256u;
-        live[u] = t < p.total;
-        unsigned rem = live[u] ? t : 0u;
-        io[u] = (unsigned)p.ibase;
-        oo[u] = (unsigned)p.obase;
-#pragma unroll
-        for (int d = PET_HIP_MAX_RANK - 1; d >= 0; --d) {
-            if (d < p.rank) {
-                unsigned q = fd_div(rem, p.ext[d]);
-                unsigned idx = rem - q * p.ext[d].d;
-                rem = q;
-                if (d == p.rank - 1)
-                    idx *= 4;
-                oo[u] += idx * (unsigned)p.os[d];
-                io[u] += idx * (unsigned)p.sr[d];
-            }
-        }
-        if (live[u]) {
-#pragma unroll
-            for (int e = 0; e < E; ++e)
-                a[u][e] = ld4<NT>(x + io[u] + (DEINT ? 4u * e : (unsigned)ip.e_stride * e));
-        }
-    }
-#pragma unroll
-    for (int u = 0; u < UN; ++u) {
-        if (!live[u])
-            continue;
-        float m[4 * E];
-#pragma unroll
-        for (int e = 0; e < E; ++e) {
-            m[4 * e + 0] = a[u][e].x;
-            m[4 * e + 1] = a[u][e].y;
-            m[4 * e + 2] = a[u][e].z;
-            m[4 * e + 3] = a[u][e].w;
-        }
-#pragma unroll
-        for (int e = 0; e < E; ++e) {
-            vf4 o;
-            if (DEINT) // m is [w][e]: pick plane e
-                o = (vf4){m[0 * E + e], m[1 * E + e], m[2 * E + e], m[3 * E + e]};
-            else       // m is [e][w]: output word e holds flat positions 4e .. 4e+3 of [w][e]
-                o = (vf4){m[((4 * e + 0) % E) * 4 + (4 * e + 0) / E],
-                          m[((4 * e + 1) % E) * 4 + (4 * e + 1) / E],
-                          m[((4 * e + 2) % E) * 4 + (4 * e + 2) / E],
-                          m[((4 * e + 3) % E) * 4 + (4 * e + 3) / E]};
-            st4<NT>(y + oo[u] + (DEINT ? (unsigned)ip.e_stride * e : 4u * e), o);
-        }
-    }
-}
 
 // The 2-wide case moves whole cache lines on both sides: a lane handles one
 // 16-byte word of the interleaved side and, with its neighbour (lane ^ 1),
@@ -317,6 +281,69 @@ __global__ __launch_bounds__(256) void view_interleave2_kernel(const float *__re
         }
         if (live[u])
             st4<NT>(y + oo[u], o);
+    }
+}
+
+// The 4-wide case: a lane holds one 16-byte word (one position, four planes, or
+// the reverse); the four lanes of a quad transpose their 4x4 block in three
+// exchange rounds. p's last dim counts positions of the interleaved row.
+template <bool DEINT, bool NT>
+__global__ __launch_bounds__(256) void view_interleave4_kernel(const float *__restrict__ x,
+                                                               float *__restrict__ y,
+                                                               InterleaveParams ip) {
+    const DirectParams &p = ip.dp;
+    constexpr int UN = 4;
+    const unsigned base = blockIdx.x * (256u * UN) + threadIdx.x;
+    const unsigned q4 = threadIdx.x & 3;
+    unsigned oo[UN];
+    bool live[UN];
+    vf4 a[UN];
+#pragma unroll
+    for (int u = 0; u < UN; ++u) {
+        const unsigned t = base + u * 256u;
+        live[u] = t < p.total; // the same for a whole quad: total is a multiple of 4
+        unsigned rem = live[u] ? t : 0u;
+        unsigned io = (unsigned)p.ibase;
+        oo[u] = (unsigned)p.obase;
+#pragma unroll
+        for (int d = PET_HIP_MAX_RANK - 1; d >= 0; --d) {
+            if (d < p.rank) {
+                unsigned q = fd_div(rem, p.ext[d]);
+                unsigned idx = rem - q * p.ext[d].d;
+                rem = q;
+                if (d == p.rank - 1) {
+                    const unsigned planar = 4u * (idx >> 2) + (idx & 3) * (unsigned)ip.e_stride;
+                    io += DEINT ? 4u * idx : planar;
+                    oo[u] += DEINT ? planar : 4u * idx;
+                } else {
+                    oo[u] += idx * (unsigned)p.os[d];
+                    io += idx * (unsigned)p.sr[d];
+                }
+            }
+        }
+        a[u] = (vf4){0.f, 0.f, 0.f, 0.f};
+        if (live[u])
+            a[u] = ld4<NT>(x + io);
+    }
+#pragma unroll
+    for (int u = 0; u < UN; ++u) {
+        const vf4 v = a[u];
+        float o[4];
+#pragma unroll
+        for (int r = 0; r < 4; ++r) {
+            // partner = q4 ^ r: it needs my element `partner`, I need its element q4
+            const unsigned pr = q4 ^ r;
+            const float send = pr == 0 ? v.x : pr == 1 ? v.y : pr == 2 ? v.z : v.w;
+            const float recv = r == 0 ? send : __shfl_xor(send, r);
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+                if (r == 0)
+                    o[j] = recv; // every slot is overwritten below except slot q4
+                else
+                    o[j] = pr == (unsigned)j ? recv : o[j];
+        }
+        if (live[u])
+            st4<NT>(y + oo[u], (vf4){o[0], o[1], o[2], o[3]});
     }
 }
 
@@ -493,6 +520,20 @@ static inline bool stream_sized(long long total) {
     return total >= thr;
 }
 
+template <bool VI, bool VO, bool NTF>
+static void launch_tiled(dim3 grid, size_t lds_bytes, hipStream_t stream, const float *x, float *y,
+                         const TiledParams &p) {
+    // tiles beyond 64 KiB of LDS need the limit raised once per kernel
+    static const bool raised = [] {
+        return hipFuncSetAttribute(
+                   reinterpret_cast<const void *>(&view_tiled_kernel<VI, VO, NTF>),
+                   hipFuncAttributeMaxDynamicSharedMemorySize, 72 * 1024) == hipSuccess;
+    }();
+    (void)raised;
+    hipLaunchKernelGGL((view_tiled_kernel<VI, VO, NTF>), grid, dim3(256), lds_bytes, stream, x, y,
+                       p);
+}
+
 static inline bool plain(const ViewDim &d) {
     return d.m >= d.ext && d.lo <= 0 && d.hi >= d.ext;
 }
@@ -658,13 +699,13 @@ int launch_view_copy(const float *x, float *y, ViewDesc v, long long in_elems,
                     put(c.d[i], c.d[i].ext);
             const int E = c.d[kE].ext;
             // E == 2: the last dim counts 16-byte words of the interleaved row
-            put(c.d[kW], E == 2 ? c.d[kW].ext / 2 : c.d[kW].ext / 4);
+            put(c.d[kW], E == 2 ? c.d[kW].ext / 2 : c.d[kW].ext);
             p.rank = r;
             ip.e_stride = deint ? c.d[kE].os : c.d[kE].sr;
-            const long long items = E == 2 ? total / 4 : total / (4 * E);
+            const long long items = total / 4;
             p.total = (unsigned)items;
             const bool nt = stream_sized(total);
-            const unsigned per_wg = 256u * (E == 2 ? 4 : 1);
+            const unsigned per_wg = 256u * 4;
             const dim3 grid((unsigned)((items + per_wg - 1) / per_wg)), block(256);
             if (E == 2) {
                 if (deint && nt)
@@ -681,22 +722,19 @@ int launch_view_copy(const float *x, float *y, ViewDesc v, long long in_elems,
                                        stream, x, y, ip);
                 return check_launch("view_interleave2_kernel");
             }
-#define PET_IL(EE, DI, NTF)                                                                       \
-    hipLaunchKernelGGL((view_interleave_kernel<EE, DI, NTF>), grid, block, 0, stream, x, y, ip)
-#define PET_IL_NT(EE, DI)                                                                         \
-    do {                                                                                          \
-        if (nt)                                                                                   \
-            PET_IL(EE, DI, true);                                                                 \
-        else                                                                                      \
-            PET_IL(EE, DI, false);                                                                \
-    } while (0)
-            if (deint)
-                PET_IL_NT(4, true);
+            if (deint && nt)
+                hipLaunchKernelGGL((view_interleave4_kernel<true, true>), grid, block, 0, stream, x,
+                                   y, ip);
+            else if (deint)
+                hipLaunchKernelGGL((view_interleave4_kernel<true, false>), grid, block, 0, stream,
+                                   x, y, ip);
+            else if (nt)
+                hipLaunchKernelGGL((view_interleave4_kernel<false, true>), grid, block, 0, stream,
+                                   x, y, ip);
             else
-                PET_IL_NT(4, false);
-#undef PET_IL_NT
-#undef PET_IL
-            return check_launch("view_interleave_kernel");
+                hipLaunchKernelGGL((view_interleave4_kernel<false, false>), grid, block, 0, stream,
+                                   x, y, ip);
+            return check_launch("view_interleave4_kernel");
         }
     }
 
@@ -749,7 +787,8 @@ int launch_view_copy(const float *x, float *y, ViewDesc v, long long in_elems,
             };
             static const int tl_env =
                 getenv("PET_HIP_VIEW_TILELOG") ? atoi(getenv("PET_HIP_VIEW_TILELOG")) : 0;
-            const int TL = tl_env ? tl_env : 12;
+            // 8192-element tiles (512-byte runs on both sides) once there are thousands of them
+            const int TL = tl_env ? tl_env : (total >= (1ll << 23) ? 13 : 12);
             const int RL = TL / 2;
             run(by_in, RL);
             run(by_out, RL);
@@ -865,8 +904,7 @@ int launch_view_copy(const float *x, float *y, ViewDesc v, long long in_elems,
                     const dim3 grid((unsigned)ngroups), block(256);
                     const size_t lds_bytes =
                         (size_t)(p.tile_elems + p.tile_elems / 32 + 1) * sizeof(float);
-#define PET_TILED(VI, VO, NTF)                                                                    \
-    hipLaunchKernelGGL((view_tiled_kernel<VI, VO, NTF>), grid, block, lds_bytes, stream, x, y, p)
+#define PET_TILED(VI, VO, NTF) launch_tiled<VI, VO, NTF>(grid, lds_bytes, stream, x, y, p)
 #define PET_TILED_NT(VI, VO)                                                                      \
     do {                                                                                          \
         if (nt)                                                                                   \
@@ -936,7 +974,7 @@ int launch_view_copy(const float *x, float *y, ViewDesc v, long long in_elems,
         if (dense) {
             p.total = (unsigned)(total / 4);
             const bool nt = stream_sized(total);
-            const dim3 grid((unsigned)((p.total + 511) / 512)), block(256);
+            const dim3 grid((unsigned)((p.total + 1023) / 1024)), block(256);
             if (nt)
                 hipLaunchKernelGGL(view_gather4_kernel<true>, grid, block, 0, stream, x, y, p);
             else

@@ -102,6 +102,40 @@ def test_conv2d_bias_act_epilogue(ops):
     np.testing.assert_array_equal(got, ref)
 
 
+@pytest.mark.parametrize("case", [CONV_CASES[11], CONV_CASES[15]])
+def test_conv2d_split_contraction_both_modes(ops, case):
+    """Layers whose K loop is split over workgroups: the default (float atomics)
+    and the deterministic mode (ordered sum of partial tiles, one launch) both meet
+    the tolerance and are bit-exact on small integers; the deterministic mode
+    repeats itself bit for bit, also right after a launch with a different shape
+    has used the same scratch."""
+    from pet_amd import abi
+    n, c, h, w, f, cpg, r, s, ph, pw, sh, sw, dh, dw = case
+    rng = np.random.default_rng(5)
+    x = rng.uniform(-1, 1, (n, c, h, w)).astype(np.float32)
+    wt = rng.uniform(-1, 1, (f, cpg, r, s)).astype(np.float32)
+    b = rng.uniform(-1, 1, (f,)).astype(np.float32)
+    xi, wi = ints(rng, (n, c, h, w)), ints(rng, (f, cpg, r, s))
+    ref = oracle.bias_act(oracle.conv2d(x, wt, ph, pw, sh, sw, dh, dw), b, "relu")
+    mag = oracle.conv2d(np.abs(x), np.abs(wt), ph, pw, sh, sw, dh, dw) + np.abs(b)[None, :, None, None]
+    refi = oracle.conv2d(xi, wi, ph, pw, sh, sw, dh, dw)
+    dx, dw_, db, dxi, dwi = dev(x), dev(wt), dev(b), dev(xi), dev(wi)
+    try:
+        for on in (0, 1):
+            abi.call("pet_hip_set_deterministic", on)
+            got = host(ops.conv2d(dx, dw_, ph, pw, sh, sw, dh, dw, bias=db, act="relu"))
+            assert max_rel_err(got, ref, mag) <= REL_TOL
+            np.testing.assert_array_equal(
+                host(ops.conv2d(dxi, dwi, ph, pw, sh, sw, dh, dw)), refi)
+            if on:
+                other = ops.conv2d(dev(ints(rng, (1, 128, 14, 14))), dev(ints(rng, (64, 128, 3, 3))), 1, 1)
+                again = host(ops.conv2d(dx, dw_, ph, pw, sh, sw, dh, dw, bias=db, act="relu"))
+                np.testing.assert_array_equal(again, got)
+                del other
+    finally:
+        abi.call("pet_hip_set_deterministic", 0)
+
+
 def test_conv2d_rejects_bad_groups(ops):
     from pet_amd import abi
     x = torch.zeros((1, 4, 5, 5), device="cuda")
