@@ -386,7 +386,8 @@ __global__ __launch_bounds__(Cfg::NT) void conv_plane_kernel(ConvParams p) {
         for (int i = 0; i < RPW; ++i) {
             const int kl = wave + NW * i; // row of the B tile: (c_local, r, s)
             const int cl = kl / RS, t = kl % RS;
-            const int r = t / p.S, s = t - r * p.S;
+            constexpr int SW = RS == 9 ? 3 : 1; // the host admits 3x3 and 1x1 planes only
+            const int r = t / SW, s = t - r * SW;
             const int rh = r * p.dh, sw_ = s * p.dw;
             const unsigned roff = (unsigned)(cl * THW + rh * p.W + sw_);
 #pragma unroll
@@ -821,8 +822,12 @@ int launch_plane(const ConvParams &p, bool is3d, hipStream_t stream) {
     using C32x64 = PlaneCfg<32, 64, 1, 2, RS, CB>;
     // 64x128 when it alone fills the GPU; otherwise 64x64 (two workgroups fit a
     // CU, and split-K supplies the missing parallelism); 32x64 for M <= 32
+    // 64x128 tiles (one workgroup per CU) once they fill the chip and the K loop
+    // is long; with 16 steps or fewer two co-resident 64x64 workgroups hide each
+    // other's prologue and epilogue
     int tile = p.M > 32 ? 1 : 2;
-    if (p.M > 32 && tiles_for(p.M, p.NPIX, 64, 128, p.G) >= 200)
+    const int nit = (p.cpg / CB) * p.KT;
+    if (p.M > 32 && tiles_for(p.M, p.NPIX, 64, 128, p.G) >= 200 && nit > 16)
         tile = 0;
     if (forced_tile() >= 0)
         tile = forced_tile() % 3;
@@ -849,7 +854,7 @@ int try_launch_plane(const ConvParams &p, hipStream_t stream) {
         return -1;
     const bool is3d = p.T > 1 || p.KT > 1 || p.pt > 0 || p.st > 1;
     const int rs = p.R * p.S;
-    if (rs == 9 && p.cpg % 8 == 0)
+    if (rs == 9 && p.R == 3 && p.cpg % 8 == 0)
         return launch_plane<9, 8>(p, is3d, stream);
     if (rs == 1 && p.cpg % 32 == 0)
         return launch_plane<1, 32>(p, is3d, stream);
