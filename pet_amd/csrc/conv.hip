@@ -280,8 +280,8 @@ __global__ __launch_bounds__(Cfg::NT) void conv_pipe_kernel(ConvParams p) {
 // 16 instructions per MFMA.
 //
 // Schedule of step kt (NM slots, one MFMA each): first half, W(kt+1): prefetch
-// registers -> LDS; barrier; second half, R(kt+1): LDS -> the other fragment
-// register set, and G(kt+2): global -> prefetch registers.
+// registers -> LDS, each piece followed by G(kt+2): global -> the registers just
+// emptied; barrier; second half, R(kt+1): LDS -> the other fragment register set.
 template <int BM_, int BN_, int WGM_, int WGN_, int RS_, int CB_>
 struct PlaneCfg {
     static constexpr int BM = BM_, BN = BN_, WGM = WGM_, WGN = WGN_, RS = RS_, CB = CB_;
@@ -539,30 +539,25 @@ __global__ __launch_bounds__(Cfg::NT) void conv_plane_kernel(ConvParams p) {
             acc[tm][tn] = __builtin_amdgcn_mfma_f32_32x32x2f32(fa[PAR][tm][j], fb[PAR][j][tn],
                                                                acc[tm][tn], 0, 0, 0);
             if (s < HALF) {
-                const int pb_ = (s * NWP + HALF - 1) / HALF, pe_ = ((s + 1) * NWP + HALF - 1) / HALF;
+                // W(kt+1) piece i, then G(kt+2) piece i straight into the registers it
+                // has just emptied: a load has a whole step to land
+                constexpr int NP = 2 * NWP;
+                const int pb_ = (s * NP + HALF - 1) / HALF, pe_ = ((s + 1) * NP + HALF - 1) / HALF;
 #pragma unroll
-                for (int q = pb_; q < pe_; ++q)
-                    w_piece(q, nxt);
+                for (int q = pb_; q < pe_; ++q) {
+                    if (q & 1)
+                        g_piece(q >> 1);
+                    else
+                        w_piece(q >> 1, nxt);
+                }
                 if (s == HALF - 1)
                     wg_barrier();
             } else {
                 const int h = s - HALF, HN = NM - HALF;
-                const int pb_ = (h * NPOST + HN - 1) / HN, pe_ = ((h + 1) * NPOST + HN - 1) / HN;
+                const int pb_ = (h * NR + HN - 1) / HN, pe_ = ((h + 1) * NR + HN - 1) / HN;
 #pragma unroll
-                for (int q = pb_; q < pe_; ++q) {
-                    // fragment reads and prefetches alternate, the longer list runs on
-                    constexpr int NMIN = NR < NG ? NR : NG;
-                    if (q < 2 * NMIN) {
-                        if (q & 1)
-                            g_piece(q >> 1);
-                        else
-                            r_piece(PAR ^ 1, q >> 1, nxt);
-                    } else if (NR > NG) {
-                        r_piece(PAR ^ 1, q - NMIN, nxt);
-                    } else {
-                        g_piece(q - NMIN);
-                    }
-                }
+                for (int q = pb_; q < pe_; ++q)
+                    r_piece(PAR ^ 1, q, nxt);
             }
             __builtin_amdgcn_sched_barrier(0);
         }
