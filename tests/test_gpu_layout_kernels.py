@@ -1,0 +1,152 @@
+"""Bit-exact checks of every kernel the layout engine can pick, with shapes chosen
+to land on each one (and on its ragged / unaligned fall-backs): direct copies
+with 1 and 4 items per thread, streaming (non-temporal) variants, the 2- and
+4-wide interleave kernels behind space-to-batch, the packed-store gather, and
+the LDS-tiled transposes with 16-byte access on either, both or neither side."""
+import numpy as np
+import pytest
+import torch
+
+import oracle
+
+pytestmark = pytest.mark.gpu
+
+
+@pytest.fixture(scope="module")
+def ops():
+    from pet_amd import ops as _ops
+    return _ops
+
+
+def dev(a):
+    return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+
+def host(t):
+    torch.cuda.synchronize()
+    return t.cpu().numpy()
+
+
+def iota(shape):
+    # distinct values, exact in fp32 up to 2^24 elements; beyond that a second
+    # pattern keeps neighbours distinguishable
+    n = int(np.prod(shape))
+    a = np.arange(n, dtype=np.int64)
+    return ((a % 16777213) - 8388606).astype(np.float32).reshape(shape)
+
+
+def check_perm(ops, flat, perm):
+    x = iota(flat)
+    ref = oracle.permute_flat(x, list(flat), list(perm))
+    got = host(ops.permute_flat(dev(x), list(flat), list(perm)))
+    assert got.shape == ref.shape
+    assert got.tobytes() == ref.tobytes()
+
+
+S2B = [3, 5, 0, 1, 2, 4]   # [n, c, h/d, d, w/d, d] -> [d, d, n, c, h/d, w/d]
+B2S = [2, 3, 4, 0, 5, 1]   # [d, d, n, c, h/d, w/d] -> [n, c, h/d, d, w/d, d]
+
+
+@pytest.mark.parametrize("n,c,h,w,d", [
+    (1, 8, 16, 16, 2),     # 2-wide interleave kernel
+    (2, 3, 6, 24, 2),
+    (1, 5, 4, 8, 2),
+    (1, 8, 16, 12, 2),     # w/d = 6: not a multiple of 4 -> tiled / direct fall-back
+    (1, 4, 6, 10, 2),
+    (1, 8, 16, 16, 4),     # 4-wide interleave kernel
+    (2, 3, 8, 32, 4),
+    (1, 4, 8, 24, 4),      # w/d = 6 -> fall-back
+    (1, 6, 12, 12, 3),     # dilation 3: never the interleave kernels
+    (1, 512, 64, 64, 2),   # the bench shape
+])
+def test_space_to_batch_and_back(ops, n, c, h, w, d):
+    check_perm(ops, [n, c, h // d, d, w // d, d], S2B)
+    check_perm(ops, [d, d, n, c, h // d, w // d], B2S)
+
+
+def test_interleave_streaming_variants_round_trip(ops):
+    """32 Mi elements: the non-temporal variants. Checked against the oracle on the
+    forward pass and by the round trip."""
+    n, c, h, w, d = 2, 256, 256, 256, 2
+    flat = [n, c, h // d, d, w // d, d]
+    x = iota(flat)
+    ref = oracle.permute_flat(x, flat, S2B)
+    dx = dev(x)
+    y = ops.permute_flat(dx, flat, S2B)
+    assert host(y).tobytes() == ref.tobytes()
+    back = ops.permute_flat(y, [d, d, n, c, h // d, w // d], B2S)
+    assert torch.equal(back.reshape(-1), dx.reshape(-1))
+    del y, back
+    d = 4
+    flat = [n, c, h // d, d, w // d, d]
+    y = ops.permute_flat(dx.reshape(flat), flat, S2B)
+    assert host(y).tobytes() == oracle.permute_flat(x.reshape(flat), flat, S2B).tobytes()
+    back = ops.permute_flat(y, [d, d, n, c, h // d, w // d], B2S)
+    assert torch.equal(back.reshape(-1), dx.reshape(-1))
+
+
+@pytest.mark.parametrize("flat,perm", [
+    ([33, 65], [1, 0]),                    # scalar tiled, ragged both ways
+    ([64, 64], [1, 0]),                    # 16 bytes on both sides
+    ([1000, 1000], [1, 0]),
+    ([128, 66], [1, 0]),                   # 16 bytes on the input side only (66 % 4 != 0 out rows)
+    ([66, 128], [1, 0]),                   # ... on the output side only
+    ([5, 300, 70], [2, 0, 1]),
+    ([12, 128, 64], [0, 2, 1]),            # matmul operand transpose
+    ([7, 9, 11, 13], [3, 2, 1, 0]),        # 4 tile dims
+    ([4, 6, 8, 10, 12], [4, 2, 0, 3, 1]),
+    ([2048, 4100], [1, 0]),                # 8.4 Mi elements: 8192-element tiles, ragged edge
+    ([64, 256, 1024], [0, 2, 1]),          # 16 Mi elements, NCHW -> NHWC
+])
+def test_tiled_transposes(ops, flat, perm):
+    check_perm(ops, flat, perm)
+
+
+@pytest.mark.parametrize("flat,perm", [
+    ([4, 64, 2, 28, 56], [2, 0, 1, 3, 4]),      # H2N: outer-dim move, 16-byte direct copy
+    ([128, 12, 64], [1, 0, 2]),                 # attention head split
+    ([16, 64, 2, 64, 128], [2, 0, 1, 3, 4]),    # 16 Mi elements: four items per thread
+    ([3, 5, 7, 9], [1, 0, 2, 3]),               # innermost extent 9: scalar direct / gather
+    ([6, 10, 14, 14], [1, 0, 2, 3]),            # innermost rows of 14*14 = 196 (merged), aligned
+    ([6, 10, 7, 7], [1, 0, 2, 3]),              # 49-element rows: unaligned gather
+])
+def test_direct_copies(ops, flat, perm):
+    check_perm(ops, flat, perm)
+
+
+def test_direct_streaming_variant(ops):
+    flat, perm = [32, 2, 64, 64, 128], [1, 0, 2, 3, 4]   # 32 Mi elements
+    check_perm(ops, flat, perm)
+
+
+@pytest.mark.parametrize("shape,begin,end", [
+    ((2, 3, 14, 14), (0, 0, 1, 1), (0, 0, 1, 1)),        # 16-wide output rows, 14-wide input
+    ((2, 3, 13, 11), (0, 0, 2, 3), (0, 0, 0, 2)),        # 16-wide output rows, odd input
+    ((4, 8, 30, 30), (0, 0, 1, 1), (0, 0, 1, 1)),
+    ((1, 64, 126, 126), (0, 0, 1, 1), (0, 0, 1, 1)),     # 1 Mi outputs
+    ((3, 5, 7), (1, 0, 1), (0, 2, 0)),                   # output rows of 8
+    ((3, 5, 7), (1, 1, 1), (1, 1, 1)),                   # output rows of 9: scalar path
+])
+def test_pad_then_slice_back(ops, shape, begin, end):
+    x = iota(shape)
+    ref = oracle.pad(x, list(begin), list(end))
+    p = ops.pad(dev(x), list(begin), list(end))
+    assert host(p).tobytes() == ref.tobytes()
+    back = ops.slice_(p, list(begin), list(end))
+    assert host(back).tobytes() == x.tobytes()
+
+
+@pytest.mark.parametrize("shape,dim,num", [((2, 6, 7, 7), 1, 2), ((4, 8, 16), 0, 1), ((3, 5, 12), 2, 3)])
+def test_extend(ops, shape, dim, num):
+    x = iota(shape)
+    assert host(ops.extend(dev(x), dim, num)).tobytes() == oracle.extend(x, dim, num).tobytes()
+
+
+def test_halo_chain_on_width(ops):
+    """W2N with a one-column halo, then N2W dropping it: the gather path with a
+    window that cuts through rows."""
+    x = iota((2, 4, 12, 16))
+    chain = [("split", 3, 8, 0, 1), ("reorder", [0, 3, 1, 2, 4]), ("fuse", 0, 0, 0)]
+    ref = oracle.trans_chain(x, chain)
+    got = host(ops.trans_chain(dev(x), chain))
+    assert got.shape == ref.shape and got.tobytes() == ref.tobytes()
