@@ -35,6 +35,8 @@ struct ConvParams {
     int splitk;    // plane kernel: K steps are dealt to this many workgroups per tile
     int xcd_chunk; // plane kernel: tiles per XCD when the tile grid is dealt in bands (0: off)
     int xcd_mg;    // ... and how many M tiles wide a band is
+    FastDiv fd_band, fd_mg, fd_splitk; // divisions by xcd_mg * grid.x, xcd_mg and splitk
+    int vec_out;   // plane kernel: OPIX % 4 == 0 and y 16-byte aligned: 16-byte output words
     int sk_mode;   // split-K: 0 partial tiles + ordered sum in one launch, 1 atomics into y
     float *ws;     // split-K: partial tiles, [tile][split][register][thread]
     int *cnt;      // split-K: arrival counter per tile, zero between launches
@@ -333,7 +335,7 @@ __global__ __launch_bounds__(Cfg::NT) void conv_plane_kernel(ConvParams p) {
     const int wm0 = (wave / Cfg::WGN) * Cfg::WM;
     const int wn0 = (wave % Cfg::WGN) * Cfg::WN;
     const int l32 = lane & 31, hk = lane >> 5;
-    const int g = blockIdx.z / p.splitk;
+    const int g = fd_div(blockIdx.z, p.fd_splitk);
     const int ks = blockIdx.z - g * p.splitk; // which share of the K steps
     // Workgroups are handed to the 8 XCDs round-robin in launch order, and each
     // XCD has its own L2. Renumber so that an XCD owns one compact band of tiles
@@ -344,10 +346,10 @@ __global__ __launch_bounds__(Cfg::NT) void conv_plane_kernel(ConvParams p) {
         const unsigned L = bx + gridDim.x * by;
         const unsigned Lp = (L & 7) * p.xcd_chunk + (L >> 3);
         const unsigned mg = p.xcd_mg;
-        const unsigned band = Lp / (mg * gridDim.x);
+        const unsigned band = fd_div(Lp, p.fd_band);
         const unsigned in_band = Lp - band * mg * gridDim.x;
-        by = band * mg + in_band % mg;
-        bx = in_band / mg;
+        bx = fd_div(in_band, p.fd_mg);
+        by = band * mg + (in_band - bx * mg);
     }
     const int m0 = by * Cfg::BM;
     const int n0 = bx * Cfg::BN;
@@ -382,21 +384,45 @@ __global__ __launch_bounds__(Cfg::NT) void conv_plane_kernel(ConvParams p) {
             ow_[pp] = (int)ow * p.sw;
             pb[pp] = n * (unsigned)(p.C * THW) + ot * (unsigned)(p.st * HW) + oh_[pp] * p.W + ow_[pp];
         }
+        // Row i of wave w is row kl = w + NW * i of the B tile, i.e. channel kl / RS and
+        // tap kl % RS: the four waves fetch neighbouring taps of one channel at the
+        // same time, which the L1 likes. The padding tests depend on the tap only, and
+        // with the wave number as a compile-time constant (one copy of this block per
+        // wave) so do the tap and all of a row's offsets.
+        constexpr int SW = RS == 9 ? 3 : 1; // the host admits 3x3 and 1x1 planes only
+        constexpr int SR = RS / SW;
+        bool okr[PPL][SR], okc[PPL][SW];
 #pragma unroll
-        for (int i = 0; i < RPW; ++i) {
-            const int kl = wave + NW * i; // row of the B tile: (c_local, r, s)
-            const int cl = kl / RS, t = kl % RS;
-            constexpr int SW = RS == 9 ? 3 : 1; // the host admits 3x3 and 1x1 planes only
-            const int r = t / SW, s = t - r * SW;
-            const int rh = r * p.dh, sw_ = s * p.dw;
-            const unsigned roff = (unsigned)(cl * THW + rh * p.W + sw_);
+        for (int pp = 0; pp < PPL; ++pp) {
 #pragma unroll
-            for (int pp = 0; pp < PPL; ++pp) {
-                const bool ok = ((unsigned)(oh_[pp] + rh - p.ph) < (unsigned)p.H) &
-                                ((unsigned)(ow_[pp] + sw_ - p.pw) < (unsigned)p.W);
-                voffB[i][pp] = ok ? (pb[pp] + roff) * 4u : kOob;
-            }
+            for (int r = 0; r < SR; ++r)
+                okr[pp][r] = (unsigned)(oh_[pp] + r * p.dh - p.ph) < (unsigned)p.H;
+#pragma unroll
+            for (int s = 0; s < SW; ++s)
+                okc[pp][s] = (unsigned)(ow_[pp] + s * p.dw - p.pw) < (unsigned)p.W;
         }
+        auto rows_of = [&](auto wc) __attribute__((always_inline)) {
+            constexpr int WV = decltype(wc)::value;
+#pragma unroll
+            for (int i = 0; i < RPW; ++i) {
+                const int kl = WV + NW * i;
+                const int cl = kl / RS, t = kl % RS;
+                const int r = t / SW, s = t % SW;
+                const unsigned roff = (unsigned)(cl * THW + r * p.dh * p.W + s * p.dw);
+#pragma unroll
+                for (int pp = 0; pp < PPL; ++pp)
+                    voffB[i][pp] = (okr[pp][r] & okc[pp][s]) ? (pb[pp] + roff) * 4u : kOob;
+            }
+        };
+        static_assert(NW == 2 || NW == 4, "one copy of the row table per wave");
+        if (wave == 0)
+            rows_of(std::integral_constant<int, 0>{});
+        else if (wave == 1)
+            rows_of(std::integral_constant<int, 1>{});
+        else if (wave == 2)
+            rows_of(std::integral_constant<int, 2 % NW>{});
+        else
+            rows_of(std::integral_constant<int, 3 % NW>{});
     }
     // ---- per-thread invariants of the A loads
     unsigned voffA[NA];
@@ -439,8 +465,9 @@ __global__ __launch_bounds__(Cfg::NT) void conv_plane_kernel(ConvParams p) {
     // step counters of the prefetch stream: channel block and kt slice
     const int ncb = p.cpg / CB;
     const int nit_all = ncb * p.KT;
-    const int it_begin = (int)((long long)ks * nit_all / p.splitk);
-    const int it_end = (int)((long long)(ks + 1) * nit_all / p.splitk);
+    // ks * nit_all stays far below 2^31 (at most 64 splits)
+    const int it_begin = (int)fd_div((unsigned)(ks * nit_all), p.fd_splitk);
+    const int it_end = (int)fd_div((unsigned)((ks + 1) * nit_all), p.fd_splitk);
     const int nit = it_end - it_begin;
     int pcb = it_begin / p.KT, pq = it_begin - pcb * p.KT;
     auto advance_prefetch = [&]() __attribute__((always_inline)) {
@@ -633,7 +660,58 @@ __global__ __launch_bounds__(Cfg::NT) void conv_plane_kernel(ConvParams p) {
                                __HIP_MEMORY_SCOPE_AGENT); // ready for the next launch
     }
 
-    // epilogue: bias + activation, NC(T)HW store
+    const bool atomic = p.splitk > 1 && p.sk_mode == 1;
+    if (!atomic && p.vec_out) {
+        // epilogue through LDS: the tile is parked as [f][pixel] and leaves as 16-byte
+        // words, 256 or 512 contiguous bytes per filter row (the pixel count of an
+        // image is a multiple of 4 here, so a word never straddles two images)
+        constexpr int C_LD = Cfg::BN + 4;
+        constexpr int QPR = Cfg::BN / 4;   // words per tile row
+        constexpr int RPP = NT / QPR;      // tile rows per pass
+        __syncthreads();                   // every wave is done with the K loop's LDS
+#pragma unroll
+        for (int tm = 0; tm < TM; ++tm)
+#pragma unroll
+            for (int tn = 0; tn < TN; ++tn)
+#pragma unroll
+                for (int r = 0; r < 16; ++r)
+                    lds[(wm0 + tm * 32 + (r / 4) * 8 + hk * 4 + (r % 4)) * C_LD + wn0 + tn * 32 +
+                        l32] = acc[tm][tn][r];
+        __syncthreads();
+        const int q = tid % QPR, r0 = tid / QPR;
+        const int pix = n0 + 4 * q;
+        if (pix < p.NPIX) {
+            const unsigned n = fd_div(pix, p.fd_opix);
+            const unsigned rem = pix - n * p.OPIX;
+            float *__restrict__ yb =
+                p.y + (((long long)n * p.F + (long long)g * p.M) * p.OPIX + rem);
+            const float *__restrict__ bias =
+                (p.bias && p.bias_mode == 1) ? p.bias + g * p.M : nullptr;
+            float cb[4] = {0.f, 0.f, 0.f, 0.f};
+            if (p.bias && p.bias_mode == 2) {
+#pragma unroll
+                for (int j = 0; j < 4; ++j)
+                    cb[j] = p.bias[rem + j];
+            }
+#pragma unroll
+            for (int pass = 0; pass < Cfg::BM / RPP; ++pass) {
+                const int fl = r0 + pass * RPP;
+                const int f = m0 + fl;
+                if (f < p.M) {
+                    float4 v = *reinterpret_cast<const float4 *>(lds + fl * C_LD + 4 * q);
+                    const float bf = bias ? bias[f] : 0.f;
+                    v.x = apply_act(v.x + bf + cb[0], p.act);
+                    v.y = apply_act(v.y + bf + cb[1], p.act);
+                    v.z = apply_act(v.z + bf + cb[2], p.act);
+                    v.w = apply_act(v.w + bf + cb[3], p.act);
+                    *reinterpret_cast<float4 *>(yb + (unsigned)f * (unsigned)p.OPIX) = v;
+                }
+            }
+        }
+        return;
+    }
+
+    // epilogue: bias + activation (or the atomic add of a split), NC(T)HW store
 #pragma unroll
     for (int tn = 0; tn < TN; ++tn) {
         int pix = n0 + wn0 + tn * 32 + l32;
@@ -645,25 +723,30 @@ __global__ __launch_bounds__(Cfg::NT) void conv_plane_kernel(ConvParams p) {
         const float *__restrict__ bias =
             (p.bias && p.bias_mode == 1) ? p.bias + g * p.M : nullptr;
         const float colbias = (p.bias && p.bias_mode == 2) ? p.bias[rem] : 0.f;
+        if (atomic) {
+            // the output was initialised with the bias by a launch before this one;
+            // the activation runs in a launch after it
 #pragma unroll
-        for (int tm = 0; tm < TM; ++tm) {
+            for (int tm = 0; tm < TM; ++tm)
 #pragma unroll
-            for (int r = 0; r < 16; ++r) {
-                int f = m0 + wm0 + tm * 32 + (r / 4) * 8 + hk * 4 + (r % 4);
-                if (f < p.M) {
-                    float v = acc[tm][tn][r];
-                    float *dst = yb + (unsigned)f * (unsigned)p.OPIX;
-                    if (p.splitk > 1 && p.sk_mode == 1) {
-                        // the output was initialised with the bias by a launch before
-                        // this one; the activation runs in a launch after it
-                        unsafeAtomicAdd(dst, v);
-                    } else {
+                for (int r = 0; r < 16; ++r) {
+                    int f = m0 + wm0 + tm * 32 + (r / 4) * 8 + hk * 4 + (r % 4);
+                    if (f < p.M)
+                        unsafeAtomicAdd(yb + (unsigned)f * (unsigned)p.OPIX, acc[tm][tn][r]);
+                }
+        } else {
+#pragma unroll
+            for (int tm = 0; tm < TM; ++tm)
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    int f = m0 + wm0 + tm * 32 + (r / 4) * 8 + hk * 4 + (r % 4);
+                    if (f < p.M) {
+                        float v = acc[tm][tn][r];
                         if (bias)
                             v += bias[f];
-                        *dst = apply_act(v + colbias, p.act);
+                        yb[(unsigned)f * (unsigned)p.OPIX] = apply_act(v + colbias, p.act);
                     }
                 }
-            }
         }
     }
 }
@@ -803,6 +886,10 @@ int launch_plane_cfg(ConvParams p, hipStream_t stream) {
         if (rc)
             return rc;
     }
+    p.fd_splitk = make_fastdiv((unsigned)p.splitk);
+    p.fd_mg = make_fastdiv((unsigned)p.xcd_mg);
+    p.fd_band = make_fastdiv((unsigned)p.xcd_mg * grid.x);
+    p.vec_out = (p.OPIX % 4 == 0) && (((uintptr_t)p.y & 15) == 0);
     hipLaunchKernelGGL((conv_plane_kernel<Cfg, IS3D>), grid, dim3(Cfg::NT), lds_bytes, stream, p);
     int rc = check_launch("conv_plane_kernel");
     if (rc == PET_HIP_OK && splitk > 1 && p.sk_mode == 1 && p.act != PET_HIP_ACT_NONE)
