@@ -825,13 +825,28 @@ int launch_plane_cfg(ConvParams p, hipStream_t stream) {
         return -1; // caller falls back to the general kernel
     const long long tiles = tiles_for(p.M, p.NPIX, Cfg::BM, Cfg::BN, p.G);
     const int nit = (p.cpg / Cfg::CB) * p.KT;
-    // Split K when the tiles alone leave most CUs idle: each workgroup keeps at
-    // least two K steps, and about 256 workgroups are aimed for.
+    // Split K when the tiles alone leave CUs idle. A small cost model, in K steps of
+    // this tile: the busiest CU runs ceil(tiles * S / 256) workgroups one after the
+    // other (co-resident workgroups share its MFMA pipes), each of nit / S steps
+    // plus a fixed prologue + epilogue; a split launch pays two more small launches
+    // and its atomics contend S ways. Every workgroup keeps at least two steps.
     int splitk = 1;
-    if (tiles < 160 && nit >= 4) {
-        splitk = (int)std::min<long long>(nit / 2, (256 + tiles - 1) / tiles);
-        static const int max_env = getenv("PET_HIP_SPLITK_MAX") ? atoi(getenv("PET_HIP_SPLITK_MAX")) : 64;
-        splitk = std::max(1, std::min(splitk, max_env));
+    if (tiles < 256 && nit >= 4) {
+        static const int max_env =
+            getenv("PET_HIP_SPLITK_MAX") ? atoi(getenv("PET_HIP_SPLITK_MAX")) : 64;
+        const double scale = (double)(Cfg::BM * Cfg::BN) / (64.0 * 64.0);
+        const double c_fixed = 3.0 / scale, c_launches = 4.0 / scale, c_contend = 0.1 / scale;
+        double best = 0;
+        for (int S = 1; S <= std::min(nit / 2, max_env); ++S) {
+            const double rounds = (double)((tiles * S + 255) / 256);
+            double cost = rounds * ((nit + S - 1) / S + c_fixed);
+            if (S > 1)
+                cost += c_launches + c_contend * S;
+            if (S == 1 || cost < best) {
+                best = cost;
+                splitk = S;
+            }
+        }
     }
     static const int forced = getenv("PET_HIP_SPLITK") ? atoi(getenv("PET_HIP_SPLITK")) : 0;
     if (forced > 0)
