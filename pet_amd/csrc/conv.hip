@@ -36,6 +36,11 @@ struct ConvParams {
     int xcd_chunk; // plane kernel: tiles per XCD when the tile grid is dealt in bands (0: off)
     int xcd_mg;    // ... and how many M tiles wide a band is
     FastDiv fd_band, fd_mg, fd_splitk; // divisions by xcd_mg * grid.x, xcd_mg and splitk
+    // stream-K (plane kernel): a 1-D grid of sk_wgs workgroups shares tiles * nit K steps
+    // evenly; a workgroup runs its range as up to three segments of consecutive tiles
+    int streamk, sk_units, sk_tiles_m;
+    FastDiv fd_sk_wgs, fd_sk_nit, fd_sk_tm;
+    int atomic_out; // partial sums are added into y with float atomics
     int vec_out;   // plane kernel: OPIX % 4 == 0 and y 16-byte aligned: 16-byte output words
     int sk_mode;   // split-K: 0 partial tiles + ordered sum in one launch, 1 atomics into y
     float *ws;     // split-K: partial tiles, [tile][split][register][thread]
@@ -335,13 +340,38 @@ __global__ __launch_bounds__(Cfg::NT) void conv_plane_kernel(ConvParams p) {
     const int wm0 = (wave / Cfg::WGN) * Cfg::WM;
     const int wn0 = (wave % Cfg::WGN) * Cfg::WN;
     const int l32 = lane & 31, hk = lane >> 5;
-    const int g = fd_div(blockIdx.z, p.fd_splitk);
-    const int ks = blockIdx.z - g * p.splitk; // which share of the K steps
+    // stream-K: this workgroup's share of the tiles * nit K steps
+    unsigned seg_u = 0, seg_end = 0;
+    if (p.streamk) {
+        seg_u = fd_div(blockIdx.x * (unsigned)p.sk_units, p.fd_sk_wgs);
+        seg_end = fd_div((blockIdx.x + 1) * (unsigned)p.sk_units, p.fd_sk_wgs);
+        if (seg_u >= seg_end)
+            return;
+    }
+    for (bool first_seg = true;; first_seg = false) { // one pass unless stream-K
+    if (p.streamk && !first_seg)
+        __syncthreads(); // the previous segment's LDS reads are over
+    const int ncb = p.cpg / CB;
+    const int nit_all = ncb * p.KT;
+    int g = 0, ks = 0, it_begin, it_end;
+    unsigned bx, by;
+    if (p.streamk) {
+        const unsigned t = fd_div(seg_u, p.fd_sk_nit); // tile; M tiles vary fastest
+        it_begin = (int)(seg_u - t * nit_all);
+        it_end = min(nit_all, it_begin + (int)(seg_end - seg_u));
+        bx = fd_div(t, p.fd_sk_tm);
+        by = t - bx * p.sk_tiles_m;
+    } else {
+    g = fd_div(blockIdx.z, p.fd_splitk);
+    ks = blockIdx.z - g * p.splitk; // which share of the K steps
+    // ks * nit_all stays far below 2^31 (at most 64 splits)
+    it_begin = (int)fd_div((unsigned)(ks * nit_all), p.fd_splitk);
+    it_end = (int)fd_div((unsigned)((ks + 1) * nit_all), p.fd_splitk);
     // Workgroups are handed to the 8 XCDs round-robin in launch order, and each
     // XCD has its own L2. Renumber so that an XCD owns one compact band of tiles
     // (xcd_mg M tiles wide) instead of every eighth tile: its L2 then holds
     // 1/8th of the operands rather than all the filters.
-    unsigned bx = blockIdx.x, by = blockIdx.y;
+    bx = blockIdx.x, by = blockIdx.y;
     if (p.xcd_chunk) {
         const unsigned L = bx + gridDim.x * by;
         const unsigned Lp = (L & 7) * p.xcd_chunk + (L >> 3);
@@ -350,6 +380,7 @@ __global__ __launch_bounds__(Cfg::NT) void conv_plane_kernel(ConvParams p) {
         const unsigned in_band = Lp - band * mg * gridDim.x;
         bx = fd_div(in_band, p.fd_mg);
         by = band * mg + (in_band - bx * mg);
+    }
     }
     const int m0 = by * Cfg::BM;
     const int n0 = bx * Cfg::BN;
@@ -463,11 +494,6 @@ __global__ __launch_bounds__(Cfg::NT) void conv_plane_kernel(ConvParams p) {
                 acc[tm][tn][r] = 0.f;
 
     // step counters of the prefetch stream: channel block and kt slice
-    const int ncb = p.cpg / CB;
-    const int nit_all = ncb * p.KT;
-    // ks * nit_all stays far below 2^31 (at most 64 splits)
-    const int it_begin = (int)fd_div((unsigned)(ks * nit_all), p.fd_splitk);
-    const int it_end = (int)fd_div((unsigned)((ks + 1) * nit_all), p.fd_splitk);
     const int nit = it_end - it_begin;
     int pcb = it_begin / p.KT, pq = it_begin - pcb * p.KT;
     auto advance_prefetch = [&]() __attribute__((always_inline)) {
@@ -660,7 +686,7 @@ __global__ __launch_bounds__(Cfg::NT) void conv_plane_kernel(ConvParams p) {
                                __HIP_MEMORY_SCOPE_AGENT); // ready for the next launch
     }
 
-    const bool atomic = p.splitk > 1 && p.sk_mode == 1;
+    const bool atomic = p.atomic_out;
     if (!atomic && p.vec_out) {
         // epilogue through LDS: the tile is parked as [f][pixel] and leaves as 16-byte
         // words, 256 or 512 contiguous bytes per filter row (the pixel count of an
@@ -749,6 +775,12 @@ __global__ __launch_bounds__(Cfg::NT) void conv_plane_kernel(ConvParams p) {
                 }
         }
     }
+    if (!p.streamk)
+        break;
+    seg_u += it_end - it_begin;
+    if (seg_u >= seg_end)
+        break;
+    } // segments
 }
 
 using Cfg128x128 = TileCfg<128, 128, 16, 2, 2>;
@@ -831,12 +863,12 @@ int launch_plane_cfg(ConvParams p, hipStream_t stream) {
     // plus a fixed prologue + epilogue; a split launch pays two more small launches
     // and its atomics contend S ways. Every workgroup keeps at least two steps.
     int splitk = 1;
+    const double scale = (double)(Cfg::BM * Cfg::BN) / (64.0 * 64.0);
+    const double c_fixed = 3.0 / scale, c_launches = 4.0 / scale, c_contend = 0.1 / scale;
+    double best = ((tiles + 255) / 256) * (nit + c_fixed); // S = 1
     if (tiles < 256 && nit >= 4) {
         static const int max_env =
             getenv("PET_HIP_SPLITK_MAX") ? atoi(getenv("PET_HIP_SPLITK_MAX")) : 64;
-        const double scale = (double)(Cfg::BM * Cfg::BN) / (64.0 * 64.0);
-        const double c_fixed = 3.0 / scale, c_launches = 4.0 / scale, c_contend = 0.1 / scale;
-        double best = 0;
         for (int S = 1; S <= std::min(nit / 2, max_env); ++S) {
             const double rounds = (double)((tiles * S + 255) / 256);
             double cost = rounds * ((nit + S - 1) / S + c_fixed);
@@ -853,6 +885,28 @@ int launch_plane_cfg(ConvParams p, hipStream_t stream) {
         splitk = std::min(forced, nit);
     if ((long long)p.G * splitk > 65535)
         splitk = 1;
+    // Stream-K instead: 256 (64x128 tiles) or 512 workgroups share the tiles * nit K
+    // steps evenly, so no CU waits for a last, partly filled round of tiles. All
+    // sums go into y as float atomics (initialising launch before, activation after).
+    // Taken when the model sees a tenth less work on the busiest CU.
+    p.streamk = 0;
+    {
+        static const int sk_env = getenv("PET_HIP_STREAMK") ? atoi(getenv("PET_HIP_STREAMK")) : -1;
+        const long long units = tiles * nit;
+        const int wgs = Cfg::BM * Cfg::BN >= 64 * 128 ? 256 : 512;
+        const double cost_sk = (double)units / 256 + 2 * c_fixed + c_launches;
+        const bool fits = p.G == 1 && units * (wgs + 1) < (1ll << 31) && units >= 2 * wgs &&
+                          Cfg::BM >= 64 && !deterministic();
+        if (fits && forced <= 0 && (sk_env == 1 || (sk_env != 0 && cost_sk < 0.9 * best))) {
+            p.streamk = 1;
+            splitk = 1;
+            p.sk_units = (int)units;
+            p.sk_tiles_m = (p.M + Cfg::BM - 1) / Cfg::BM;
+            p.fd_sk_wgs = make_fastdiv((unsigned)wgs);
+            p.fd_sk_nit = make_fastdiv((unsigned)nit);
+            p.fd_sk_tm = make_fastdiv((unsigned)p.sk_tiles_m);
+        }
+    }
     // Float atomics into the output (an initialising launch before, the activation
     // in a launch after) are the faster way by 10-30% on small layers: the ordered
     // single-launch sum adds three dependent round trips through memory to every
@@ -870,13 +924,14 @@ int launch_plane_cfg(ConvParams p, hipStream_t stream) {
             splitk = 1;
     }
     p.splitk = splitk;
+    p.atomic_out = p.streamk || (splitk > 1 && p.sk_mode == 1);
     dim3 grid((p.NPIX + Cfg::BN - 1) / Cfg::BN, (p.M + Cfg::BM - 1) / Cfg::BM, p.G * splitk);
     // XCD bands: only when every z plane starts on XCD 0 and has several tiles per XCD
     p.xcd_chunk = 0;
     p.xcd_mg = 1;
     static const bool xcd_off = getenv("PET_HIP_XCD") && atoi(getenv("PET_HIP_XCD")) == 0;
     const unsigned plane_tiles = grid.x * grid.y;
-    if (!xcd_off && plane_tiles % 8 == 0 && plane_tiles >= 64) {
+    if (!xcd_off && !p.streamk && plane_tiles % 8 == 0 && plane_tiles >= 64) {
         const unsigned chunk = plane_tiles / 8;
         // bytes an XCD pulls for a band mg tiles wide: its filters + its pixels
         double best = 0;
@@ -892,7 +947,7 @@ int launch_plane_cfg(ConvParams p, hipStream_t stream) {
         }
         p.xcd_chunk = (int)chunk;
     }
-    if (splitk > 1 && p.sk_mode == 1) {
+    if (p.atomic_out) {
         const size_t total = (size_t)p.NPIX * p.F;
         unsigned igrid = (unsigned)std::min<size_t>((total + 255) / 256, 4096);
         hipLaunchKernelGGL(splitk_init_kernel, dim3(igrid), dim3(256), 0, stream, p.y, p.bias,
@@ -905,9 +960,11 @@ int launch_plane_cfg(ConvParams p, hipStream_t stream) {
     p.fd_mg = make_fastdiv((unsigned)p.xcd_mg);
     p.fd_band = make_fastdiv((unsigned)p.xcd_mg * grid.x);
     p.vec_out = (p.OPIX % 4 == 0) && (((uintptr_t)p.y & 15) == 0);
+    if (p.streamk)
+        grid = dim3(Cfg::BM * Cfg::BN >= 64 * 128 ? 256 : 512, 1, 1);
     hipLaunchKernelGGL((conv_plane_kernel<Cfg, IS3D>), grid, dim3(Cfg::NT), lds_bytes, stream, p);
     int rc = check_launch("conv_plane_kernel");
-    if (rc == PET_HIP_OK && splitk > 1 && p.sk_mode == 1 && p.act != PET_HIP_ACT_NONE)
+    if (rc == PET_HIP_OK && p.atomic_out && p.act != PET_HIP_ACT_NONE)
         rc = pet_hip_activation(p.y, p.y, (size_t)p.NPIX * p.F, p.act, (pet_hip_stream_t)stream);
     return rc;
 }
