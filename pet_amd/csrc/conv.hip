@@ -318,7 +318,7 @@ __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void *base) {
 
 constexpr unsigned kOob = 0x80000000u; // voffset that the range check rejects
 
-template <class Cfg, bool IS3D>
+template <class Cfg, bool IS3D, bool SK>
 __global__ __launch_bounds__(Cfg::NT) void conv_plane_kernel(ConvParams p) {
     extern __shared__ __attribute__((aligned(16))) float lds[];
     constexpr int KH = Cfg::KH, TM = Cfg::TM, TN = Cfg::TN, RS = Cfg::RS, CB = Cfg::CB;
@@ -342,20 +342,20 @@ __global__ __launch_bounds__(Cfg::NT) void conv_plane_kernel(ConvParams p) {
     const int l32 = lane & 31, hk = lane >> 5;
     // stream-K: this workgroup's share of the tiles * nit K steps
     unsigned seg_u = 0, seg_end = 0;
-    if (p.streamk) {
+    if (SK) {
         seg_u = fd_div(blockIdx.x * (unsigned)p.sk_units, p.fd_sk_wgs);
         seg_end = fd_div((blockIdx.x + 1) * (unsigned)p.sk_units, p.fd_sk_wgs);
         if (seg_u >= seg_end)
             return;
     }
     for (bool first_seg = true;; first_seg = false) { // one pass unless stream-K
-    if (p.streamk && !first_seg)
+    if (SK && !first_seg)
         __syncthreads(); // the previous segment's LDS reads are over
     const int ncb = p.cpg / CB;
     const int nit_all = ncb * p.KT;
     int g = 0, ks = 0, it_begin, it_end;
     unsigned bx, by;
-    if (p.streamk) {
+    if (SK) {
         const unsigned t = fd_div(seg_u, p.fd_sk_nit); // tile; M tiles vary fastest
         it_begin = (int)(seg_u - t * nit_all);
         it_end = min(nit_all, it_begin + (int)(seg_end - seg_u));
@@ -775,7 +775,7 @@ __global__ __launch_bounds__(Cfg::NT) void conv_plane_kernel(ConvParams p) {
                 }
         }
     }
-    if (!p.streamk)
+    if (!SK)
         break;
     seg_u += it_end - it_begin;
     if (seg_u >= seg_end)
@@ -844,13 +844,25 @@ __global__ __launch_bounds__(256) void splitk_init_kernel(float *__restrict__ y,
     }
 }
 
+// Stream-K is instantiated for the 3x3 tiles of 64 rows only (it needs its own copy of the
+// kernel: the segment loop's bookkeeping would otherwise push scalars of every launch
+// out of the SGPR file).
+template <class Cfg>
+constexpr bool has_streamk = Cfg::BM >= 64 && Cfg::RS == 9;
+
 template <class Cfg, bool IS3D>
 int launch_plane_cfg(ConvParams p, hipStream_t stream) {
     const size_t lds_bytes = 2 * (size_t)Cfg::STAGE * sizeof(float);
     static int attr_status = [&] {
         hipError_t e = hipFuncSetAttribute(
-            reinterpret_cast<const void *>(&conv_plane_kernel<Cfg, IS3D>),
+            reinterpret_cast<const void *>(&conv_plane_kernel<Cfg, IS3D, false>),
             hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
+        if constexpr (has_streamk<Cfg>) {
+            if (e == hipSuccess)
+                e = hipFuncSetAttribute(
+                    reinterpret_cast<const void *>(&conv_plane_kernel<Cfg, IS3D, true>),
+                    hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
+        }
         return e == hipSuccess ? 0 : 1;
     }();
     if (attr_status)
@@ -896,7 +908,7 @@ int launch_plane_cfg(ConvParams p, hipStream_t stream) {
         const int wgs = Cfg::BM * Cfg::BN >= 64 * 128 ? 256 : 512;
         const double cost_sk = (double)units / 256 + 2 * c_fixed + c_launches;
         const bool fits = p.G == 1 && units * (wgs + 1) < (1ll << 31) && units >= 2 * wgs &&
-                          Cfg::BM >= 64 && !deterministic();
+                          has_streamk<Cfg> && !deterministic();
         if (fits && forced <= 0 && (sk_env == 1 || (sk_env != 0 && cost_sk < 0.9 * best))) {
             p.streamk = 1;
             splitk = 1;
@@ -960,9 +972,16 @@ int launch_plane_cfg(ConvParams p, hipStream_t stream) {
     p.fd_mg = make_fastdiv((unsigned)p.xcd_mg);
     p.fd_band = make_fastdiv((unsigned)p.xcd_mg * grid.x);
     p.vec_out = (p.OPIX % 4 == 0) && (((uintptr_t)p.y & 15) == 0);
-    if (p.streamk)
-        grid = dim3(Cfg::BM * Cfg::BN >= 64 * 128 ? 256 : 512, 1, 1);
-    hipLaunchKernelGGL((conv_plane_kernel<Cfg, IS3D>), grid, dim3(Cfg::NT), lds_bytes, stream, p);
+    if constexpr (has_streamk<Cfg>) {
+        if (p.streamk) {
+            grid = dim3(Cfg::BM * Cfg::BN >= 64 * 128 ? 256 : 512, 1, 1);
+            hipLaunchKernelGGL((conv_plane_kernel<Cfg, IS3D, true>), grid, dim3(Cfg::NT), lds_bytes,
+                               stream, p);
+        }
+    }
+    if (!p.streamk)
+        hipLaunchKernelGGL((conv_plane_kernel<Cfg, IS3D, false>), grid, dim3(Cfg::NT), lds_bytes,
+                           stream, p);
     int rc = check_launch("conv_plane_kernel");
     if (rc == PET_HIP_OK && p.atomic_out && p.act != PET_HIP_ACT_NONE)
         rc = pet_hip_activation(p.y, p.y, (size_t)p.NPIX * p.F, p.act, (pet_hip_stream_t)stream);
