@@ -136,6 +136,21 @@ def test_conv2d_split_contraction_both_modes(ops, case):
         abi.call("pet_hip_set_deterministic", 0)
 
 
+def test_conv_shapes_that_take_the_stream_k_path(ops):
+    """Tile counts that quantise badly against 256 CUs (300 tiles of 64x128 in 2-D,
+    280 tiles of 64x64 in 3-D) run as a fixed grid of workgroups sharing the K steps,
+    with float atomics into the output: exact on small integers whatever the order."""
+    rng = np.random.default_rng(21)
+    x, wt, b = ints(rng, (1, 256, 160, 240)), ints(rng, (64, 256, 3, 3)), ints(rng, (64,))
+    ref = oracle.bias_act(oracle.conv2d(x, wt, 1, 1), b, "relu")
+    got = host(ops.conv2d(dev(x), dev(wt), 1, 1, bias=dev(b), act="relu"))
+    np.testing.assert_array_equal(got, ref)
+    x3, w3 = ints(rng, (1, 64, 8, 40, 56)), ints(rng, (64, 64, 3, 3, 3))
+    ref3 = oracle.conv3d(x3, w3, (1, 1, 1))
+    got3 = host(ops.conv3d(dev(x3), dev(w3), (1, 1, 1)))
+    np.testing.assert_array_equal(got3, ref3)
+
+
 def test_conv2d_rejects_bad_groups(ops):
     from pet_amd import abi
     x = torch.zeros((1, 4, 5, 5), device="cuda")
