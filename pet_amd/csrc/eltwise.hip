@@ -167,7 +167,13 @@ __global__ __launch_bounds__(256) void global_avgpool_kernel(const float *__rest
         y[plane] = acc / (float)hw;
 }
 
-// One wave per row; rows of any length.
+// One wave per row. Rows of up to 64 * kRowRegs elements are read once into
+// registers with all loads in flight (a row of BERT's 768 columns is 12 loads per
+// lane; read three times one load after the other it costs 36 round trips);
+// longer rows take the streaming variant. Both add in the same order.
+constexpr int kRowRegs = 32;
+
+template <bool RESIDENT>
 __global__ __launch_bounds__(256) void softmax_kernel(const float *__restrict__ x,
                                                       float *__restrict__ y, size_t rows,
                                                       size_t cols) {
@@ -177,6 +183,36 @@ __global__ __launch_bounds__(256) void softmax_kernel(const float *__restrict__ 
         return;
     const float *xp = x + row * cols;
     float *yp = y + row * cols;
+    if (RESIDENT) {
+        float v[kRowRegs];
+#pragma unroll
+        for (int i = 0; i < kRowRegs; ++i) {
+            const size_t j = lane + 64 * (size_t)i;
+            v[i] = j < cols ? xp[j] : -INFINITY;
+        }
+        float mx = -INFINITY;
+#pragma unroll
+        for (int i = 0; i < kRowRegs; ++i)
+            mx = fmaxf(mx, v[i]);
+        mx = wave_max(mx);
+        float sum = 0.f;
+#pragma unroll
+        for (int i = 0; i < kRowRegs; ++i) {
+            const size_t j = lane + 64 * (size_t)i;
+            v[i] = expf(v[i] - mx);
+            if (j < cols)
+                sum += v[i];
+        }
+        sum = wave_sum(sum);
+        const float inv = 1.f / sum;
+#pragma unroll
+        for (int i = 0; i < kRowRegs; ++i) {
+            const size_t j = lane + 64 * (size_t)i;
+            if (j < cols)
+                yp[j] = v[i] * inv;
+        }
+        return;
+    }
     float mx = -INFINITY;
     for (size_t j = lane; j < cols; j += 64)
         mx = fmaxf(mx, xp[j]);
@@ -190,6 +226,7 @@ __global__ __launch_bounds__(256) void softmax_kernel(const float *__restrict__ 
         yp[j] = expf(xp[j] - mx) * inv;
 }
 
+template <bool RESIDENT>
 __global__ __launch_bounds__(256) void layernorm_kernel(const float *__restrict__ x,
                                                         const float *__restrict__ gamma,
                                                         const float *__restrict__ beta,
@@ -201,6 +238,44 @@ __global__ __launch_bounds__(256) void layernorm_kernel(const float *__restrict_
         return;
     const float *xp = x + row * cols;
     float *yp = y + row * cols;
+    if (RESIDENT) {
+        float v[kRowRegs], gm[kRowRegs], bt[kRowRegs];
+#pragma unroll
+        for (int i = 0; i < kRowRegs; ++i) {
+            const size_t j = lane + 64 * (size_t)i;
+            const bool in = j < cols;
+            v[i] = in ? xp[j] : 0.f;
+            gm[i] = (in && gamma) ? gamma[j] : 1.f;
+            bt[i] = (in && beta) ? beta[j] : 0.f;
+        }
+        float s = 0.f;
+#pragma unroll
+        for (int i = 0; i < kRowRegs; ++i)
+            if (lane + 64 * (size_t)i < cols)
+                s += v[i];
+        const float mean = wave_sum(s) / (float)cols;
+        float q = 0.f;
+#pragma unroll
+        for (int i = 0; i < kRowRegs; ++i)
+            if (lane + 64 * (size_t)i < cols) {
+                const float d = v[i] - mean;
+                q += d * d;
+            }
+        const float inv = rsqrtf(wave_sum(q) / (float)cols + eps);
+#pragma unroll
+        for (int i = 0; i < kRowRegs; ++i) {
+            const size_t j = lane + 64 * (size_t)i;
+            if (j < cols) {
+                float o = (v[i] - mean) * inv;
+                if (gamma)
+                    o *= gm[i];
+                if (beta)
+                    o += bt[i];
+                yp[j] = o;
+            }
+        }
+        return;
+    }
     float s = 0.f;
     for (size_t j = lane; j < cols; j += 64)
         s += xp[j];
@@ -353,8 +428,12 @@ int pet_hip_softmax(const float *x, float *y, size_t rows, size_t cols, pet_hip_
         return set_error(PET_HIP_ERR_INVALID, "null pointer");
     if ((rows + 3) / 4 >= (1ull << 31))
         return set_error(PET_HIP_ERR_UNSUPPORTED, "too many rows");
-    hipLaunchKernelGGL(softmax_kernel, dim3((unsigned)((rows + 3) / 4)), dim3(256), 0,
-                       as_stream(stream), x, y, rows, cols);
+    if (cols <= 64 * (size_t)kRowRegs)
+        hipLaunchKernelGGL(softmax_kernel<true>, dim3((unsigned)((rows + 3) / 4)), dim3(256), 0,
+                           as_stream(stream), x, y, rows, cols);
+    else
+        hipLaunchKernelGGL(softmax_kernel<false>, dim3((unsigned)((rows + 3) / 4)), dim3(256), 0,
+                           as_stream(stream), x, y, rows, cols);
     return check_launch("softmax_kernel");
 }
 
@@ -367,8 +446,12 @@ int pet_hip_layernorm(const float *x, const float *gamma, const float *beta, flo
         return set_error(PET_HIP_ERR_INVALID, "null pointer");
     if ((rows + 3) / 4 >= (1ull << 31))
         return set_error(PET_HIP_ERR_UNSUPPORTED, "too many rows");
-    hipLaunchKernelGGL(layernorm_kernel, dim3((unsigned)((rows + 3) / 4)), dim3(256), 0,
-                       as_stream(stream), x, gamma, beta, y, rows, cols, eps);
+    if (cols <= 64 * (size_t)kRowRegs)
+        hipLaunchKernelGGL(layernorm_kernel<true>, dim3((unsigned)((rows + 3) / 4)), dim3(256), 0,
+                           as_stream(stream), x, gamma, beta, y, rows, cols, eps);
+    else
+        hipLaunchKernelGGL(layernorm_kernel<false>, dim3((unsigned)((rows + 3) / 4)), dim3(256), 0,
+                           as_stream(stream), x, gamma, beta, y, rows, cols, eps);
     return check_launch("layernorm_kernel");
 }
 

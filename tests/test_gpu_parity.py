@@ -438,6 +438,19 @@ def test_activation_pool_softmax_layernorm(ops):
                                oracle.layernorm(h, g, be), rtol=1e-4, atol=1e-5)
 
 
+@pytest.mark.parametrize("cols", [1, 63, 65, 700, 2048, 2049, 5000])
+def test_softmax_layernorm_row_lengths(ops, cols):
+    """Rows up to 2048 elements live in registers, longer ones stream; ragged
+    lengths on both sides of the switch."""
+    rng = np.random.default_rng(cols)
+    s = rng.standard_normal((5, cols)).astype(np.float32)
+    np.testing.assert_allclose(host(ops.softmax(dev(s))), oracle.softmax(s), rtol=1e-5, atol=1e-7)
+    g = rng.standard_normal(cols).astype(np.float32)
+    be = rng.standard_normal(cols).astype(np.float32)
+    np.testing.assert_allclose(host(ops.layernorm(dev(s), dev(g), dev(be))),
+                               oracle.layernorm(s, g, be), rtol=1e-4, atol=1e-5)
+
+
 def test_config1_original_vs_corrected_transform(ops):
     # BASELINE config 1: conv 1x64x56x56, 3x3 p1, U[-1,1] from seed 0 (x then w);
     # original op vs H2N(halo 1) -> conv -> N2H(drop 1).
