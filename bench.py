@@ -231,7 +231,7 @@ def main():
     dom_flop = conv_flop(DIL * DIL, 512, hs, hs, 512, 3, 3)
     dom_ms = conv_ms[0]
     achieved = dom_flop / dom_ms / 1e9
-    roofline = {"bound": "mfma", "kernel": "conv_plane_kernel<64x128, RS=9, CB=8> (512->512, 4x32x32, 3x3, ReLU)",
+    roofline = {"bound": "mfma", "kernel": "conv_plane_kernel<64x64, RS=9, CB=8> (512->512, 4x32x32, 3x3, ReLU)",
                 "achieved": achieved, "peak": MFMA_FP32_PEAK_TFLOPS, "unit": "TFLOP/s",
                 "frac": achieved / MFMA_FP32_PEAK_TFLOPS,
                 "traffic": DOMINANT_TRAFFIC_BYTES, "traffic_unit": "bytes per launch",

@@ -332,7 +332,6 @@ __global__ __launch_bounds__(Cfg::NT) void conv_plane_kernel(ConvParams p) {
     constexpr int NRA = TM * (KH / 4);
     constexpr int NR = NRA + KH;                       // R pieces
     constexpr int NG = NA + RPW;                       // G pieces
-    constexpr int NPOST = NR + NG;                     // second half
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -993,14 +992,17 @@ int launch_plane(const ConvParams &p, bool is3d, hipStream_t stream) {
     using C64x128 = PlaneCfg<64, 128, 2, 2, RS, CB>;
     using C64x64 = PlaneCfg<64, 64, 2, 2, RS, CB>;
     using C32x64 = PlaneCfg<32, 64, 1, 2, RS, CB>;
-    // 64x128 when it alone fills the GPU; otherwise 64x64 (two workgroups fit a
-    // CU, and split-K supplies the missing parallelism); 32x64 for M <= 32
-    // 64x128 tiles (one workgroup per CU) once they fill the chip and the K loop
-    // is long; with 16 steps or fewer two co-resident 64x64 workgroups hide each
-    // other's prologue and epilogue
+    // 64x64 tiles, two workgroups to a CU (each hides the other's prologue, epilogue and
+    // barrier waits), measured equal or better than one 64x128 workgroup per CU up to
+    // a few rounds of tiles; beyond that 64x128 wins through its lower LDS traffic per
+    // MFMA (2048 tiles of 64x128 with 8 steps: 212 vs 230 us). 32x64 for M <= 32.
+    // The 3-D kernel carries more registers and is the exception: it keeps 64x128 once
+    // those tiles fill the chip and the K loop is long (R3D-18 layer 1: 152 vs 165 us).
     int tile = p.M > 32 ? 1 : 2;
     const int nit = (p.cpg / CB) * p.KT;
-    if (p.M > 32 && tiles_for(p.M, p.NPIX, 64, 128, p.G) >= 200 && nit > 16)
+    if (p.M > 32 && !is3d && tiles_for(p.M, p.NPIX, 64, 64, p.G) > 2048)
+        tile = 0;
+    if (p.M > 32 && is3d && tiles_for(p.M, p.NPIX, 64, 128, p.G) >= 200 && nit > 16)
         tile = 0;
     if (forced_tile() >= 0)
         tile = forced_tile() % 3;
