@@ -36,11 +36,11 @@ def conv_flop(n, f, oh, ow, c, r, s):
 
 
 # HBM-side bytes one launch of the dominant kernel moves, from rocprofv3 --pmc runs of
-# `bench.py --dominant-only 20`: FETCH_SIZE 25952.0 KiB per dispatch scaled by 1.9989
+# `bench.py --dominant-only 20`: FETCH_SIZE 25818.6 KiB per dispatch scaled by 1.9989
 # (what a 256 MiB plain copy reads on that counter), WRITE_SIZE 8192.0 KiB scaled by 0.9996.
 # A counter cannot be read from inside this process; the summary is
-# profiles/conv_plane_64x128_rs9_c2_layer_512to512.txt.
-DOMINANT_TRAFFIC_BYTES = int((25952.0 * 1.9989 + 8192.0 * 0.9996) * 1024)
+# profiles/conv_plane_64x64_rs9_c2_layer_512to512.txt.
+DOMINANT_TRAFFIC_BYTES = int((25818.6 * 1.9989 + 8192.0 * 0.9996) * 1024)
 
 
 def main():
