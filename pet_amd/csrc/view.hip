@@ -46,9 +46,13 @@ struct DirectParams {
     long long os[PET_HIP_MAX_RANK], sq[PET_HIP_MAX_RANK], sr[PET_HIP_MAX_RANK];
     long long ibase, obase;
     unsigned total; // number of work items (elements / VEC)
+    int inner_contig; // the innermost dim is contiguous in the input and has no div level
 };
 
 typedef float vf4 __attribute__((ext_vector_type(4)));
+// the same four floats at 4-byte alignment: the hardware takes a 16-byte load at any
+// dword address (the compiler itself emits one for this type)
+typedef float vf4u __attribute__((ext_vector_type(4), aligned(4)));
 
 // Streaming (non-temporal) accesses for tensors too large to stay in cache.
 template <bool NT>
@@ -190,6 +194,19 @@ __global__ __launch_bounds__(256) void view_gather4_kernel(const float *__restri
         unsigned inner, io_outer;
         bool ok_outer = live;
         decode_outer(p, e0, inner, io_outer, ok_outer);
+        // the common case: all four inside one row and inside its window, the row
+        // contiguous in the input -> one 16-byte load at whatever dword alignment
+        const int L = p.rank - 1;
+        if (p.inner_contig && ok_outer && inner + 3 < ext_inner && (int)inner >= p.lo[L] &&
+            (int)inner + 3 < p.hi[L]) {
+            const vf4u *src = reinterpret_cast<const vf4u *>(x + (io_outer + inner * (unsigned)p.sr[L]));
+            const vf4u w = NT ? __builtin_nontemporal_load(src) : *src;
+            v[u][0] = w.x;
+            v[u][1] = w.y;
+            v[u][2] = w.z;
+            v[u][3] = w.w;
+            continue;
+        }
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
             if (j > 0 && ++inner == ext_inner) { // next row: decode afresh
@@ -901,7 +918,7 @@ int launch_view_copy(const float *x, float *y, ViewDesc v, long long in_elems,
                     };
                     const bool vin = vec_ok(tin, true), vout = vec_ok(tout, false);
                     const bool nt = stream_sized(total);
-                    const dim3 grid((unsigned)ngroups), block(256);
+                    const dim3 grid((unsigned)ngroups);
                     const size_t lds_bytes =
                         (size_t)(p.tile_elems + p.tile_elems / 32 + 1) * sizeof(float);
 #define PET_TILED(VI, VO, NTF) launch_tiled<VI, VO, NTF>(grid, lds_bytes, stream, x, y, p)
@@ -972,6 +989,7 @@ int launch_view_copy(const float *x, float *y, ViewDesc v, long long in_elems,
             expect *= c.d[i].ext;
         }
         if (dense) {
+            p.inner_contig = c.d[L].sr == 1 && c.d[L].m >= c.d[L].ext;
             p.total = (unsigned)(total / 4);
             const bool nt = stream_sized(total);
             const dim3 grid((unsigned)((p.total + 1023) / 1024)), block(256);
