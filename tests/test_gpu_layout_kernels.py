@@ -150,3 +150,27 @@ def test_halo_chain_on_width(ops):
     ref = oracle.trans_chain(x, chain)
     got = host(ops.trans_chain(dev(x), chain))
     assert got.shape == ref.shape and got.tobytes() == ref.tobytes()
+
+
+def test_random_permutes_pads_slices_against_numpy(ops):
+    """300 seeded random cases across the kernel-selection boundaries: ranks 2-6,
+    extents mixing multiples of 4, of 2 and odd numbers, any permutation; then a
+    random pad and the slice that undoes it. Expected values from numpy itself."""
+    rng = np.random.default_rng(2024)
+    pool = [1, 2, 3, 4, 5, 6, 7, 8, 12, 16, 17, 24, 32, 33, 64]
+    for case in range(300):
+        rank = int(rng.integers(2, 7))
+        dims = [int(rng.choice(pool)) for _ in range(rank)]
+        while np.prod(dims) > 1 << 18:
+            dims[int(rng.integers(0, rank))] = 2
+        perm = [int(v) for v in rng.permutation(rank)]
+        x = iota(dims)
+        ref = np.ascontiguousarray(x.transpose(perm))
+        got = host(ops.permute_flat(dev(x), dims, perm))
+        assert got.tobytes() == ref.tobytes(), ("permute", case, dims, perm)
+        begin = [int(rng.integers(0, 3)) for _ in range(rank)]
+        end = [int(rng.integers(0, 3)) for _ in range(rank)]
+        refp = np.pad(x, list(zip(begin, end)))
+        p = ops.pad(dev(x), begin, end)
+        assert host(p).tobytes() == refp.tobytes(), ("pad", case, dims, begin, end)
+        assert host(ops.slice_(p, begin, end)).tobytes() == x.tobytes(), ("slice", case, dims)

@@ -151,6 +151,55 @@ def test_conv_shapes_that_take_the_stream_k_path(ops):
     np.testing.assert_array_equal(got3, ref3)
 
 
+def test_conv_random_configurations_integer_tier(ops):
+    """80 seeded random 2-D and 3-D convolutions (channels on and off the multiples
+    of 8 that select the plane kernel, groups, strides, dilations, paddings, ragged
+    sizes, bias + ReLU), bit-exact against the oracle on small integers."""
+    rng = np.random.default_rng(77)
+    for case in range(80):
+        groups = int(rng.choice([1, 1, 1, 2, 4]))
+        cpg = int(rng.choice([1, 3, 8, 8, 16, 24, 32]))
+        fpg = int(rng.choice([1, 5, 8, 32, 64, 72]))
+        c, f = cpg * groups, fpg * groups
+        k = int(rng.choice([1, 3, 3, 3, 5]))
+        st, dl = int(rng.choice([1, 1, 2])), int(rng.choice([1, 1, 2]))
+        pd = int(rng.integers(0, 3))
+        n = int(rng.integers(1, 4))
+        h, w = int(rng.integers(5, 23)), int(rng.integers(5, 23))
+        if (h + 2 * pd - dl * (k - 1) - 1) < 0 or (w + 2 * pd - dl * (k - 1) - 1) < 0:
+            continue
+        b = ints(rng, (f,))
+        if case % 4 == 3:  # 3-D
+            t = int(rng.integers(2, 6))
+            kt = int(rng.choice([1, 3]))
+            if t + 2 * pd - dl * (kt - 1) - 1 < 0:
+                continue
+            x, wt = ints(rng, (n, c, t, h, w)), ints(rng, (f, cpg, kt, k, k))
+            ref = oracle.bias_act(oracle.conv3d(x, wt, (pd, pd, pd), (st, st, st), (dl, dl, dl)), b, "relu")
+            got = host(ops.conv3d(dev(x), dev(wt), (pd, pd, pd), (st, st, st), (dl, dl, dl),
+                                  bias=dev(b), act="relu"))
+        else:
+            x, wt = ints(rng, (n, c, h, w)), ints(rng, (f, cpg, k, k))
+            ref = oracle.bias_act(oracle.conv2d(x, wt, pd, pd, st, st, dl, dl), b, "relu")
+            got = host(ops.conv2d(dev(x), dev(wt), pd, pd, st, st, dl, dl, bias=dev(b), act="relu"))
+        assert got.shape == ref.shape, (case, got.shape, ref.shape)
+        assert np.array_equal(got, ref), (case, n, c, h, w, f, cpg, k, st, dl, pd)
+
+
+def test_matmul_random_configurations_integer_tier(ops):
+    rng = np.random.default_rng(78)
+    for case in range(60):
+        bsz = int(rng.choice([1, 2, 3, 12]))
+        m, n, k = (int(rng.choice([1, 7, 32, 64, 96, 128, 200])) for _ in range(3))
+        tA, tB = bool(rng.integers(0, 2)), bool(rng.integers(0, 2))
+        A, B = ints(rng, (bsz, m, k)), ints(rng, (bsz, k, n))
+        ref = oracle.matmul(A, B)
+        dA = dev(np.ascontiguousarray(A.transpose(0, 2, 1)) if tA else A)
+        dB = dev(np.ascontiguousarray(B.transpose(0, 2, 1)) if tB else B)
+        got = host(ops.matmul(dA, dB, tA, tB))
+        assert np.array_equal(got, ref), (case, bsz, m, n, k, tA, tB)
+
+
 def test_conv2d_rejects_bad_groups(ops):
     from pet_amd import abi
     x = torch.zeros((1, 4, 5, 5), device="cuda")
