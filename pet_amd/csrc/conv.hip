@@ -47,7 +47,6 @@ struct ConvParams {
     int *cnt;      // split-K: arrival counter per tile, zero between launches
     FastDiv fd_krs, fd_rs, fd_s;     // k -> (c, kt, r, s)
     FastDiv fd_opix, fd_ohw, fd_ow;  // pixel -> (n, ot, oh, ow)
-    int tiles_n;                     // pixel tiles (for the workgroup swizzle)
 };
 
 
@@ -282,9 +281,9 @@ __global__ __launch_bounds__(Cfg::NT) void conv_pipe_kernel(ConvParams p) {
 // that fixed byte offset, or 2^31 for a padding tap, which the buffer range
 // check answers with 0; the step only moves the scalar base. Per element and
 // step the wave issues one load and half a ds_write and no address arithmetic,
-// which is what lets one wave per SIMD keep the MFMA pipe busy: a wave issues
-// at most one instruction every four cycles, so the whole step has to fit in
-// 16 instructions per MFMA.
+// which is what lets one or two waves per SIMD keep the MFMA pipe busy: a wave
+// issues at most one instruction every four cycles, so with one wave per SIMD the
+// whole step has to fit in 16 instructions per MFMA.
 //
 // Schedule of step kt (NM slots, one MFMA each): first half, W(kt+1): prefetch
 // registers -> LDS, each piece followed by G(kt+2): global -> the registers just
