@@ -190,7 +190,24 @@ def main():
     ms = time_kernel(lambda: ops.permute_flat(big, bflat, bperm, out=big_out), reps=10, warm=2)
     per_op.append({"op": "space_to_batch 1x4096x256x256 (1 GiB)", "ms": ms,
                    "GB/s": big_bytes / ms / 1e6, "frac_hbm": big_bytes / ms / 1e6 / HBM_PEAK_GBS})
-    del big, big_out
+    # ... its inverse, the H2N transform (an outer-dimension move), and the same H2N with
+    # the one-row halo that makes the transformed convolution exact
+    ms = time_kernel(lambda: ops.permute_flat(big_out, [2, 2, 1, 4096, 128, 128],
+                                              [2, 3, 4, 0, 5, 1], out=big), reps=10, warm=2)
+    per_op.append({"op": "batch_to_space 4x4096x128x128 (1 GiB)", "ms": ms,
+                   "GB/s": big_bytes / ms / 1e6, "frac_hbm": big_bytes / ms / 1e6 / HBM_PEAK_GBS})
+    ms = time_kernel(lambda: ops.permute_flat(big, [1, 4096, 2, 128, 256], [0, 2, 1, 3, 4],
+                                              out=big_out), reps=10, warm=2)
+    per_op.append({"op": "H2N 1x4096x256x256 -> 2x4096x128x256 (1 GiB)", "ms": ms,
+                   "GB/s": big_bytes / ms / 1e6, "frac_hbm": big_bytes / ms / 1e6 / HBM_PEAK_GBS})
+    del big_out
+    halo_chain = [("split", 2, 128, 0, 1), ("reorder", [0, 2, 1, 3, 4]), ("fuse", 0, 0, 0)]
+    halo_out = ops.trans_chain(big, halo_chain)
+    halo_bytes = 4.0 * (big.numel() + halo_out.numel())
+    ms = time_kernel(lambda: ops.trans_chain(big, halo_chain, out=halo_out), reps=10, warm=2)
+    per_op.append({"op": "H2N with 1-row halo, same tensor", "ms": ms,
+                   "GB/s": halo_bytes / ms / 1e6, "frac_hbm": halo_bytes / ms / 1e6 / HBM_PEAK_GBS})
+    del big, halo_out
 
     # ---- the other configurations: batch-1 latency of the original network and of
     # its PET-transformed program, each replayed as one HIP graph
