@@ -52,6 +52,8 @@ def main():
     ap.add_argument("--cpu-seconds", type=float, default=15.0)
     ap.add_argument("--no-configs", action="store_true",
                     help="skip the latency table of the other four configurations")
+    ap.add_argument("--layout-only", type=int, default=0, metavar="N",
+                    help="launch only the 1 GiB layout operators N times each and exit (for rocprofv3)")
     ap.add_argument("--dominant-only", type=int, default=0, metavar="N",
                     help="launch only the dominant kernel N times and exit (for rocprofv3)")
     args = ap.parse_args()
@@ -100,6 +102,24 @@ def main():
 
     stream = torch.cuda.Stream()
     sp = ctypes.c_void_p(stream.cuda_stream)
+
+    if args.layout_only:
+        # profiling aid: a 256 MiB calibration copy, then the 1 GiB layout operators
+        cal = torch.zeros((64, 1024, 1024), device=dev)
+        cal_out = torch.empty_like(cal)
+        ops.pad(cal, [0, 0, 0], [0, 0, 0], out=cal_out)
+        del cal, cal_out
+        big = torch.randn((1, 4096, 256, 256), device=dev)
+        big_out = torch.empty((4, 4096, 128, 128), device=dev)
+        halo_chain = [("split", 2, 128, 0, 1), ("reorder", [0, 2, 1, 3, 4]), ("fuse", 0, 0, 0)]
+        halo_out = ops.trans_chain(big, halo_chain)
+        for _ in range(args.layout_only):
+            ops.permute_flat(big, [1, 4096, 128, 2, 128, 2], [3, 5, 0, 1, 2, 4], out=big_out)
+            ops.permute_flat(big_out, [2, 2, 1, 4096, 128, 128], [2, 3, 4, 0, 5, 1], out=big)
+            ops.permute_flat(big, [1, 4096, 2, 128, 256], [0, 2, 1, 3, 4], out=big_out)
+            ops.trans_chain(big, halo_chain, out=halo_out)
+        torch.cuda.synchronize()
+        return
 
     if args.dominant_only:
         # profiling aid: the 512->512 layer of the optimised program, nothing else
