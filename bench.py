@@ -52,6 +52,8 @@ def main():
     ap.add_argument("--cpu-seconds", type=float, default=15.0)
     ap.add_argument("--no-configs", action="store_true",
                     help="skip the latency table of the other four configurations")
+    ap.add_argument("--config-only", default="", metavar="c1|c3|c4|c5[:pet]",
+                    help="replay that configuration's graph 20 times and exit (for rocprofv3)")
     ap.add_argument("--layout-only", type=int, default=0, metavar="N",
                     help="launch only the 1 GiB layout operators N times each and exit (for rocprofv3)")
     ap.add_argument("--dominant-only", type=int, default=0, metavar="N",
@@ -102,6 +104,27 @@ def main():
 
     stream = torch.cuda.Stream()
     sp = ctypes.c_void_p(stream.cuda_stream)
+
+    if args.config_only:
+        # profiling aid: one configuration (original program, or PET's with ":pet") as a graph
+        from pet_amd import programs
+        name, _, variant = args.config_only.partition(":")
+        run, params = getattr(programs, "run_" + name), getattr(programs, "params_" + name)(0)
+        ns, table = programs.GpuNS(keep=True), {}
+        with torch.cuda.stream(stream):
+            run(ns, params, variant == "pet", T=table)
+            stream.synchronize()
+            ns.kept.clear()
+            abi.call("pet_hip_graph_begin_capture", sp)
+            try:
+                run(ns, params, variant == "pet", T=table)
+            finally:
+                gh = ctypes.c_void_p(0)
+                abi.call("pet_hip_graph_end_capture", sp, ctypes.byref(gh))
+        for _ in range(20):
+            abi.call("pet_hip_graph_launch", gh, sp)
+        torch.cuda.synchronize()
+        return
 
     if args.layout_only:
         # profiling aid: a 256 MiB calibration copy, then the 1 GiB layout operators
