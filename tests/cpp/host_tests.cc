@@ -359,6 +359,80 @@ static bool test_split_ratio_and_eltwise() {
     return true;
 }
 
+// src/Mutant/generator.cc:1327-1381: two convolutions of one input become one
+// (weights concatenated on dim 0, result split on dim 1); :1159-1234: two
+// convolutions of different inputs and filter counts 8 and 12 become one
+// grouped convolution with gcd(8, 12) = 4 filters per group, the inputs
+// repeated 2 and 3 times. Same random data on both sides, results bit-equal.
+static bool runAll(Graph &g) {
+    OpVec order;
+    if (!g.topoOrder(order))
+        return false;
+    for (auto op : order)
+        if (op->compute() == nullptr)
+            return false;
+    return true;
+}
+
+static bool test_conv_merge_programs() {
+    {
+        Graph g0, g1;
+        auto x0 = g0.tensor({1, 8, 10, 10}), a0 = g0.tensor({8, 8, 3, 3}), b0 = g0.tensor({24, 8, 3, 3});
+        auto c0 = g0.conv(x0, a0, 1, 1), c1 = g0.conv(x0, b0, 1, 1);
+        g0.updateConnection();
+        auto x1 = g1.tensor({1, 8, 10, 10}), a1 = g1.tensor({8, 8, 3, 3}), b1 = g1.tensor({24, 8, 3, 3});
+        auto cw = g1.concat({a1, b1}, 0);
+        auto cv = g1.conv(x1, cw->getOutputs()[0], 1, 1);
+        auto sp = g1.split(cv->getOutputs()[0], 1, std::vector<int>{1, 3});
+        EXPECT(sp->getOutputs()[1]->getDims() == (Dim{1, 24, 10, 10}));
+        g1.updateConnection();
+        x0->dataRand(1);
+        a0->dataRand(2);
+        b0->dataRand(3);
+        x1->setData(x0->getDataPtr());
+        a1->setData(a0->getDataPtr());
+        b1->setData(b0->getDataPtr());
+        EXPECT(runAll(g0) && runAll(g1));
+        for (int i = 0; i < 2; ++i) {
+            Tensor *ref = (i ? c1 : c0)->getOutputs()[0], *got = sp->getOutputs()[i];
+            EXPECT(ref->getDims() == got->getDims());
+            EXPECT(equalArrays(got->getDataPtr(), ref->getDataPtr(), ref->size()));
+        }
+    }
+    {
+        Graph g0, g1;
+        auto x0 = g0.tensor({1, 8, 9, 9}), y0 = g0.tensor({1, 8, 9, 9});
+        auto a0 = g0.tensor({8, 8, 3, 3}), b0 = g0.tensor({12, 8, 3, 3});
+        auto c0 = g0.conv(x0, a0, 1, 1), c1 = g0.conv(y0, b0, 1, 1);
+        g0.updateConnection();
+        auto x1 = g1.tensor({1, 8, 9, 9}), y1 = g1.tensor({1, 8, 9, 9});
+        auto a1 = g1.tensor({8, 8, 3, 3}), b1 = g1.tensor({12, 8, 3, 3});
+        auto ex = g1.extend(x1, 1, 1), ey = g1.extend(y1, 1, 2);
+        auto ci = g1.concat({ex->getOutputs()[0], ey->getOutputs()[0]}, 1);
+        auto cw = g1.concat({a1, b1}, 0);
+        EXPECT(ci->getOutputs()[0]->getDims() == (Dim{1, 40, 9, 9}));
+        auto cv = g1.conv(ci->getOutputs()[0], cw->getOutputs()[0], 1, 1); // 5 groups of 8 channels
+        EXPECT(cv->getOutputs()[0]->getDims() == (Dim{1, 20, 9, 9}));
+        auto sp = g1.split(cv->getOutputs()[0], 1, std::vector<int>{2, 3});
+        g1.updateConnection();
+        x0->dataRand(4);
+        y0->dataRand(5);
+        a0->dataRand(6);
+        b0->dataRand(7);
+        x1->setData(x0->getDataPtr());
+        y1->setData(y0->getDataPtr());
+        a1->setData(a0->getDataPtr());
+        b1->setData(b0->getDataPtr());
+        EXPECT(runAll(g0) && runAll(g1));
+        for (int i = 0; i < 2; ++i) {
+            Tensor *ref = (i ? c1 : c0)->getOutputs()[0], *got = sp->getOutputs()[i];
+            EXPECT(ref->getDims() == got->getDims());
+            EXPECT(equalArrays(got->getDataPtr(), ref->getDataPtr(), ref->size()));
+        }
+    }
+    return true;
+}
+
 int main(int argc, char **argv) {
     std::vector<std::pair<std::string, std::function<bool()>>> cases = {
         {"conv_vs_oracle", test_conv_vs_oracle},
@@ -372,6 +446,7 @@ int main(int argc, char **argv) {
         {"emit_program", test_emit_program},
         {"perf_engine_memo", test_perf_engine_memo},
         {"split_ratio_and_eltwise", test_split_ratio_and_eltwise},
+        {"conv_merge_programs", test_conv_merge_programs},
     };
     std::string only = argc > 1 ? argv[1] : "";
     if (argc > 2)
