@@ -317,14 +317,19 @@ __device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void *base) {
 
 constexpr unsigned kOob = 0x80000000u; // voffset that the range check rejects
 
-template <class Cfg, bool IS3D, bool SK>
+// DIM 2: 2-D. DIM 3: 3-D with kt > 1 (one kt slice of a filter row is runs of r*s
+// floats, loaded one float at a time). DIM 4: 3-D with kt == 1 (filter rows are
+// contiguous as in 2-D and load as 16-byte words).
+template <class Cfg, int DIM, bool SK>
 __global__ __launch_bounds__(Cfg::NT) void conv_plane_kernel(ConvParams p) {
+    constexpr bool IS3D = DIM != 2;
+    constexpr bool SCALAR_A = DIM == 3;
     extern __shared__ __attribute__((aligned(16))) float lds[];
     constexpr int KH = Cfg::KH, TM = Cfg::TM, TN = Cfg::TN, RS = Cfg::RS, CB = Cfg::CB;
     constexpr int BK = Cfg::BK, NT = Cfg::NT, NW = Cfg::NW;
     constexpr int RPW = Cfg::RPW, PPL = Cfg::PPL;
     constexpr int A_LD = Cfg::A_LD, B_LD = Cfg::B_LD;
-    constexpr int NA = IS3D ? Cfg::A_SPT : Cfg::A_VPT; // A pieces per thread
+    constexpr int NA = SCALAR_A ? Cfg::A_SPT : Cfg::A_VPT; // A pieces per thread
     constexpr int NM = KH * TM * TN;                   // slots per step
     constexpr int HALF = NM / 2;
     constexpr int NWP = NA + RPW;                      // W pieces (first half)
@@ -458,7 +463,7 @@ __global__ __launch_bounds__(Cfg::NT) void conv_plane_kernel(ConvParams p) {
     int ldsA[NA];
 #pragma unroll
     for (int i = 0; i < NA; ++i) {
-        if (IS3D) {
+        if (SCALAR_A) {
             const int e = tid + i * NT;
             const int f = e / BK, kl = e % BK;
             const int cl = kl / RS, t = kl % RS;
@@ -477,8 +482,8 @@ __global__ __launch_bounds__(Cfg::NT) void conv_plane_kernel(ConvParams p) {
     const int b_frag = Cfg::A_ELEMS + hk * KH * B_LD + wn0 + l32;
     const int b_lds = Cfg::A_ELEMS + wave * B_LD + lane;
 
-    float4 preA4[IS3D ? 1 : NA];
-    float preA1[IS3D ? NA : 1];
+    float4 preA4[SCALAR_A ? 1 : NA];
+    float preA1[SCALAR_A ? NA : 1];
     float preB[RPW][PPL];
     float fa[2][TM][KH];
     float fb[2][KH][TN];
@@ -509,7 +514,7 @@ __global__ __launch_bounds__(Cfg::NT) void conv_plane_kernel(ConvParams p) {
         if (i < NA) {
             const unsigned so = (unsigned)(pcb * CB * KRS + pq * RS) * 4u;
             const __amdgpu_buffer_rsrc_t ra = make_rsrc(wg);
-            if (IS3D) {
+            if (SCALAR_A) {
                 preA1[i] = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(ra, voffA[i], so, 0));
             } else {
                 uintx4 v = __builtin_amdgcn_raw_buffer_load_b128(ra, voffA[i], so, 0);
@@ -531,7 +536,7 @@ __global__ __launch_bounds__(Cfg::NT) void conv_plane_kernel(ConvParams p) {
     };
     auto w_piece = [&](int i, float *st) __attribute__((always_inline)) {
         if (i < NA) {
-            if (IS3D) {
+            if (SCALAR_A) {
                 st[ldsA[i]] = preA1[i];
             } else {
                 // the last, partly filled round only exists for the first threads
@@ -848,17 +853,17 @@ __global__ __launch_bounds__(256) void splitk_init_kernel(float *__restrict__ y,
 template <class Cfg>
 constexpr bool has_streamk = Cfg::BM >= 64 && Cfg::RS == 9;
 
-template <class Cfg, bool IS3D>
+template <class Cfg, int DIM>
 int launch_plane_cfg(ConvParams p, hipStream_t stream) {
     const size_t lds_bytes = 2 * (size_t)Cfg::STAGE * sizeof(float);
     static int attr_status = [&] {
         hipError_t e = hipFuncSetAttribute(
-            reinterpret_cast<const void *>(&conv_plane_kernel<Cfg, IS3D, false>),
+            reinterpret_cast<const void *>(&conv_plane_kernel<Cfg, DIM, false>),
             hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
         if constexpr (has_streamk<Cfg>) {
             if (e == hipSuccess)
                 e = hipFuncSetAttribute(
-                    reinterpret_cast<const void *>(&conv_plane_kernel<Cfg, IS3D, true>),
+                    reinterpret_cast<const void *>(&conv_plane_kernel<Cfg, DIM, true>),
                     hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds_bytes);
         }
         return e == hipSuccess ? 0 : 1;
@@ -973,12 +978,12 @@ int launch_plane_cfg(ConvParams p, hipStream_t stream) {
     if constexpr (has_streamk<Cfg>) {
         if (p.streamk) {
             grid = dim3(Cfg::BM * Cfg::BN >= 64 * 128 ? 256 : 512, 1, 1);
-            hipLaunchKernelGGL((conv_plane_kernel<Cfg, IS3D, true>), grid, dim3(Cfg::NT), lds_bytes,
+            hipLaunchKernelGGL((conv_plane_kernel<Cfg, DIM, true>), grid, dim3(Cfg::NT), lds_bytes,
                                stream, p);
         }
     }
     if (!p.streamk)
-        hipLaunchKernelGGL((conv_plane_kernel<Cfg, IS3D, false>), grid, dim3(Cfg::NT), lds_bytes,
+        hipLaunchKernelGGL((conv_plane_kernel<Cfg, DIM, false>), grid, dim3(Cfg::NT), lds_bytes,
                            stream, p);
     int rc = check_launch("conv_plane_kernel");
     if (rc == PET_HIP_OK && p.atomic_out && p.act != PET_HIP_ACT_NONE)
@@ -1005,14 +1010,18 @@ int launch_plane(const ConvParams &p, bool is3d, hipStream_t stream) {
         tile = 0;
     if (forced_tile() >= 0)
         tile = forced_tile() % 3;
+    const int dim = !is3d ? 2 : (p.KT == 1 ? 4 : 3);
     if (tile == 0)
-        return is3d ? launch_plane_cfg<C64x128, true>(p, stream)
-                    : launch_plane_cfg<C64x128, false>(p, stream);
+        return dim == 2   ? launch_plane_cfg<C64x128, 2>(p, stream)
+               : dim == 3 ? launch_plane_cfg<C64x128, 3>(p, stream)
+                          : launch_plane_cfg<C64x128, 4>(p, stream);
     if (tile == 1)
-        return is3d ? launch_plane_cfg<C64x64, true>(p, stream)
-                    : launch_plane_cfg<C64x64, false>(p, stream);
-    return is3d ? launch_plane_cfg<C32x64, true>(p, stream)
-                : launch_plane_cfg<C32x64, false>(p, stream);
+        return dim == 2   ? launch_plane_cfg<C64x64, 2>(p, stream)
+               : dim == 3 ? launch_plane_cfg<C64x64, 3>(p, stream)
+                          : launch_plane_cfg<C64x64, 4>(p, stream);
+    return dim == 2   ? launch_plane_cfg<C32x64, 2>(p, stream)
+           : dim == 3 ? launch_plane_cfg<C32x64, 3>(p, stream)
+                      : launch_plane_cfg<C32x64, 4>(p, stream);
 }
 
 // Returns -1 when the plane kernel does not apply.
