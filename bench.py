@@ -1,7 +1,7 @@
 #!/usr/bin/env python3
 """Benchmark: batch-1 latency of the PET-optimised dilated-conv block on one MI355X.
 
-Workload (BASELINE config 2): six fp32 3x3 convolutions, dilation 2 / pad 2,
+Workload (benchmark configuration 2): six fp32 3x3 convolutions, dilation 2 / pad 2,
 channels 512->512->512->512->256->128->64 on a 1x512x64x64 input, ReLU after
 each, weights N(0, 0.01). The PET-optimised program is space-to-batch (4 phase
 images of 32x32), six dense convolutions (dilation 1, pad 1) with fused ReLU,

@@ -160,7 +160,7 @@ static bool test_pad_conv_slice_verification() {
     return true;
 }
 
-// BASELINE config 1, small: conv == H2N (halo) -> conv -> N2H (drop). Without
+// Benchmark configuration 1, small: conv == H2N (halo) -> conv -> N2H (drop). Without
 // the correction the two programs differ at the seam.
 static bool test_corrected_h2n_program() {
     const int c = 8, h = 12, w = 10, f = 8;

@@ -501,7 +501,7 @@ def test_softmax_layernorm_row_lengths(ops, cols):
 
 
 def test_config1_original_vs_corrected_transform(ops):
-    # BASELINE config 1: conv 1x64x56x56, 3x3 p1, U[-1,1] from seed 0 (x then w);
+    # benchmark configuration 1: conv 1x64x56x56, 3x3 p1, U[-1,1] from seed 0 (x then w);
     # original op vs H2N(halo 1) -> conv -> N2H(drop 1).
     rng = np.random.default_rng(0)
     x = rng.uniform(-1, 1, (1, 64, 56, 56)).astype(np.float32)
