@@ -179,7 +179,7 @@ class ConvOp : public Operator {
 
     Dim computeShape() override;
     Dim computeOutputPenalty(const Dim &p);
-    double perf(PerfEngine *pe, int rounds, int warmupRounds) override;
+    double perf(PerfEngine *pe, int rounds = 200, int warmupRounds = 200) override;
     int launch(pet_hip_stream_t stream) override;
     std::string toString() const override;
     int numInputs() override { return 2; }
@@ -220,7 +220,7 @@ class Conv3dOp : public Operator {
     Conv3dOp(const Conv3dOp &rhs);
     Conv3dOp *clone() override { return new Conv3dOp(*this); }
     Dim computeShape() override;
-    double perf(PerfEngine *pe, int rounds, int warmupRounds) override;
+    double perf(PerfEngine *pe, int rounds = 200, int warmupRounds = 200) override;
     int launch(pet_hip_stream_t stream) override;
     std::string toString() const override;
     int numInputs() override { return 2; }
@@ -253,7 +253,7 @@ class MatmulOp : public Operator {
     MatmulOp *clone() override { return new MatmulOp(*this); }
 
     Dim computeShape() override;
-    double perf(PerfEngine *pe, int rounds, int warmupRounds) override;
+    double perf(PerfEngine *pe, int rounds = 200, int warmupRounds = 200) override;
     int launch(pet_hip_stream_t stream) override;
     std::string toString() const override;
     int numInputs() override { return 2; }
@@ -284,7 +284,7 @@ class PadOp : public Operator {
     PadOp(const PadOp &rhs) : Operator(rhs), begin(rhs.begin), end(rhs.end) {}
     PadOp *clone() override { return new PadOp(*this); }
     Dim computeShape() override;
-    double perf(PerfEngine *pe, int rounds, int warmupRounds) override;
+    double perf(PerfEngine *pe, int rounds = 200, int warmupRounds = 200) override;
     int launch(pet_hip_stream_t stream) override;
     std::string toString() const override;
     int numInputs() override { return 1; }
@@ -306,7 +306,7 @@ class SliceOp : public Operator {
     SliceOp(const SliceOp &rhs) : Operator(rhs), begin(rhs.begin), end(rhs.end) {}
     SliceOp *clone() override { return new SliceOp(*this); }
     Dim computeShape() override;
-    double perf(PerfEngine *pe, int rounds, int warmupRounds) override;
+    double perf(PerfEngine *pe, int rounds = 200, int warmupRounds = 200) override;
     int launch(pet_hip_stream_t stream) override;
     std::string toString() const override;
     int numInputs() override { return 1; }
@@ -329,7 +329,7 @@ class ConcatOp : public Operator {
     ConcatOp(const ConcatOp &rhs) : Operator(rhs), dim(rhs.dim) {}
     ConcatOp *clone() override { return new ConcatOp(*this); }
     Dim computeShape() override;
-    double perf(PerfEngine *pe, int rounds, int warmupRounds) override;
+    double perf(PerfEngine *pe, int rounds = 200, int warmupRounds = 200) override;
     int launch(pet_hip_stream_t stream) override;
     std::string toString() const override;
     int numInputs() override { return (int)inputs.size(); }
@@ -357,7 +357,7 @@ class SplitOp : public Operator {
     Dim computeShape() override;            // dims of output 0
     std::vector<Dim> computeShapeV();       // ratio rule; empty when not divisible
     bool computeShape(const TensorVec &ins, const TensorVec &outs) override;
-    double perf(PerfEngine *pe, int rounds, int warmupRounds) override;
+    double perf(PerfEngine *pe, int rounds = 200, int warmupRounds = 200) override;
     int launch(pet_hip_stream_t stream) override;
     std::string toString() const override;
     int numInputs() override { return 1; }
@@ -420,7 +420,7 @@ class TransposeOp : public Operator {
     TransposeOp *clone() override { return new TransposeOp(*this); }
 
     Dim computeShape() override;
-    double perf(PerfEngine *pe, int rounds, int warmupRounds) override;
+    double perf(PerfEngine *pe, int rounds = 200, int warmupRounds = 200) override;
     int launch(pet_hip_stream_t stream) override;
     std::string toString() const override;
     int numInputs() override { return 1; }
@@ -470,7 +470,7 @@ class ExtendOp : public Operator {
     ExtendOp(const ExtendOp &rhs) : Operator(rhs), dim(rhs.dim), num(rhs.num) {}
     ExtendOp *clone() override { return new ExtendOp(*this); }
     Dim computeShape() override;
-    double perf(PerfEngine *pe, int rounds, int warmupRounds) override;
+    double perf(PerfEngine *pe, int rounds = 200, int warmupRounds = 200) override;
     int launch(pet_hip_stream_t stream) override;
     std::string toString() const override;
     int numInputs() override { return 1; }
@@ -491,7 +491,7 @@ class EltwiseOp : public Operator {
     explicit EltwiseOp(OpType type) : Operator(type) { initHash(); }
     EltwiseOp(const EltwiseOp &rhs) : Operator(rhs) {}
     Dim computeShape() override;
-    double perf(PerfEngine *pe, int rounds, int warmupRounds) override;
+    double perf(PerfEngine *pe, int rounds = 200, int warmupRounds = 200) override;
     int launch(pet_hip_stream_t stream) override;
     std::string toString() const override;
     int numInputs() override { return type == Sub ? 2 : (int)inputs.size(); }
@@ -535,7 +535,7 @@ class ActivationOp : public Operator {
     ActivationOp(const ActivationOp &rhs) : Operator(rhs), actType(rhs.actType) {}
     ActivationOp *clone() override { return new ActivationOp(*this); }
     Dim computeShape() override;
-    double perf(PerfEngine *pe, int rounds, int warmupRounds) override;
+    double perf(PerfEngine *pe, int rounds = 200, int warmupRounds = 200) override;
     int launch(pet_hip_stream_t stream) override;
     std::string toString() const override;
     int numInputs() override { return 1; }
@@ -556,7 +556,7 @@ class PoolOp : public Operator {
     PoolOp(const PoolOp &rhs);
     PoolOp *clone() override { return new PoolOp(*this); }
     Dim computeShape() override;
-    double perf(PerfEngine *pe, int rounds, int warmupRounds) override;
+    double perf(PerfEngine *pe, int rounds = 200, int warmupRounds = 200) override;
     int launch(pet_hip_stream_t stream) override;
     std::string toString() const override;
     int numInputs() override { return 1; }
@@ -574,12 +574,18 @@ class MaxPoolOp : public PoolOp {
     MaxPoolOp(Tensor *input, Tensor *output, int kh, int kw, int dh, int dw, int ph, int pw,
               int sh, int sw)
         : PoolOp(MaxPool, input, output, kh, kw, dh, dw, ph, pw, sh, sw) {}
+    // Output tensor made by the operator (reference include/operator.h:1332).
+    MaxPoolOp(Tensor *input, int kh, int kw, int dh, int dw, int ph, int pw, int sh, int sw)
+        : MaxPoolOp(input, new Tensor(), kh, kw, dh, dw, ph, pw, sh, sw) {}
 };
 
 class AvgPoolOp : public PoolOp {
   public:
     AvgPoolOp(Tensor *input, Tensor *output, int kh, int kw, int ph, int pw, int sh, int sw)
         : PoolOp(AvgPool, input, output, kh, kw, 1, 1, ph, pw, sh, sw) {}
+    // Output tensor made by the operator (reference include/operator.h:1411).
+    AvgPoolOp(Tensor *input, int kh, int kw, int ph, int pw, int sh, int sw)
+        : AvgPoolOp(input, new Tensor(), kh, kw, ph, pw, sh, sw) {}
     // global average pool
     AvgPoolOp(Tensor *input, Tensor *output);
 };
@@ -590,7 +596,7 @@ class SoftmaxOp : public Operator {
     SoftmaxOp(const SoftmaxOp &rhs) : Operator(rhs), axis(rhs.axis) {}
     SoftmaxOp *clone() override { return new SoftmaxOp(*this); }
     Dim computeShape() override;
-    double perf(PerfEngine *pe, int rounds, int warmupRounds) override;
+    double perf(PerfEngine *pe, int rounds = 200, int warmupRounds = 200) override;
     int launch(pet_hip_stream_t stream) override;
     std::string toString() const override;
     int numInputs() override { return 1; }
@@ -609,7 +615,7 @@ class LayerNormOp : public Operator {
         : Operator(rhs), gamma(rhs.gamma), beta(rhs.beta), eps(rhs.eps) {}
     LayerNormOp *clone() override { return new LayerNormOp(*this); }
     Dim computeShape() override;
-    double perf(PerfEngine *pe, int rounds, int warmupRounds) override;
+    double perf(PerfEngine *pe, int rounds = 200, int warmupRounds = 200) override;
     int launch(pet_hip_stream_t stream) override;
     std::string toString() const override;
     int numInputs() override { return 1; }
@@ -632,7 +638,7 @@ class ReshapeOp : public Operator {
     ReshapeOp(const ReshapeOp &rhs) : Operator(rhs) {}
     ReshapeOp *clone() override { return new ReshapeOp(*this); }
     Dim computeShape() override;
-    double perf(PerfEngine *pe, int rounds, int warmupRounds) override;
+    double perf(PerfEngine *pe, int rounds = 200, int warmupRounds = 200) override;
     int launch(pet_hip_stream_t stream) override;
     std::string toString() const override;
     int numInputs() override { return 1; }

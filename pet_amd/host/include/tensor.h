@@ -88,6 +88,14 @@ class Tensor {
 
     size_t getOffset(const Dim &pos) const; // (size_t)-1 when out of range
 
+    // Row-major position cursor over the tensor's index space, as the
+    // reference's tests walk outputs (include/tensor.h:275-304).
+    void itInit() { it.assign(dims.size(), 0); }
+    void itReset() { itInit(); }
+    bool itValid() const;
+    const Dim &itGet() const { return it; }
+    void itNext();
+
     // splitting points (kept for the search-side API)
     const SplittingPoints *getSplittingPoints() const { return &splittingPoints; }
     bool setSplittingPoints(SplittingPoints v) {
@@ -110,6 +118,7 @@ class Tensor {
     ComputeState computed = NotComputed;
     SplittingPoints splittingPoints;
     Dim dimPenalty;
+    Dim it;
 
     float *dev = nullptr;
     size_t devElems = 0;

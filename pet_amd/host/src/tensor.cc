@@ -196,6 +196,28 @@ size_t Tensor::getOffset(const Dim &pos) const {
     return off;
 }
 
+bool Tensor::itValid() const {
+    if (it.size() != dims.size())
+        return false;
+    for (size_t i = 0; i < it.size(); ++i)
+        if (it[i] >= dims[i])
+            return false;
+    return true;
+}
+
+// Odometer step: the last axis moves fastest; running off the end of axis 0
+// leaves it[0] == dims[0], which itValid() reports.
+void Tensor::itNext() {
+    if (it.empty())
+        return;
+    size_t p = it.size() - 1;
+    ++it[p];
+    while (p > 0 && it[p] == dims[p]) {
+        it[p] = 0;
+        ++it[--p];
+    }
+}
+
 VType Tensor::getData(const Dim &pos) {
     size_t off = getOffset(pos);
     if (off == (size_t)-1)
