@@ -251,6 +251,10 @@ class MatmulOp : public Operator {
     MatmulOp(const MatmulOp &rhs)
         : Operator(rhs), transA(rhs.transA), transB(rhs.transB), bias(rhs.bias), act(rhs.act) {}
     MatmulOp *clone() override { return new MatmulOp(*this); }
+    // One output point -> the input points it depends on; the closure runs the
+    // whole operator on the device.
+    std::pair<std::vector<DimRange>, std::function<bool()>> compute(DimRange dr) override;
+    using Operator::compute;
 
     Dim computeShape() override;
     double perf(PerfEngine *pe, int rounds = 200, int warmupRounds = 200) override;
@@ -328,6 +332,10 @@ class ConcatOp : public Operator {
     explicit ConcatOp(int dim);
     ConcatOp(const ConcatOp &rhs) : Operator(rhs), dim(rhs.dim) {}
     ConcatOp *clone() override { return new ConcatOp(*this); }
+    // One output point -> the input points it depends on; the closure runs the
+    // whole operator on the device.
+    std::pair<std::vector<DimRange>, std::function<bool()>> compute(DimRange dr) override;
+    using Operator::compute;
     Dim computeShape() override;
     double perf(PerfEngine *pe, int rounds = 200, int warmupRounds = 200) override;
     int launch(pet_hip_stream_t stream) override;
@@ -354,6 +362,11 @@ class SplitOp : public Operator {
 
     Tensor *compute() override; // returns outputs[0] (the reference asserts here)
     TensorVec computeV();
+    using Operator::compute;
+    // Point `dr` of output `idx` -> the input point it is copied from
+    // (reference src/Graph/operator.cc:2027-2045). The closure splits the
+    // whole tensor on the device.
+    std::pair<std::vector<DimRange>, std::function<bool()>> compute(size_t idx, DimRange dr);
     Dim computeShape() override;            // dims of output 0
     std::vector<Dim> computeShapeV();       // ratio rule; empty when not divisible
     bool computeShape(const TensorVec &ins, const TensorVec &outs) override;
@@ -418,6 +431,10 @@ class TransposeOp : public Operator {
     TransposeOp(int split, const Perm &after, int factor = 2, TransType trans_type = NoneType);
     TransposeOp(const TransposeOp &rhs);
     TransposeOp *clone() override { return new TransposeOp(*this); }
+    // One output point -> the input points it depends on; the closure runs the
+    // whole operator on the device.
+    std::pair<std::vector<DimRange>, std::function<bool()>> compute(DimRange dr) override;
+    using Operator::compute;
 
     Dim computeShape() override;
     double perf(PerfEngine *pe, int rounds = 200, int warmupRounds = 200) override;
@@ -469,6 +486,10 @@ class ExtendOp : public Operator {
     ExtendOp(int dim, int num);
     ExtendOp(const ExtendOp &rhs) : Operator(rhs), dim(rhs.dim), num(rhs.num) {}
     ExtendOp *clone() override { return new ExtendOp(*this); }
+    // One output point -> the input points it depends on; the closure runs the
+    // whole operator on the device.
+    std::pair<std::vector<DimRange>, std::function<bool()>> compute(DimRange dr) override;
+    using Operator::compute;
     Dim computeShape() override;
     double perf(PerfEngine *pe, int rounds = 200, int warmupRounds = 200) override;
     int launch(pet_hip_stream_t stream) override;
@@ -496,6 +517,10 @@ class EltwiseOp : public Operator {
     std::string toString() const override;
     int numInputs() override { return type == Sub ? 2 : (int)inputs.size(); }
     int numOutputs() override { return 1; }
+    // One output point -> the input points it depends on; the closure runs the
+    // whole operator on the device.
+    std::pair<std::vector<DimRange>, std::function<bool()>> compute(DimRange dr) override;
+    using Operator::compute;
     bool computeShape(const TensorVec &ins, const TensorVec &outs) override;
 
   protected:

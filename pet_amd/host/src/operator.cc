@@ -769,6 +769,23 @@ TensorVec SplitOp::computeV() {
     return outputs;
 }
 
+std::pair<std::vector<DimRange>, std::function<bool()>> SplitOp::compute(size_t idx,
+                                                                         DimRange dr) {
+    if (dr.notValid() || idx >= outputs.size())
+        return {};
+    if (dr.isEmpty())
+        return {{DimRange::getEmpty()}, []() { return true; }};
+    auto whole = [this]() { return !computeV().empty(); };
+    if (!dr.isSinglePos())
+        return {{DimRange::getAllPos()}, whole};
+    Dim src = dr.getBegin();
+    if (src.size() != inputs[0]->getDims().size())
+        return {};
+    for (size_t i = 0; i < idx; ++i)
+        src[dim] += outputs[i]->getDims()[dim];
+    return {{DimRange(src)}, whole};
+}
+
 int SplitOp::launch(pet_hip_stream_t stream) {
     std::vector<float *> ptrs;
     std::vector<int> outSizes;
@@ -1344,6 +1361,125 @@ double ReshapeOp::perf(PerfEngine *, int, int) { return 0.0; }
 std::string ReshapeOp::toString() const {
     return getOpName(type) + "(" + dimToString(inputs[0]->getDims()) + "->" +
            dimToString(outputs[0]->getDims()) + ")";
+}
+
+// ---- point dependences ------------------------------------------------------------
+// For one output point, the input points it is computed from; the reference
+// reports the same ranges (src/Graph/operator.cc:664-698, 1852-1880,
+// 2212-2303, 2600-2616, 3005-3023) and evaluates the point on the host, here
+// the returned closure runs the whole operator on the device.
+namespace {
+using PointDeps = std::pair<std::vector<DimRange>, std::function<bool()>>;
+
+// Handles the ranges that are not a single point. Returns true when `out`
+// already holds the answer.
+bool symbolicRange(Operator *op, const DimRange &dr, size_t nIn, PointDeps &out) {
+    if (dr.notValid()) {
+        out = {};
+        return true;
+    }
+    if (dr.isEmpty()) {
+        out = {std::vector<DimRange>(nIn, DimRange::getEmpty()), []() { return true; }};
+        return true;
+    }
+    if (!dr.isSinglePos()) {
+        out = {std::vector<DimRange>(nIn, DimRange::getAllPos()),
+               [op]() { return op->compute() != nullptr; }};
+        return true;
+    }
+    return false;
+}
+
+bool insideDims(const Dim &pos, const Dim &dims) {
+    if (pos.size() != dims.size())
+        return false;
+    for (size_t i = 0; i < pos.size(); ++i)
+        if (pos[i] < 0 || pos[i] >= dims[i])
+            return false;
+    return true;
+}
+} // namespace
+
+PointDeps MatmulOp::compute(DimRange dr) {
+    PointDeps ret;
+    if (symbolicRange(this, dr, inputs.size(), ret))
+        return ret;
+    const Dim &pos = dr.getBegin();
+    if (pos.size() != 3 || !insideDims(pos, outputs[0]->getDims()))
+        return {};
+    int b = pos[0], m = pos[1], n = pos[2];
+    int k = inputs[0]->getDims()[transA ? 1 : 2];
+    DimRange lhs = transA ? DimRange({b, 0, m}, {b, k - 1, m}) : DimRange({b, m, 0}, {b, m, k - 1});
+    DimRange rhs = transB ? DimRange({b, n, 0}, {b, n, k - 1}) : DimRange({b, 0, n}, {b, k - 1, n});
+    return {{lhs, rhs}, [this]() { return compute() != nullptr; }};
+}
+
+PointDeps ConcatOp::compute(DimRange dr) {
+    PointDeps ret;
+    if (symbolicRange(this, dr, inputs.size(), ret))
+        return ret;
+    Dim src = dr.getBegin();
+    if (!insideDims(src, outputs[0]->getDims()))
+        return {};
+    size_t which = 0;
+    while (which < inputs.size() && src[dim] >= inputs[which]->getDims()[dim])
+        src[dim] -= inputs[which++]->getDims()[dim];
+    std::vector<DimRange> deps(inputs.size(), DimRange::getEmpty());
+    deps[which] = DimRange(src);
+    return {deps, [this]() { return compute() != nullptr; }};
+}
+
+PointDeps ExtendOp::compute(DimRange dr) {
+    PointDeps ret;
+    if (symbolicRange(this, dr, inputs.size(), ret))
+        return ret;
+    Dim src = dr.getBegin();
+    if (!insideDims(src, outputs[0]->getDims()))
+        return {};
+    src[dim] %= inputs[0]->getDims()[dim];
+    return {{DimRange(src)}, [this]() { return compute() != nullptr; }};
+}
+
+PointDeps EltwiseOp::compute(DimRange dr) {
+    PointDeps ret;
+    if (symbolicRange(this, dr, inputs.size(), ret))
+        return ret;
+    const Dim &pos = dr.getBegin();
+    size_t flat = outputs[0]->getOffset(pos);
+    if (flat == (size_t)-1)
+        return {};
+    std::vector<DimRange> deps;
+    for (Tensor *in : inputs) // flat-modulo broadcast
+        deps.emplace_back(cntToIdx(in->getDims(), flat % in->size()));
+    return {deps, [this]() { return compute() != nullptr; }};
+}
+
+// y = x.reshape(flat).transpose(after).reshape(out): the output point's linear
+// index over the permuted flat dims gives its flat coordinates; un-permuted,
+// they give the linear index into the input. With boundary correction on, the
+// dependence is reported as the whole input.
+PointDeps TransposeOp::compute(DimRange dr) {
+    PointDeps ret;
+    if (symbolicRange(this, dr, inputs.size(), ret))
+        return ret;
+    auto whole = [this]() { return compute() != nullptr; };
+    if (corrected())
+        return {{DimRange::getAllPos()}, whole};
+    Dim flat;
+    size_t outOff = outputs[0]->getOffset(dr.getBegin());
+    if (outOff == (size_t)-1 || !flatDims(flat))
+        return {};
+    std::vector<int> order = after.asVector();
+    Dim permuted(order.size());
+    for (size_t i = 0; i < order.size(); ++i)
+        permuted[i] = flat[order[i]];
+    Dim at = cntToIdx(permuted, outOff), src(flat.size(), 0);
+    for (size_t i = 0; i < order.size(); ++i)
+        src[order[i]] = at[i];
+    size_t inOff = 0;
+    for (size_t i = 0; i < flat.size(); ++i)
+        inOff = inOff * (size_t)flat[i] + (size_t)src[i];
+    return {{DimRange(cntToIdx(inputs[0]->getDims(), inOff))}, whole};
 }
 
 } // namespace tpm

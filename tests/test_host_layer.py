@@ -71,11 +71,13 @@ def test_emitted_program_compiles_and_runs(tmp_path):
 # by empty files made at test time.
 REFERENCE_PROGRAMS = [
     "SampleGraph3.cpp", "SampleGraph4.cpp", "batch_gemm_test.cc", "concat_test_1.cc",
-    "conv_test_1.cc", "conv_test_2.cc", "conv_test_4_perf.cc", "conv_test_5_trans_kernel.cc",
+    "conv_test_1.cc", "conv_test_2.cc", "conv_test_3.cc", "conv_test_4_perf.cc",
+    "conv_test_5_trans_kernel.cc",
     "extend_test_1.cc", "gemm_test_1_perf.cc", "gemm_test_2_conv1x1_perf.cc",
     "group_conv_test_1.cc", "group_conv_test_2.cc", "mutant_test_2.cc", "pad_slice_test.cc",
-    "perf_pool.cc", "split_test_1.cc", "tensor_test.cc", "transpose_test_1.cc",
-    "transpose_test_2.cc", "transpose_test_3.cc", "transpose_test_5.cc",
+    "perf_pool.cc", "split_test_1.cc", "split_test_2.cc", "tensor_test.cc",
+    "transpose_test_1.cc", "transpose_test_2.cc", "transpose_test_3.cc", "transpose_test_4.cc",
+    "transpose_test_5.cc",
 ]
 REFERENCE_TESTS = "/root/reference/src/Test"
 
@@ -133,3 +135,109 @@ def test_tensor_cursor_and_pool_constructors_without_a_gpu(tmp_path):
                     "-Wl,-rpath," + LIB, "-o", str(exe)], check=True)
     run = subprocess.run([str(exe)], capture_output=True, text=True, timeout=60)
     assert run.returncode == 0, (run.returncode, run.stdout, run.stderr)
+
+
+# Prints, for every output point of a few operators, the linear offset of the
+# input point the operator reports as its dependence (input index:offset).
+DEPENDENCE_PROGRAM = r"""
+#include "operator.h"
+#include "tensor.h"
+#include <cstdio>
+using namespace tpm;
+static void walk(const char *name, Operator *op, Tensor *out) {
+    std::printf("%s", name);
+    for (out->itInit(); out->itValid(); out->itNext()) {
+        auto deps = op->compute(DimRange(out->itGet())).first;
+        for (size_t i = 0; i < deps.size(); ++i)
+            if (deps[i].isSinglePos())
+                std::printf(" %zu:%zu", i, op->getInputs()[i]->getOffset(deps[i].getBegin()));
+    }
+    std::printf("\n");
+}
+int main() {
+    Tensor x({2, 4, 6, 8});
+    // the forms of src/Mutant/generator.cc:1028-1092
+    TransposeOp h2n(&x, 2, {{0, 2}, 1, -1, 3}, -2, TransposeOp::H2N);
+    walk("h2n", &h2n, h2n.getOutputs()[0]);
+    TransposeOp n2h(&x, 0, {0, 1, {-1, 2}, 3}, 2, TransposeOp::N2H);
+    walk("n2h", &n2h, n2h.getOutputs()[0]);
+    TransposeOp d2h(&x, 2, {0, 1, {-1, 2}, 3}, 2, TransposeOp::D2H);
+    walk("d2h", &d2h, d2h.getOutputs()[0]);
+    TransposeOp d2hInv(&x, 2, {0, 1, {-1, 2}, 3}, -2, TransposeOp::D2H);
+    walk("d2hInv", &d2hInv, d2hInv.getOutputs()[0]);
+    TransposeOp swap(&x, -1, {0, 1, 3, 2});
+    walk("swap", &swap, swap.getOutputs()[0]);
+    Tensor a({2, 3, 4}), b({2, 5, 4});
+    ConcatOp cat({&a, &b}, 1);
+    walk("concat", &cat, cat.getOutputs()[0]);
+    ExtendOp ext(&a, 1, 2);
+    walk("extend", &ext, ext.getOutputs()[0]);
+    Tensor bias({4});
+    Tensor sum;
+    AddOp add({&a, &bias}, &sum);
+    walk("add", &add, &sum);
+    SplitOp split(&b, 1, {2, 3});
+    for (size_t k = 0; k < 2; ++k) {
+        Tensor *o = split.getOutputs()[k];
+        std::printf("split%zu", k);
+        for (o->itInit(); o->itValid(); o->itNext())
+            std::printf(" 0:%zu", b.getOffset(split.compute(k, DimRange(o->itGet())).first[0].getBegin()));
+        std::printf("\n");
+    }
+    Tensor A({3, 4, 5}), B({3, 6, 5});
+    MatmulOp mm(&A, &B, false, true);
+    auto deps = mm.compute(DimRange(Dim{2, 1, 4})).first;
+    std::printf("matmul %d %d %d %d %d %d %d %d %d %d %d %d\n",
+                deps[0].getBegin()[0], deps[0].getBegin()[1], deps[0].getBegin()[2],
+                deps[0].getEnd()[0], deps[0].getEnd()[1], deps[0].getEnd()[2],
+                deps[1].getBegin()[0], deps[1].getBegin()[1], deps[1].getBegin()[2],
+                deps[1].getEnd()[0], deps[1].getEnd()[1], deps[1].getEnd()[2]);
+    return 0;
+}
+"""
+
+
+def test_point_dependences_match_numpy_index_maps(tmp_path):
+    import numpy as np
+    src = tmp_path / "deps.cc"
+    src.write_text(DEPENDENCE_PROGRAM)
+    exe = tmp_path / "deps"
+    subprocess.run(["g++", "-std=c++17", "-O1", str(src),
+                    "-I", os.path.join(ROOT, "pet_amd", "host", "include"),
+                    "-I", os.path.join(ROOT, "include"), "-L", LIB, "-lpet_host", "-lpet_hip",
+                    "-Wl,-rpath," + LIB, "-o", str(exe)], check=True)
+    run = subprocess.run([str(exe)], capture_output=True, text=True, timeout=60)
+    assert run.returncode == 0, (run.returncode, run.stdout, run.stderr)
+    got = {}
+    for line in run.stdout.splitlines():
+        name, *rest = line.split()
+        got[name] = rest
+
+    def offsets(name, which=None):
+        pairs = [t.split(":") for t in got[name]]
+        return [int(o) for i, o in pairs if which is None or int(i) == which]
+
+    x = np.arange(2 * 4 * 6 * 8).reshape(2, 4, 6, 8)
+    # the closed forms the reference gives for these rewrites
+    h2n = x.reshape(2, 4, 2, 3, 8).transpose(0, 2, 1, 3, 4).reshape(4, 4, 3, 8)
+    assert offsets("h2n") == h2n.ravel().tolist()
+    n2h = x.reshape(1, 2, 4, 6, 8).transpose(0, 2, 1, 3, 4).reshape(1, 4, 12, 8)
+    assert offsets("n2h") == n2h.ravel().tolist()
+    d2h = x.reshape(2, 4, 3, 2, 8).transpose(0, 1, 3, 2, 4).reshape(2, 4, 6, 8)
+    assert offsets("d2h") == d2h.ravel().tolist()
+    d2h_inv = x.reshape(2, 4, 2, 3, 8).transpose(0, 1, 3, 2, 4).reshape(2, 4, 6, 8)
+    assert offsets("d2hInv") == d2h_inv.ravel().tolist()
+    assert offsets("swap") == x.transpose(0, 1, 3, 2).ravel().tolist()
+
+    a = np.arange(24).reshape(2, 3, 4)
+    b = np.arange(40).reshape(2, 5, 4)
+    tagged = np.concatenate([a * 2, b * 2 + 1], axis=1).ravel()      # low bit = which input
+    pairs = [tuple(map(int, t.split(":"))) for t in got["concat"]]
+    assert [o * 2 + i for i, o in pairs] == tagged.tolist()
+    assert offsets("extend") == np.tile(a, (1, 3, 1)).ravel().tolist()
+    assert offsets("add", 0) == list(range(24))
+    assert offsets("add", 1) == [i % 4 for i in range(24)]
+    assert offsets("split0") == b[:, :2].ravel().tolist()
+    assert offsets("split1") == b[:, 2:].ravel().tolist()
+    # C[2,1,4] = sum_k A[2,1,k] * B[2,4,k] with B stored [b,n,k]
+    assert got["matmul"] == "2 1 0 2 1 4 2 4 0 2 4 4".split()
