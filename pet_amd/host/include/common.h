@@ -8,6 +8,7 @@
 #include <cmath>
 #include <cstdint>
 #include <cstdio>
+#include <cstdlib>
 #include <functional>
 #include <iostream>
 #include <map>
@@ -52,6 +53,28 @@ inline uint64_t hashAppend(uint64_t a, uint64_t b) {
 }
 inline uint64_t hashPack(uint64_t x) { return (x * 10000103ull) % 2147483647ull; }
 
+// Small integer helpers the mutators use (reference include/common.h:164-187).
+inline int gcd(int a, int b) {
+    while (b != 0) {
+        int t = a % b;
+        a = b;
+        b = t;
+    }
+    return a;
+}
+inline int gcd(const std::vector<int> &v) {
+    int g = v.empty() ? 1 : v[0];
+    for (int x : v)
+        g = gcd(g, x);
+    return g;
+}
+inline int max(const std::vector<int> &v) {
+    int m = 0;
+    for (size_t i = 0; i < v.size(); ++i)
+        m = i == 0 ? v[0] : std::max(m, v[i]);
+    return m;
+}
+
 // Every C-ABI status goes through here: the reference exits on a CUDA error
 // (include/common.h:30-38); this layer reports and lets the caller decide.
 inline bool petOk(int status, const char *what) {
@@ -59,6 +82,12 @@ inline bool petOk(int status, const char *what) {
         return true;
     std::fprintf(stderr, "[pet] %s failed (status %d): %s\n", what, status, pet_hip_last_error());
     return false;
+}
+
+// PET_HOST_TRACE=1: say on stderr why an operator or graph did not compute.
+inline bool hostTrace() {
+    static const bool on = std::getenv("PET_HOST_TRACE") != nullptr;
+    return on;
 }
 
 // One stream for the whole process (the reference uses the null stream).

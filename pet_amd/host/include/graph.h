@@ -113,9 +113,19 @@ class SubGraph : public GraphBase {
 
     // Runs every operator on the device in topological order.
     bool compute();
-    // One output value; computes the graph if that has not happened yet.
+    // One output value; computes on the device whatever part of the graph has
+    // not been computed yet. const like the reference's (the tensors it
+    // updates are reached through pointers).
     const std::pair<bool, VType> compute(const Dim &point, size_t outputId = 0,
-                                         bool getAllPos = false);
+                                         bool getAllPos = false) const;
+    // Re-wires the graph around a borrowed operator list whose tensors are the
+    // first `ntensor` (0: all) of this graph's tensors; false when an operator
+    // touches a tensor outside the graph (reference src/Graph/graph.cc:736-778).
+    // This is how the mutation generator reuses one scratch graph for every
+    // candidate it tries.
+    bool resetOps(OpVec oplist, size_t ntensor = 0);
+    void cleanConnection();
+    int findTensor(Tensor *tensor, int ntensor = 0);
     // Seeds both graphs' inputs with the same data, runs both on the device
     // and compares every output element for equality.
     bool verification(SubGraph *mutant_graph, bool isFullComputing = true);

@@ -279,6 +279,76 @@ class MatmulOp : public Operator {
     ActType act;
 };
 
+// ---- band matrix products (declared, not executed) --------------------------------
+// G2BMM (general x general -> band) and GBMML (band x general -> general) are the
+// Longformer attention products the reference runs through generated kernels
+// (include/custom_ops.cuh) and has no host evaluation for
+// (src/Graph/operator.cc:1365-1391). They are declared here, with the
+// reference's shape rules, so that code that names the classes builds; this
+// backend does not run them: launch() reports PET_HIP_ERR_UNSUPPORTED and perf()
+// returns INFINITY, the reference's convention for an operator a backend rejects.
+typedef std::tuple<int, int, int, int, int> G2BMMGBMMLArgs; // b, m, k, width, dilation
+
+class G2BMMOp : public Operator {
+  public:
+    G2BMMOp(Tensor *A, Tensor *B, Tensor *C, int width, int dilation, Tensor *bias = nullptr,
+            ActType act = None);
+    G2BMMOp(Tensor *A, Tensor *B, int width, int dilation, Tensor *bias = nullptr,
+            ActType act = None);
+    G2BMMOp(int width, int dilation, Tensor *bias = nullptr, ActType act = None);
+    G2BMMOp(const G2BMMOp &rhs)
+        : Operator(rhs), width(rhs.width), dilation(rhs.dilation), bias(rhs.bias), act(rhs.act) {}
+    G2BMMOp *clone() override { return new G2BMMOp(*this); }
+    Dim computeShape() override; // [b, m, 2 * width + 1]
+    double perf(PerfEngine *pe, int rounds = 200, int warmupRounds = 200) override;
+    int launch(pet_hip_stream_t stream) override;
+    std::string toString() const override;
+    int numInputs() override { return 2; }
+    int numOutputs() override { return 1; }
+    int getWidth() const { return width; }
+    int getDilation() const { return dilation; }
+    Tensor *getBias() const { return bias; }
+    void setAct(ActType a) { act = a; }
+    ActType getAct() const { return act; }
+    G2BMMGBMMLArgs getArgs() const;
+
+  private:
+    bool checkValid(const TensorVec &inputs) override;
+    void initHash() override;
+    int width, dilation;
+    Tensor *bias; // not part of the graph connections
+    ActType act;
+};
+
+class GBMMLOp : public Operator {
+  public:
+    GBMMLOp(Tensor *A, Tensor *B, Tensor *C, int dilation, Tensor *bias = nullptr,
+            ActType act = None);
+    GBMMLOp(Tensor *A, Tensor *B, int dilation, Tensor *bias = nullptr, ActType act = None);
+    GBMMLOp(int dilation, Tensor *bias = nullptr, ActType act = None);
+    GBMMLOp(const GBMMLOp &rhs)
+        : Operator(rhs), dilation(rhs.dilation), bias(rhs.bias), act(rhs.act) {}
+    GBMMLOp *clone() override { return new GBMMLOp(*this); }
+    Dim computeShape() override; // [b, m, k] from A[b, m, 2w+1], B[b, m, k]
+    double perf(PerfEngine *pe, int rounds = 200, int warmupRounds = 200) override;
+    int launch(pet_hip_stream_t stream) override;
+    std::string toString() const override;
+    int numInputs() override { return 2; }
+    int numOutputs() override { return 1; }
+    int getDilation() const { return dilation; }
+    Tensor *getBias() const { return bias; }
+    void setAct(ActType a) { act = a; }
+    ActType getAct() const { return act; }
+    G2BMMGBMMLArgs getArgs() const;
+
+  private:
+    bool checkValid(const TensorVec &inputs) override;
+    void initHash() override;
+    int dilation;
+    Tensor *bias;
+    ActType act;
+};
+
 // ---- Pad / Slice --------------------------------------------------------------
 class PadOp : public Operator {
   public:

@@ -66,7 +66,8 @@ class Tensor {
     bool dataMalloc();
     // Fills with the reference's LCG stream (include/tensor.h:371-374), one
     // thread's worth, reduced modulo `kRandMod` so that fp32 contractions of
-    // the values stay exact (the reference uses % 10000 in uint32).
+    // the values stay exact (the reference uses % 10000 in uint32). Seed 0
+    // continues a process-wide stream; other seeds are reproducible streams.
     bool dataRand(int seed = 0);
     static constexpr int kRandMod = 8;
     // Copies size() values from a host array to the device.
@@ -85,6 +86,9 @@ class Tensor {
     void aliasDevice(float *ptr);
     // Marks the device copy as just written by a kernel.
     void deviceWritten();
+    // Marks every tensor computed (directly or not) from this one as not
+    // computed; dataRand and setData call it.
+    void invalidateDependents();
 
     size_t getOffset(const Dim &pos) const; // (size_t)-1 when out of range
 

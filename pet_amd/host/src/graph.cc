@@ -2,6 +2,7 @@
 #include "perf_engine.h"
 
 #include <algorithm>
+#include <functional>
 #include <unordered_map>
 
 namespace tpm {
@@ -257,15 +258,101 @@ bool SubGraph::compute() {
     return petOk(pet_hip_stream_sync(petStream()), "pet_hip_stream_sync");
 }
 
-const std::pair<bool, VType> SubGraph::compute(const Dim &point, size_t outputId, bool) {
+const std::pair<bool, VType> SubGraph::compute(const Dim &point, size_t outputId, bool) const {
     if (outputId >= outputs.size())
         return {false, 0};
     Tensor *out = outputs[outputId];
-    if (!out->isComputed() && !compute())
+    if (!out->isComputed()) {
+        OpVec order;
+        if (!topoOrder(order))
+            return {false, 0};
+        for (auto op : order)
+            if (op->compute() == nullptr) {
+                if (hostTrace())
+                    std::fprintf(stderr, "[pet] graph point compute: %s failed\n",
+                                 op->toString().c_str());
+                return {false, 0};
+            }
+        if (!petOk(pet_hip_stream_sync(petStream()), "pet_hip_stream_sync"))
+            return {false, 0};
+    }
+    if (out->getOffset(point) == (size_t)-1) {
+        if (hostTrace())
+            std::fprintf(stderr, "[pet] graph point compute: point outside output %s\n",
+                         dimToString(out->getDims()).c_str());
         return {false, 0};
-    if (out->getOffset(point) == (size_t)-1)
-        return {false, 0};
-    return {true, out->getData(point)};
+    }
+    VType value = out->getData(point);
+    if (hostTrace())
+        std::fprintf(stderr, "[pet] graph %p output %zu %s at %s = %g\n", (const void *)this,
+                     outputId, dimToString(out->getDims()).c_str(), dimToString(point).c_str(),
+                     (double)value);
+    return {true, value};
+}
+
+void SubGraph::cleanConnection() {
+    for (auto t : tensors) {
+        t->setOutputOf(nullptr);
+        t->setInputOf({});
+    }
+    for (auto op : ops) {
+        op->setPredecessors({});
+        op->setSuccessors({});
+    }
+    inputs.clear();
+    outputs.clear();
+}
+
+int SubGraph::findTensor(Tensor *tensor, int ntensor) {
+    int n = ntensor == 0 ? (int)tensors.size() : std::min(ntensor, (int)tensors.size());
+    for (int i = 0; i < n; ++i)
+        if (tensors[i] == tensor)
+            return i;
+    return -1;
+}
+
+bool SubGraph::resetOps(OpVec oplist, size_t ntensor) {
+    ntensor = ntensor == 0 ? tensors.size() : std::min(ntensor, tensors.size());
+    hash = 2147483647;
+    cleanConnection();
+    ops = std::move(oplist);
+    for (auto op : ops) {
+        op->setPredecessors({});
+        op->setSuccessors({});
+    }
+    for (auto op : ops) {
+        for (auto t : op->getInputs()) {
+            if (findTensor(t) < 0)
+                return false;
+            t->addInputOf(op);
+        }
+        for (auto t : op->getOutputs()) {
+            if (findTensor(t) < 0)
+                return false;
+            t->setOutputOf(op);
+        }
+    }
+    for (size_t i = 0; i < ntensor; ++i) {
+        Tensor *t = tensors[i];
+        Operator *producer = t->getOutputOf();
+        for (auto consumer : t->getInputOf())
+            if (producer != nullptr) {
+                consumer->addPredecessors(producer);
+                producer->addSuccessors(consumer);
+            }
+        if (!t->getInputOf().empty() && producer == nullptr)
+            inputs.push_back(t);
+        if (t->getInputOf().empty() && producer != nullptr)
+            outputs.push_back(t);
+    }
+    if (hostTrace()) {
+        std::fprintf(stderr, "[pet] resetOps: %zu ops, %zu inputs, %zu outputs:", ops.size(),
+                     inputs.size(), outputs.size());
+        for (auto op : ops)
+            std::fprintf(stderr, " %s;", op->toString().c_str());
+        std::fprintf(stderr, "\n");
+    }
+    return true;
 }
 
 bool SubGraph::verification(SubGraph *mutant, bool) {
@@ -275,7 +362,7 @@ bool SubGraph::verification(SubGraph *mutant, bool) {
         Tensor *a = inputs[i], *b = mutant->getInputs()[i];
         if (a->size() != b->size())
             return false;
-        a->dataRand((int)i);
+        a->dataRand((int)i + 1);
         b->setData(a->getDataPtr());
     }
     resetComputed();
@@ -305,15 +392,33 @@ double SubGraph::perf(PerfEngine *pe, bool withPenalty) {
     return total;
 }
 
+// Wiring-aware hash (role of the reference's src/Graph/graph.cc:842-897): a
+// node's value folds its operator hash with, per input, the tensor hash of a
+// graph input or the value of the producing node; the graph's value folds the
+// output tensors with their producers. Two graphs with the same operators but
+// different connections hash differently, which the generator's visited-set
+// pruning relies on.
 uint64_t SubGraph::getHash() {
     if (hash != 2147483647)
         return hash;
+    std::unordered_map<const Operator *, uint64_t> memo;
+    std::function<uint64_t(Operator *)> nodeValue = [&](Operator *op) -> uint64_t {
+        auto it = memo.find(op);
+        if (it != memo.end())
+            return it->second;
+        memo[op] = 0; // a cycle would be a wiring bug; do not recurse forever
+        uint64_t h = hashPack(op->getHash());
+        for (auto t : op->getInputs()) {
+            Operator *producer = t->getOutputOf();
+            h = hashAppend(h, producer == nullptr ? t->getHash() : nodeValue(producer));
+        }
+        return memo[op] = hashPack(h);
+    };
     uint64_t h = 0;
-    OpVec order;
-    topoOrder(order);
-    for (auto op : order)
-        h = hashAppend(h, op->getHash());
-    hash = hashPack(h);
+    for (auto t : outputs)
+        if (t->getOutputOf() != nullptr)
+            h = hashAppend(h, hashPack(hashAppend(t->getHash(), nodeValue(t->getOutputOf()))));
+    hash = h;
     return hash;
 }
 

@@ -39,12 +39,23 @@ Tensor *Operator::compute() {
     if (done)
         return outputs[0];
     for (auto t : inputs)
-        if (t == nullptr || !t->isValid())
+        if (t == nullptr || !t->isValid()) {
+            if (hostTrace())
+                std::fprintf(stderr, "[pet] %s: invalid input\n", toString().c_str());
             return nullptr;
-    if (!allocOutputs())
+        }
+    if (!allocOutputs()) {
+        if (hostTrace())
+            std::fprintf(stderr, "[pet] %s: output allocation failed\n", toString().c_str());
         return nullptr;
-    if (launch(petStream()) != PET_HIP_OK)
+    }
+    int status = launch(petStream());
+    if (status != PET_HIP_OK) {
+        if (hostTrace())
+            std::fprintf(stderr, "[pet] %s: launch status %d: %s\n", toString().c_str(), status,
+                         pet_hip_last_error());
         return nullptr;
+    }
     for (auto t : outputs) {
         t->deviceWritten();
         t->setComputed();
@@ -1326,15 +1337,14 @@ ReshapeOp::ReshapeOp(OpType type, Tensor *input, Tensor *output)
     : Operator(type, {input}, {output}) {
     initHash();
 }
-ReshapeOp::ReshapeOp(Tensor *input, Tensor *output) : ReshapeOp(Reshape, input, output) {
-    assert(checkValid({input}));
-}
+ReshapeOp::ReshapeOp(Tensor *input, Tensor *output) : ReshapeOp(Reshape, input, output) {}
 
 void ReshapeOp::initHash() { hash = hashPack(type); }
 
-bool ReshapeOp::checkValid(const TensorVec &ins) {
-    return outputs.size() == 1 && ins[0]->size() == outputs[0]->size();
-}
+// Always valid, as in the reference (include/operator.h:1788): callers build the
+// operator first and give the output its dims afterwards
+// (src/Mutant/generator.cc:1455-1457). launch() rejects a size mismatch.
+bool ReshapeOp::checkValid(const TensorVec &) { return true; }
 
 Dim ReshapeOp::computeShape() {
     outputs[0]->setType(inputs[0]->getType());
@@ -1361,6 +1371,114 @@ double ReshapeOp::perf(PerfEngine *, int, int) { return 0.0; }
 std::string ReshapeOp::toString() const {
     return getOpName(type) + "(" + dimToString(inputs[0]->getDims()) + "->" +
            dimToString(outputs[0]->getDims()) + ")";
+}
+
+// ---- band matrix products: shape rules only ------------------------------------
+G2BMMOp::G2BMMOp(Tensor *A, Tensor *B, Tensor *C, int width, int dilation, Tensor *bias,
+                 ActType act)
+    : Operator(G2BMM, {A, B}, {C}), width(width), dilation(dilation), bias(bias), act(act) {
+    if (A->getType() == Tensor::Input && B->getType() == Tensor::Input)
+        B->setType(Tensor::Weight);
+    assert(checkValid({A, B}));
+    computeShape();
+    initHash();
+}
+
+G2BMMOp::G2BMMOp(Tensor *A, Tensor *B, int width, int dilation, Tensor *bias, ActType act)
+    : G2BMMOp(A, B, new Tensor(), width, dilation, bias, act) {}
+
+G2BMMOp::G2BMMOp(int width, int dilation, Tensor *bias, ActType act)
+    : Operator(G2BMM), width(width), dilation(dilation), bias(bias), act(act) {
+    initHash();
+}
+
+G2BMMGBMMLArgs G2BMMOp::getArgs() const {
+    if (inputs.empty())
+        return G2BMMGBMMLArgs{0, 0, 0, width, dilation};
+    const Dim &a = inputs[0]->getDims();
+    return G2BMMGBMMLArgs{a[0], a[1], a[2], width, dilation};
+}
+
+void G2BMMOp::initHash() {
+    auto [b, m, k, w, d] = getArgs();
+    hash = type;
+    for (int v : {b, m, k, w, d})
+        hash = hashAppend(hash, (uint64_t)(int64_t)v);
+    hash = hashPack(hash);
+}
+
+bool G2BMMOp::checkValid(const TensorVec &ins) {
+    const Tensor *A = ins[0], *B = ins[1];
+    if (A->getType() == Tensor::Weight && B->getType() == Tensor::Weight)
+        return false;
+    return A->getDims().size() == 3 && A->getDims() == B->getDims() && width >= 0;
+}
+
+Dim G2BMMOp::computeShape() {
+    const Dim &a = inputs[0]->getDims();
+    Dim ret = {a[0], a[1], 2 * width + 1};
+    outputs[0]->setDims(ret);
+    outputs[0]->setType(Tensor::Input);
+    return ret;
+}
+
+int G2BMMOp::launch(pet_hip_stream_t) { return PET_HIP_ERR_UNSUPPORTED; }
+double G2BMMOp::perf(PerfEngine *, int, int) { return INFINITY; }
+std::string G2BMMOp::toString() const {
+    return "G2BMM(width=" + std::to_string(width) + ",dilation=" + std::to_string(dilation) + ")";
+}
+
+GBMMLOp::GBMMLOp(Tensor *A, Tensor *B, Tensor *C, int dilation, Tensor *bias, ActType act)
+    : Operator(GBMML, {A, B}, {C}), dilation(dilation), bias(bias), act(act) {
+    if (A->getType() == Tensor::Input && B->getType() == Tensor::Input)
+        B->setType(Tensor::Weight);
+    assert(checkValid({A, B}));
+    computeShape();
+    initHash();
+}
+
+GBMMLOp::GBMMLOp(Tensor *A, Tensor *B, int dilation, Tensor *bias, ActType act)
+    : GBMMLOp(A, B, new Tensor(), dilation, bias, act) {}
+
+GBMMLOp::GBMMLOp(int dilation, Tensor *bias, ActType act)
+    : Operator(GBMML), dilation(dilation), bias(bias), act(act) {
+    initHash();
+}
+
+G2BMMGBMMLArgs GBMMLOp::getArgs() const {
+    if (inputs.size() < 2)
+        return G2BMMGBMMLArgs{0, 0, 0, 0, dilation};
+    const Dim &a = inputs[0]->getDims();
+    return G2BMMGBMMLArgs{a[0], a[1], inputs[1]->getDims()[2], (a[2] - 1) / 2, dilation};
+}
+
+void GBMMLOp::initHash() {
+    auto [b, m, k, w, d] = getArgs();
+    hash = type;
+    for (int v : {b, m, k, w, d})
+        hash = hashAppend(hash, (uint64_t)(int64_t)v);
+    hash = hashPack(hash);
+}
+
+bool GBMMLOp::checkValid(const TensorVec &ins) {
+    const Tensor *A = ins[0], *B = ins[1];
+    if (A->getType() == Tensor::Weight && B->getType() == Tensor::Weight)
+        return false;
+    const Dim &a = A->getDims(), &b = B->getDims();
+    return a.size() == 3 && b.size() == 3 && a[0] == b[0] && a[1] == b[1] && a[2] % 2 == 1;
+}
+
+Dim GBMMLOp::computeShape() {
+    Dim ret = {inputs[0]->getDims()[0], inputs[0]->getDims()[1], inputs[1]->getDims()[2]};
+    outputs[0]->setDims(ret);
+    outputs[0]->setType(Tensor::Input);
+    return ret;
+}
+
+int GBMMLOp::launch(pet_hip_stream_t) { return PET_HIP_ERR_UNSUPPORTED; }
+double GBMMLOp::perf(PerfEngine *, int, int) { return INFINITY; }
+std::string GBMMLOp::toString() const {
+    return "GBMML(dilation=" + std::to_string(dilation) + ")";
 }
 
 // ---- point dependences ------------------------------------------------------------

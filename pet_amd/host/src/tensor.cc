@@ -119,17 +119,37 @@ bool Tensor::dataMalloc() {
     return true;
 }
 
+// New values in this tensor make everything computed from it stale. The
+// reference re-evaluates a requested point from the current inputs every time
+// (src/Graph/graph.cc:780-842); here results are kept on the device, so the
+// invalidation is explicit.
+void Tensor::invalidateDependents() {
+    for (auto op : inputOf)
+        for (auto out : op->getOutputs())
+            if (out != this && out->computed != NotComputed) {
+                out->computed = NotComputed;
+                out->invalidateDependents();
+            }
+}
+
 bool Tensor::dataRand(int seed) {
     // one stream of the 214013 / 2531011 generator, reduced to small integers
+    // seed 0 (the default) continues one process-wide stream, so that tensors
+    // filled one after another differ, as with the reference's persistent
+    // generator state; any other seed starts a reproducible stream of its own.
+    static int shared = 0;
     host.resize(size());
-    int g = seed;
+    int g = seed == 0 ? shared : seed;
     for (size_t i = 0; i < host.size(); ++i) {
         g = (int)(214013u * (unsigned)g + 2531011u);
         host[i] = (VType)(((g >> 16) & 0x7FFF) % kRandMod);
     }
+    if (seed == 0)
+        shared = g;
     hostFresh = true;
     devFresh = false;
     computed = ComputedFull;
+    invalidateDependents();
     return true;
 }
 
@@ -140,6 +160,7 @@ bool Tensor::setData(const VType *hostPtr) {
     hostFresh = true;
     devFresh = false;
     computed = ComputedFull;
+    invalidateDependents();
     return true;
 }
 
@@ -245,6 +266,7 @@ bool Tensor::setData(size_t pos, VType val) {
     if (pos >= size())
         return false;
     getDataPtr()[pos] = val;
+    invalidateDependents();
     return true;
 }
 

@@ -241,3 +241,61 @@ def test_point_dependences_match_numpy_index_maps(tmp_path):
     assert offsets("split1") == b[:, 2:].ravel().tolist()
     # C[2,1,4] = sum_k A[2,1,k] * B[2,4,k] with B stored [b,n,k]
     assert got["matmul"] == "2 1 0 2 1 4 2 4 0 2 4 4".split()
+
+
+# ---- the reference's own mutation generator on this backend ----------------------
+# libpet_refsearch.so is the reference's src/Mutant/generator.cc, reciprocity.cc and
+# src/Graph/trans_eliminator.cc compiled unchanged against pet_amd/host/include
+# (make -C pet_amd/host refsearch, run where the reference tree is present; the
+# binaries travel with the tree). The programs under pet_amd/lib/refsearch are the
+# reference's src/Test/single_rule_test_*.cc, also unchanged.
+REFSEARCH = os.path.join(LIB, "libpet_refsearch.so")
+GENERATOR_DRIVER = os.path.join(LIB, "pet_generator_driver")
+needs_refsearch = pytest.mark.skipif(not os.path.exists(REFSEARCH),
+                                     reason="libpet_refsearch.so was not built")
+
+# program -> candidates the generator must at least find. The assertions inside
+# the programs were written for an earlier generator: at the reference's head the
+# input graph itself is no longer added to the candidates
+# (src/Mutant/generator.cc:23) and candidates deeper than max_depth are dropped
+# (:1960-1964), so most of their counts are one higher than the head can give
+# and the preprocess-only rules (6, 13, 15) give none.
+SINGLE_RULE_PROGRAMS = {
+    "single_rule_test_1_n2h": 2, "single_rule_test_2_n2w": 2, "single_rule_test_3_c2h": 2,
+    "single_rule_test_4_c2w": 2, "single_rule_test_5_dilated": 1,
+    "single_rule_test_7_trans_gemm": 1, "single_rule_test_8_conv2group": 1,
+    "single_rule_test_9_group_conv_a": 1, "single_rule_test_12_1xk_trans": 1,
+    "single_rule_test_14_split_group_conv": 4, "single_rule_test_16_group_conv_d": 1,
+}
+
+
+@pytest.mark.gpu
+@needs_refsearch
+@pytest.mark.parametrize("program", sorted(SINGLE_RULE_PROGRAMS))
+def test_reference_single_rule_program_finds_mutants_on_the_device(program):
+    import re
+    exe = os.path.join(LIB, "refsearch", program)
+    res = subprocess.run([exe], capture_output=True, text=True, timeout=300)
+    print(res.stdout[-3000:])
+    print(res.stderr[-2000:])
+    # 0: the program's own assertion held; 134 (-6): it aborted on its assertion
+    assert res.returncode in (0, -6, 134), res.returncode
+    found = re.findall(r"candidates found: (\d+)", res.stdout)
+    assert found, "the program did not reach its report"
+    assert int(found[-1]) >= SINGLE_RULE_PROGRAMS[program]
+    if res.returncode != 0:
+        assert "candidates.size()" in res.stderr      # nothing but the stale count
+
+
+@pytest.mark.gpu
+@needs_refsearch
+@pytest.mark.parametrize("args", [
+    "1 64 56 56 64 3 1 1 1",       # benchmark configuration 1: needs an exact candidate
+    "1 32 32 32 32 3 2 2 0",       # dilated convolution: de-interleave candidates, partial
+])
+def test_generator_candidates_run_and_are_ranked_on_the_device(args):
+    res = subprocess.run([GENERATOR_DRIVER] + args.split(), capture_output=True, text=True,
+                         timeout=600)
+    print(res.stdout[-6000:])
+    print(res.stderr[-2000:])
+    assert res.returncode == 0
