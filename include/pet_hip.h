@@ -136,6 +136,26 @@ PET_HIP_API int pet_hip_conv3d_f32(const float *x, const float *w, const float *
                        int pt, int ph, int pw, int st, int sh, int sw, int dt, int dh,
                        int dw, int groups, int act, pet_hip_stream_t stream);
 
+/* Constant 3-D filters, reordered once: [f][c/groups][kt][r][s] -> kt-major
+ * [kt][f][c/groups][r][s] (same element count), so that each kt slice is a 2-D
+ * filter bank the convolution kernel reads with 16-byte loads. This is a
+ * single-input operator on a Weight tensor, i.e. what the reference's emitted
+ * program runs once before its timed loop ("Preprocess operators for weights",
+ * src/Graph/code_engine.cc:187-193). Returns PET_HIP_ERR_UNSUPPORTED, writing
+ * nothing, for shapes that would not profit (kt == 1, or filters other than
+ * 3x3 with c/groups % 8 == 0 and 1x1 with c/groups % 32 == 0): keep calling
+ * pet_hip_conv3d_f32 for those. */
+PET_HIP_API int pet_hip_conv3d_pack_filters(const float *w, float *packed, int f, int cpg, int kt,
+                                int r, int s, pet_hip_stream_t stream);
+
+/* pet_hip_conv3d_f32 on filters reordered by pet_hip_conv3d_pack_filters; same
+ * arguments and results. PET_HIP_ERR_UNSUPPORTED for the shapes that function
+ * rejects. */
+PET_HIP_API int pet_hip_conv3d_packed_f32(const float *x, const float *packed, const float *bias,
+                              float *y, int n, int c, int t, int h, int wd, int f, int kt, int r,
+                              int s, int pt, int ph, int pw, int st, int sh, int sw, int dt,
+                              int dh, int dw, int groups, int act, pet_hip_stream_t stream);
+
 /* Batched row-major matmul C[b,m,n] = A'[b,m,k] * B'[b,k,n]; transA: A stored
  * [b,k,m]; transB: B stored [b,n,k]. bias (may be NULL) is [n], added per
  * output column. Semantics: MatmulOp::compute, src/Graph/operator.cc:620-654;

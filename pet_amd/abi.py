@@ -46,6 +46,8 @@ SIGNATURES = {
     "pet_hip_conv_out_dim": [_i] * 5,
     "pet_hip_conv2d_f32": [_vp] * 4 + [_i] * 15 + [_vp],
     "pet_hip_conv3d_f32": [_vp] * 4 + [_i] * 20 + [_vp],
+    "pet_hip_conv3d_pack_filters": [_vp, _vp] + [_i] * 5 + [_vp],
+    "pet_hip_conv3d_packed_f32": [_vp] * 4 + [_i] * 20 + [_vp],
     "pet_hip_bmm_f32": [_i] * 6 + [_vp] * 4 + [_i, _vp],
     "pet_hip_transpose": [_vp, _vp, _c_int_p, _c_int_p, _i, _vp],
     "pet_hip_trans_chain": [_vp, _vp, _c_int_p, _i, _c_int_p, _i, _c_int_p, _c_int_p, _c_int_p, _vp],

@@ -42,6 +42,7 @@ struct ConvParams {
     FastDiv fd_sk_wgs, fd_sk_nit, fd_sk_tm;
     int atomic_out; // partial sums are added into y with float atomics
     int vec_out;   // plane kernel: OPIX % 4 == 0 and y 16-byte aligned: 16-byte output words
+    int wpacked;   // 3-D filters are stored kt-major, [kt][f][c/g][r][s] (plane kernel only)
     int sk_mode;   // split-K: 0 partial tiles + ordered sum in one launch, 1 atomics into y
     float *ws;     // split-K: partial tiles, [tile][split][register][thread]
     int *cnt;      // split-K: arrival counter per tile, zero between launches
@@ -319,11 +320,14 @@ constexpr unsigned kOob = 0x80000000u; // voffset that the range check rejects
 
 // DIM 2: 2-D. DIM 3: 3-D with kt > 1 (one kt slice of a filter row is runs of r*s
 // floats, loaded one float at a time). DIM 4: 3-D with kt == 1 (filter rows are
-// contiguous as in 2-D and load as 16-byte words).
+// contiguous as in 2-D and load as 16-byte words). DIM 5: 3-D with kt > 1 and
+// filters repacked kt-major, [kt][f][c/g][r][s]: every kt slice is a 2-D filter
+// bank and loads as 16-byte words.
 template <class Cfg, int DIM, bool SK>
 __global__ __launch_bounds__(Cfg::NT) void conv_plane_kernel(ConvParams p) {
     constexpr bool IS3D = DIM != 2;
     constexpr bool SCALAR_A = DIM == 3;
+    constexpr bool PACKED = DIM == 5;
     extern __shared__ __attribute__((aligned(16))) float lds[];
     constexpr int KH = Cfg::KH, TM = Cfg::TM, TN = Cfg::TN, RS = Cfg::RS, CB = Cfg::CB;
     constexpr int BK = Cfg::BK, NT = Cfg::NT, NW = Cfg::NW;
@@ -393,7 +397,9 @@ __global__ __launch_bounds__(Cfg::NT) void conv_plane_kernel(ConvParams p) {
     // bases: the pad offset is folded into the image base so every voffset is >= 0
     const int padoff = p.pt * HW + p.ph * p.W + p.pw;
     const float *xg = p.x + (long long)g * p.cpg * THW - padoff;
-    const float *wg = p.w + (long long)g * p.M * p.K;
+    // floats per filter row as stored: all of K, or one kt slice of it when packed
+    const int a_row = PACKED ? p.cpg * RS : p.K;
+    const float *wg = p.w + (long long)g * p.M * a_row;
 
     // ---- per-thread invariants of the B gather
     unsigned voffB[RPW][PPL];
@@ -473,7 +479,7 @@ __global__ __launch_bounds__(Cfg::NT) void conv_plane_kernel(ConvParams p) {
             const int v = tid + i * NT;
             const int row = v / (BK / 4), kq = (v % (BK / 4)) * 4;
             voffA[i] = v < Cfg::A_V4
-                           ? ((unsigned)min(m0 + row, p.M - 1) * (unsigned)p.K + kq) * 4u
+                           ? ((unsigned)min(m0 + row, p.M - 1) * (unsigned)a_row + kq) * 4u
                            : kOob;
             ldsA[i] = min(row, Cfg::BM - 1) * A_LD + kq;
         }
@@ -512,7 +518,8 @@ __global__ __launch_bounds__(Cfg::NT) void conv_plane_kernel(ConvParams p) {
     // ---- pieces ---------------------------------------------------------------
     auto g_piece = [&](int i) __attribute__((always_inline)) {
         if (i < NA) {
-            const unsigned so = (unsigned)(pcb * CB * KRS + pq * RS) * 4u;
+            const unsigned so = PACKED ? (unsigned)(pq * (p.F * a_row) + pcb * CB * RS) * 4u
+                                       : (unsigned)(pcb * CB * KRS + pq * RS) * 4u;
             const __amdgpu_buffer_rsrc_t ra = make_rsrc(wg);
             if (SCALAR_A) {
                 preA1[i] = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(ra, voffA[i], so, 0));
@@ -1010,18 +1017,21 @@ int launch_plane(const ConvParams &p, bool is3d, hipStream_t stream) {
         tile = 0;
     if (forced_tile() >= 0)
         tile = forced_tile() % 3;
-    const int dim = !is3d ? 2 : (p.KT == 1 ? 4 : 3);
+    const int dim = !is3d ? 2 : (p.KT == 1 ? 4 : (p.wpacked ? 5 : 3));
     if (tile == 0)
         return dim == 2   ? launch_plane_cfg<C64x128, 2>(p, stream)
                : dim == 3 ? launch_plane_cfg<C64x128, 3>(p, stream)
-                          : launch_plane_cfg<C64x128, 4>(p, stream);
+               : dim == 4 ? launch_plane_cfg<C64x128, 4>(p, stream)
+                          : launch_plane_cfg<C64x128, 5>(p, stream);
     if (tile == 1)
         return dim == 2   ? launch_plane_cfg<C64x64, 2>(p, stream)
                : dim == 3 ? launch_plane_cfg<C64x64, 3>(p, stream)
-                          : launch_plane_cfg<C64x64, 4>(p, stream);
+               : dim == 4 ? launch_plane_cfg<C64x64, 4>(p, stream)
+                          : launch_plane_cfg<C64x64, 5>(p, stream);
     return dim == 2   ? launch_plane_cfg<C32x64, 2>(p, stream)
            : dim == 3 ? launch_plane_cfg<C32x64, 3>(p, stream)
-                      : launch_plane_cfg<C32x64, 4>(p, stream);
+           : dim == 4 ? launch_plane_cfg<C32x64, 4>(p, stream)
+                      : launch_plane_cfg<C32x64, 5>(p, stream);
 }
 
 // Returns -1 when the plane kernel does not apply.
@@ -1044,10 +1054,33 @@ int try_launch_plane(const ConvParams &p, hipStream_t stream) {
     return -1;
 }
 
+// Shapes whose kt slices the plane kernel reads as 2-D filter banks.
+bool packed_filters_apply(long long f, int cpg, int kt, int r, int s) {
+    static const bool off = getenv("PET_HIP_PLANE") && atoi(getenv("PET_HIP_PLANE")) == 0;
+    if (off || kt <= 1 || 4ll * f * cpg * kt * r * s >= (1ll << 31))
+        return false;
+    return (r == 3 && s == 3 && cpg % 8 == 0) || (r == 1 && s == 1 && cpg % 32 == 0);
+}
+
+__global__ void pack_filters_kernel(const float *__restrict__ w, float *__restrict__ out,
+                                    unsigned rows, unsigned kt, unsigned rs) {
+    // out[q][row][t] = w[row][q][t], row = f * cpg + c
+    const unsigned total = rows * kt * rs;
+    for (unsigned i = blockIdx.x * blockDim.x + threadIdx.x; i < total;
+         i += gridDim.x * blockDim.x) {
+        const unsigned t = i % rs, row = (i / rs) % rows, q = i / (rs * rows);
+        out[i] = w[(row * kt + q) * rs + t];
+    }
+}
+
 int launch_conv(ConvParams &p, hipStream_t stream) {
     int rc = try_launch_plane(p, stream);
     if (rc >= 0)
         return rc;
+    if (p.wpacked)
+        return set_error(PET_HIP_ERR_UNSUPPORTED,
+                         "kt-major filters are only read by the plane kernel; this shape does "
+                         "not use it (pet_hip_conv3d_pack_filters would have said so)");
     const bool veca = (p.K % 4 == 0) && (((uintptr_t)p.w & 15) == 0);
     switch (pick_tile(p.M, p.NPIX, p.G)) {
     case 0:
@@ -1063,7 +1096,8 @@ int launch_conv(ConvParams &p, hipStream_t stream) {
 
 int conv_common(const float *x, const float *w, const float *bias, float *y, int n, int c, int t,
                 int h, int wd, int f, int kt, int r, int s, int pt, int ph, int pw, int st, int sh,
-                int sw, int dt, int dh, int dw, int groups, int act, hipStream_t stream) {
+                int sw, int dt, int dh, int dw, int groups, int act, hipStream_t stream,
+                bool wpacked = false) {
     if (n < 0 || c <= 0 || t <= 0 || h <= 0 || wd <= 0 || f <= 0 || kt <= 0 || r <= 0 || s <= 0 ||
         groups <= 0 || st <= 0 || sh <= 0 || sw <= 0 || dt <= 0 || dh <= 0 || dw <= 0 || pt < 0 ||
         ph < 0 || pw < 0)
@@ -1125,6 +1159,9 @@ int conv_common(const float *x, const float *w, const float *bias, float *y, int
     p.act = act;
     p.bias_mode = 1;
     p.splitk = 1;
+    p.wpacked = wpacked;
+    if (wpacked && !packed_filters_apply(f, c / groups, kt, r, s))
+        return set_error(PET_HIP_ERR_UNSUPPORTED, "no kt-major form for this filter shape");
     p.fd_krs = make_fastdiv((unsigned)(kt * r * s));
     p.fd_rs = make_fastdiv((unsigned)(r * s));
     p.fd_s = make_fastdiv((unsigned)s);
@@ -1203,6 +1240,31 @@ int pet_hip_conv3d_f32(const float *x, const float *w, const float *bias, float 
     PET_REQUIRE_INIT();
     return conv_common(x, w, bias, y, n, c, t, h, wd, f, kt, r, s, pt, ph, pw, st, sh, sw, dt, dh,
                        dw, groups, act, as_stream(stream));
+}
+
+int pet_hip_conv3d_pack_filters(const float *w, float *packed, int f, int cpg, int kt, int r,
+                                int s, pet_hip_stream_t stream) {
+    PET_REQUIRE_INIT();
+    if (f <= 0 || cpg <= 0 || kt <= 0 || r <= 0 || s <= 0)
+        return set_error(PET_HIP_ERR_INVALID, "bad filter shape");
+    if (!packed_filters_apply(f, cpg, kt, r, s))
+        return set_error(PET_HIP_ERR_UNSUPPORTED, "no kt-major form for this filter shape");
+    if (!w || !packed || w == packed)
+        return set_error(PET_HIP_ERR_INVALID, "filters and their packed copy must be two buffers");
+    const unsigned rows = (unsigned)f * (unsigned)cpg, total = rows * kt * r * s;
+    const unsigned blocks = std::min<unsigned>((total + 255) / 256, 4096);
+    hipLaunchKernelGGL(pack_filters_kernel, dim3(blocks), dim3(256), 0, as_stream(stream), w,
+                       packed, rows, (unsigned)kt, (unsigned)(r * s));
+    return check_launch("pack_filters_kernel");
+}
+
+int pet_hip_conv3d_packed_f32(const float *x, const float *packed, const float *bias, float *y,
+                              int n, int c, int t, int h, int wd, int f, int kt, int r, int s,
+                              int pt, int ph, int pw, int st, int sh, int sw, int dt, int dh,
+                              int dw, int groups, int act, pet_hip_stream_t stream) {
+    PET_REQUIRE_INIT();
+    return conv_common(x, packed, bias, y, n, c, t, h, wd, f, kt, r, s, pt, ph, pw, st, sh, sw, dt,
+                       dh, dw, groups, act, as_stream(stream), true);
 }
 
 } // extern "C"

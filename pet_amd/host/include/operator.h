@@ -218,7 +218,15 @@ class Conv3dOp : public Operator {
     Conv3dOp(Tensor *input, Tensor *weight, Tensor *output, const Dim &pad, const Dim &stride,
              const Dim &dilation, Tensor *bias = nullptr, ActType act = None);
     Conv3dOp(const Conv3dOp &rhs);
+    ~Conv3dOp() override;
     Conv3dOp *clone() override { return new Conv3dOp(*this); }
+    // Weight preprocessing, run once by whoever treats the filters as constants
+    // (CodeEngine before it captures a graph): keeps a kt-major copy of the
+    // filters that launch() then reads through pet_hip_conv3d_packed_f32 for as
+    // long as the weight tensor is not written again. False (and no copy) when
+    // the backend has no such form for this shape.
+    bool prepackFilters(pet_hip_stream_t stream);
+    bool usesPackedFilters() const;
     Dim computeShape() override;
     double perf(PerfEngine *pe, int rounds = 200, int warmupRounds = 200) override;
     int launch(pet_hip_stream_t stream) override;
@@ -238,6 +246,9 @@ class Conv3dOp : public Operator {
     Dim pad, stride, dilation; // (t, h, w)
     Tensor *bias;
     ActType act;
+    float *packed = nullptr;     // kt-major filters, owned
+    size_t packedElems = 0;
+    uint64_t packedVersion = 0;  // weight tensor's dataVersion() the copy was made from
 };
 
 // ---- Matmul -------------------------------------------------------------------

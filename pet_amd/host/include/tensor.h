@@ -86,6 +86,10 @@ class Tensor {
     void aliasDevice(float *ptr);
     // Marks the device copy as just written by a kernel.
     void deviceWritten();
+    // Counts the writes to this tensor's values (dataRand, setData, a kernel's
+    // output, a host pointer handed out): lets a holder of derived data, such as
+    // repacked filters, see that it is out of date.
+    uint64_t dataVersion() const { return version; }
     // Marks every tensor computed (directly or not) from this one as not
     // computed; dataRand and setData call it.
     void invalidateDependents();
@@ -130,6 +134,7 @@ class Tensor {
     std::vector<VType> host;
     bool hostFresh = false; // host mirror holds the current values
     bool devFresh = false;  // device buffer holds the current values
+    uint64_t version = 0;
 };
 
 void printTensor(Tensor *tensor);

@@ -2,6 +2,7 @@
 
 #include <algorithm>
 #include <fstream>
+#include <map>
 #include <set>
 #include <sstream>
 #include <unordered_map>
@@ -160,6 +161,11 @@ std::unique_ptr<GraphExec> CodeEngine::instantiate(std::shared_ptr<SubGraph> &gr
             for (auto t : op->getOutputs())
                 t->deviceWritten();
         }
+    // constant 3-D filters get their kt-major copy here, once, for the same reason
+    for (auto op : order)
+        if (auto c3 = dynamic_cast<Conv3dOp *>(op))
+            if (c3->getInputs()[1]->getType() == Tensor::Weight && !plan.skipped.count(op))
+                c3->prepackFilters(s);
     if (!petOk(pet_hip_stream_sync(s), "pet_hip_stream_sync"))
         return nullptr;
     if (!petOk(pet_hip_graph_begin_capture(s), "pet_hip_graph_begin_capture"))
@@ -315,6 +321,7 @@ std::string CodeEngine::genCode(std::shared_ptr<SubGraph> &graph) {
     for (auto &l : aliasLines)
         e.line(l);
 
+    std::map<const Operator *, std::string> packedName; // Conv3d -> its kt-major filter copy
     auto emitOp = [&](Operator *op) -> bool {
         std::ostringstream c;
         auto in = [&](size_t i) { return e.name(op->getInputs()[i]); };
@@ -329,8 +336,14 @@ std::string CodeEngine::genCode(std::shared_ptr<SubGraph> &graph) {
               << d[1] / w[1] << ", " << (int)conv->getAct() << ", s)";
         } else if (auto c3 = dynamic_cast<Conv3dOp *>(op)) {
             auto d = op->getInputs()[0]->getDims(), w = op->getInputs()[1]->getDims();
-            c << "pet_hip_conv3d_f32(" << in(0) << ", " << in(1) << ", "
-              << nullable(e, c3->getBias()) << ", " << out(0);
+            // filters with a kt-major copy (made before capture, below) use it
+            if (packedName.count(op))
+                c << "(" << packedName[op] << "_ok ? pet_hip_conv3d_packed_f32 : "
+                  << "pet_hip_conv3d_f32)(" << in(0) << ", " << packedName[op] << "_ok ? "
+                  << packedName[op] << " : " << in(1) << ", ";
+            else
+                c << "pet_hip_conv3d_f32(" << in(0) << ", " << in(1) << ", ";
+            c << nullable(e, c3->getBias()) << ", " << out(0);
             for (int v : {d[0], d[1], d[2], d[3], d[4], w[0], w[2], w[3], w[4]})
                 c << ", " << v;
             for (const Dim *v : {&c3->getPad(), &c3->getStride(), &c3->getDilation()})
@@ -454,6 +467,22 @@ std::string CodeEngine::genCode(std::shared_ptr<SubGraph> &graph) {
     for (auto op : order)
         if (weightOnly(op) && !skipped.count(op) && !emitOp(op))
             return "";
+    e.line("    // constant 3-D filters: kt-major copy where the backend has that form");
+    for (auto op : order) {
+        auto c3 = dynamic_cast<Conv3dOp *>(op);
+        if (!c3 || skipped.count(op) || op->getInputs()[1]->getType() != Tensor::Weight)
+            continue;
+        Tensor *w = op->getInputs()[1];
+        const Dim &wd = w->getDims();
+        std::string n = e.name(w) + "_kt" + std::to_string(packedName.size());
+        packedName[op] = n;
+        std::ostringstream l;
+        l << "    float *" << n << "; CHECK(pet_hip_malloc((void **)&" << n << ", " << w->size()
+          << " * sizeof(float))); int " << n << "_ok = pet_hip_conv3d_pack_filters(" << e.name(w)
+          << ", " << n << ", " << wd[0] << ", " << wd[1] << ", " << wd[2] << ", " << wd[3] << ", "
+          << wd[4] << ", s) == PET_HIP_OK;";
+        e.line(l.str());
+    }
     e.line("    CHECK(pet_hip_stream_sync(s));");
     e.line("    // the rest is captured once and replayed as a HIP graph");
     e.line("    CHECK(pet_hip_graph_begin_capture(s));");

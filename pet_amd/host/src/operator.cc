@@ -366,6 +366,43 @@ Conv3dOp::Conv3dOp(const Conv3dOp &rhs)
     : Operator(rhs), pad(rhs.pad), stride(rhs.stride), dilation(rhs.dilation), bias(rhs.bias),
       act(rhs.act) {}
 
+Conv3dOp::~Conv3dOp() {
+    if (packed)
+        pet_hip_free(packed);
+}
+
+bool Conv3dOp::usesPackedFilters() const {
+    return packed != nullptr && packedElems == inputs[1]->size() &&
+           packedVersion == inputs[1]->dataVersion();
+}
+
+bool Conv3dOp::prepackFilters(pet_hip_stream_t stream) {
+    Tensor *w = inputs[1];
+    const Dim &wt = w->getDims();
+    const float *src = w->devicePtr(); // settles the upload, and with it the version
+    if (src == nullptr)
+        return false;
+    if (packed == nullptr || packedElems != w->size()) {
+        if (packed)
+            pet_hip_free(packed);
+        packed = nullptr;
+        void *buf = nullptr;
+        if (pet_hip_malloc(&buf, w->size() * sizeof(float)) != PET_HIP_OK)
+            return false;
+        packed = (float *)buf;
+        packedElems = w->size();
+    }
+    int rc = pet_hip_conv3d_pack_filters(src, packed, wt[0], wt[1], wt[2], wt[3], wt[4], stream);
+    if (rc != PET_HIP_OK) { // PET_HIP_ERR_UNSUPPORTED: this shape keeps its layout
+        pet_hip_free(packed);
+        packed = nullptr;
+        packedElems = 0;
+        return false;
+    }
+    packedVersion = w->dataVersion();
+    return true;
+}
+
 void Conv3dOp::initHash() {
     hash = type;
     hash = hashDims(hashDims(hashDims(hash, pad), stride), dilation);
@@ -395,11 +432,16 @@ int Conv3dOp::launch(pet_hip_stream_t stream) {
     int groups = in[1] / wt[1];
     if (groups <= 0 || wt[0] % groups != 0)
         return PET_HIP_ERR_INVALID;
-    return pet_hip_conv3d_f32(inputs[0]->devicePtr(), inputs[1]->devicePtr(),
-                              bias ? bias->devicePtr() : nullptr, outputs[0]->devicePtr(), in[0],
-                              in[1], in[2], in[3], in[4], wt[0], wt[2], wt[3], wt[4], pad[0],
-                              pad[1], pad[2], stride[0], stride[1], stride[2], dilation[0],
-                              dilation[1], dilation[2], groups, (int)act, stream);
+    const float *w = inputs[1]->devicePtr();
+    auto entry = pet_hip_conv3d_f32;
+    if (usesPackedFilters()) {
+        w = packed;
+        entry = pet_hip_conv3d_packed_f32;
+    }
+    return entry(inputs[0]->devicePtr(), w, bias ? bias->devicePtr() : nullptr,
+                 outputs[0]->devicePtr(), in[0], in[1], in[2], in[3], in[4], wt[0], wt[2], wt[3],
+                 wt[4], pad[0], pad[1], pad[2], stride[0], stride[1], stride[2], dilation[0],
+                 dilation[1], dilation[2], groups, (int)act, stream);
 }
 
 double Conv3dOp::perf(PerfEngine *, int rounds, int warmupRounds) {

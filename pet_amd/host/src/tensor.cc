@@ -149,6 +149,7 @@ bool Tensor::dataRand(int seed) {
     hostFresh = true;
     devFresh = false;
     computed = ComputedFull;
+    ++version;
     invalidateDependents();
     return true;
 }
@@ -160,6 +161,7 @@ bool Tensor::setData(const VType *hostPtr) {
     hostFresh = true;
     devFresh = false;
     computed = ComputedFull;
+    ++version;
     invalidateDependents();
     return true;
 }
@@ -176,6 +178,7 @@ VType *Tensor::getDataPtr() {
     }
     // the caller may write through the pointer: the device copy is stale from now on
     devFresh = false;
+    ++version;
     return host.data();
 }
 
@@ -191,6 +194,7 @@ float *Tensor::devicePtr() {
 }
 
 void Tensor::aliasDevice(float *ptr) {
+    ++version;
     if (dev && ownsDev)
         pet_hip_free(dev);
     dev = ptr;
@@ -203,6 +207,7 @@ void Tensor::aliasDevice(float *ptr) {
 void Tensor::deviceWritten() {
     devFresh = true;
     hostFresh = false;
+    ++version;
 }
 
 size_t Tensor::getOffset(const Dim &pos) const {
@@ -250,8 +255,10 @@ VType Tensor::getData(size_t pos) {
     if (pos >= size())
         return 0;
     bool keepDev = devFresh;
+    uint64_t keepVersion = version;
     VType v = getDataPtr()[pos];
     devFresh = keepDev; // a read does not invalidate the device copy
+    version = keepVersion;
     return v;
 }
 

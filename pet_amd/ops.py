@@ -48,10 +48,39 @@ def conv2d(x, w, ph, pw, sh=1, sw=1, dh=1, dw=1, bias=None, act="none", out=None
     return out
 
 
+class PackedFilters:
+    """Constant 3-D filters in the kt-major layout of pet_hip_conv3d_pack_filters."""
+
+    def __init__(self, data, shape):
+        self.data, self.shape = data, tuple(shape)
+
+
+def conv3d_pack_filters(w):
+    """kt-major copy of constant filters [f, c/g, kt, r, s], or None when the shape
+    has no such form (the caller keeps using the filters as they are). One-time
+    weight preprocessing, outside any timed or captured region."""
+    _chk(w)
+    f, cpg, kt, r, s = w.shape
+    packed = torch.empty_like(w)
+    rc = abi.status("pet_hip_conv3d_pack_filters", _ptr(w), _ptr(packed), f, cpg, kt, r, s,
+                    _stream())
+    if rc == 2:     # PET_HIP_ERR_UNSUPPORTED
+        return None
+    if rc != 0:
+        raise abi.PetHipError(rc, abi.last_error())
+    return PackedFilters(packed, w.shape)
+
+
 def conv3d(x, w, pad, stride=(1, 1, 1), dil=(1, 1, 1), bias=None, act="none", out=None):
+    """w: filters [f, c/g, kt, r, s], or a PackedFilters made from them."""
+    entry = "pet_hip_conv3d_f32"
+    if isinstance(w, PackedFilters):
+        entry, wshape, w = "pet_hip_conv3d_packed_f32", w.shape, w.data
+    else:
+        wshape = w.shape
     _chk(x, w, bias, out)
     n, c, t, h, wd = x.shape
-    f, cpg, kt, r, s = w.shape
+    f, cpg, kt, r, s = wshape
     if cpg <= 0 or c % cpg:
         raise abi.PetHipError(1, "input channels not divisible by weight channels")
     groups = c // cpg
@@ -60,7 +89,7 @@ def conv3d(x, w, pad, stride=(1, 1, 1), dil=(1, 1, 1), bias=None, act="none", ou
     ow = conv_out_dim(wd, s, pad[2], stride[2], dil[2])
     if out is None:
         out = torch.empty((n, f, ot, oh, ow), device=x.device, dtype=torch.float32)
-    abi.call("pet_hip_conv3d_f32", _ptr(x), _ptr(w), _ptr(bias), _ptr(out), n, c, t, h, wd, f, kt,
+    abi.call(entry, _ptr(x), _ptr(w), _ptr(bias), _ptr(out), n, c, t, h, wd, f, kt,
              r, s, *pad, *stride, *dil, groups, abi.ACT[act], _stream())
     return out
 

@@ -42,6 +42,12 @@ class GpuNS:
     def conv3d(self, x, w, pad, stride=(1, 1, 1), dil=(1, 1, 1), bias=None, act="none"):
         return self._k(self.ops.conv3d(x, w, pad, stride, dil, bias=bias, act=act))
 
+    def filters3d(self, w):
+        """Constant 3-D filters in the form conv3d reads fastest (kt-major where
+        the backend has one, else unchanged). A weight-only operator: run once."""
+        packed = self.ops.conv3d_pack_filters(w)
+        return w if packed is None else packed
+
     def matmul(self, A, B, transA=False, transB=False, bias=None, act="none"):
         return self._k(self.ops.matmul(A, B, transA, transB, bias=bias, act=act))
 
@@ -337,6 +343,13 @@ def run_c5(ns, p, transformed=False, T=None):
     T, get = _table(ns, p, T)
     for k in p:
         get(k)
+    # weight-only preprocessing, once per table (a namespace without it keeps the
+    # filters as they are)
+    prep = getattr(ns, "filters3d", None)
+    for k in p:
+        if prep is not None and k.endswith(".w") and p[k].ndim == 5 and (k + "#") not in T:
+            T[k + "#"] = True
+            T[k] = prep(T[k])
     x = ns.conv3d(T["x"], T["stem.w"], (1, 3, 3), (1, 2, 2), bias=T["stem.b"], act="relu")
     for li in range(4):
         for bi in range(2):

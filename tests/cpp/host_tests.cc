@@ -268,6 +268,51 @@ static bool test_code_engine_graph_runtime() {
     return true;
 }
 
+// Conv3dOp in the graph runtime: CodeEngine gives constant filters their kt-major
+// copy before capture, the replayed graph equals the eager operator (which reads
+// the filters as they are), and rewriting the weight tensor retires the copy.
+static bool test_conv3d_prepacked_graph() {
+    Graph g;
+    auto x = g.tensor({1, 16, 6, 12, 12}), wt = g.tensor({32, 16, 3, 3, 3});
+    auto c3 = static_cast<Conv3dOp *>(g.conv3d(x, wt, g.tensor({}), {1, 1, 1}, {1, 1, 1}, {1, 1, 1}));
+    c3->setAct(Operator::Relu);
+    g.relu(c3->getOutputs()[0]);
+    g.updateConnection();
+    auto s1 = std::make_shared<SubGraph>(g.getOperators());
+    auto s2 = std::make_shared<SubGraph>(g.getOperators());
+    for (size_t i = 0; i < s1->getInputs().size(); ++i) {
+        s1->getInputs()[i]->dataRand((int)i + 11);
+        s2->getInputs()[i]->setData(s1->getInputs()[i]->getDataPtr());
+    }
+    Conv3dOp *eager = nullptr, *replayed = nullptr;
+    for (auto op : s1->getOperators())
+        if (op->getType() == Operator::Conv3d)
+            eager = static_cast<Conv3dOp *>(op);
+    for (auto op : s2->getOperators())
+        if (op->getType() == Operator::Conv3d)
+            replayed = static_cast<Conv3dOp *>(op);
+    EXPECT(eager && replayed);
+    EXPECT(s1->compute());
+    EXPECT(!eager->usesPackedFilters());
+    CodeEngine ce;
+    auto exec = ce.instantiate(s2);
+    EXPECT(exec != nullptr);
+    EXPECT(replayed->usesPackedFilters());
+    for (int rep = 0; rep < 2; ++rep) {
+        EXPECT(exec->launch() && exec->sync());
+        Tensor *o1 = s1->getOutputs()[0], *o2 = s2->getOutputs()[0];
+        o2->deviceWritten();
+        EXPECT(equalArrays(o1->getDataPtr(), o2->getDataPtr(), o1->size()));
+    }
+    std::string code = ce.genCode(s2);
+    EXPECT(code.find("pet_hip_conv3d_pack_filters(") != std::string::npos);
+    EXPECT(code.find("pet_hip_conv3d_packed_f32") != std::string::npos);
+    // new weights: the copy no longer describes them
+    replayed->getInputs()[1]->dataRand(99);
+    EXPECT(!replayed->usesPackedFilters());
+    return true;
+}
+
 // Writes the emitted program of the config-1 transformed graph to argv[2]; the
 // python test compiles and runs it.
 static std::string g_emit_path;
@@ -443,6 +488,7 @@ int main(int argc, char **argv) {
         {"corrected_h2n_program", test_corrected_h2n_program},
         {"dilated_space_to_batch_program", test_dilated_space_to_batch_program},
         {"code_engine_graph_runtime", test_code_engine_graph_runtime},
+        {"conv3d_prepacked_graph", test_conv3d_prepacked_graph},
         {"emit_program", test_emit_program},
         {"perf_engine_memo", test_perf_engine_memo},
         {"split_ratio_and_eltwise", test_split_ratio_and_eltwise},

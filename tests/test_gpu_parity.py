@@ -236,6 +236,48 @@ def test_conv3d_integer_tier_bit_exact(ops, case):
     np.testing.assert_array_equal(got, ref)
 
 
+PACKED_CONV3D_CASES = [
+    # n, c, t, h, w, f, cpg, kt, r, s, pad, stride, dil
+    (1, 64, 4, 14, 14, 64, 64, 3, 3, 3, (1, 1, 1), (1, 1, 1), (1, 1, 1)),     # 64x64 tiles, split K
+    (1, 16, 6, 20, 20, 24, 8, 3, 3, 3, (1, 1, 1), (2, 1, 2), (1, 1, 1)),      # 2 groups, 32x64 tiles
+    (2, 8, 7, 9, 11, 70, 8, 5, 3, 3, (2, 1, 1), (1, 1, 1), (1, 1, 1)),        # kt 5, ragged M and pixels
+    (1, 32, 5, 12, 12, 16, 32, 3, 1, 1, (2, 0, 0), (1, 1, 1), (2, 1, 1)),     # 1x1 taps, dilated in t
+    (1, 64, 8, 28, 28, 64, 64, 3, 3, 3, (1, 1, 1), (1, 1, 1), (1, 1, 1)),     # stream-K sized grid
+]
+
+
+@pytest.mark.parametrize("case", PACKED_CONV3D_CASES)
+def test_conv3d_packed_filters_bit_exact(ops, case):
+    """kt-major filters (pet_hip_conv3d_pack_filters + pet_hip_conv3d_packed_f32)
+    against the oracle and against the plain entry point."""
+    n, c, t, h, w, f, cpg, kt, r, s, pad, st, dl = case
+    rng = np.random.default_rng(15)
+    x, wt = ints(rng, (n, c, t, h, w), -2, 3), ints(rng, (f, cpg, kt, r, s), -2, 3)
+    b = ints(rng, (f,), -3, 4)
+    ref = oracle.bias_act(oracle.conv3d(x, wt, pad, st, dl), b, "relu")
+    packed = ops.conv3d_pack_filters(dev(wt))
+    assert packed is not None
+    np.testing.assert_array_equal(host(packed.data).reshape(kt, f, cpg, r, s),
+                                  wt.transpose(2, 0, 1, 3, 4))
+    got = host(ops.conv3d(dev(x), packed, pad, st, dl, bias=dev(b), act="relu"))
+    plain = host(ops.conv3d(dev(x), dev(wt), pad, st, dl, bias=dev(b), act="relu"))
+    assert got.shape == ref.shape
+    np.testing.assert_array_equal(got, ref)
+    np.testing.assert_array_equal(plain, ref)
+
+
+def test_conv3d_pack_filters_declines_other_shapes(ops):
+    from pet_amd import abi
+    for shape in [(8, 8, 1, 3, 3), (8, 3, 3, 7, 7), (8, 4, 3, 3, 3), (8, 8, 3, 1, 3)]:
+        assert ops.conv3d_pack_filters(torch.zeros(shape, device="cuda")) is None
+    # and the packed entry point refuses them instead of misreading the buffer
+    x = torch.zeros((1, 4, 4, 6, 6), device="cuda")
+    w = torch.zeros((8, 4, 3, 3, 3), device="cuda")
+    with pytest.raises(abi.PetHipError) as e:
+        ops.conv3d(x, ops.PackedFilters(w, w.shape), (1, 1, 1))
+    assert e.value.status == 2
+
+
 def test_conv3d_kt1_equals_conv2d(ops):
     rng = np.random.default_rng(6)
     x, wt = ints(rng, (1, 8, 1, 12, 12)), ints(rng, (8, 8, 1, 3, 3))
