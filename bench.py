@@ -288,6 +288,23 @@ def main():
                 entry["pet_TFLOP/s"] = gflop / entry["pet_ms"]
             other[name] = entry
 
+    # ---- the same networks through the C++ host layer (tpm::Graph -> SubGraph ->
+    # CodeEngine::instantiate -> HIP graph replay), the path a PET user takes
+    host_path = {}
+    run_model = os.path.join(ROOT, "pet_amd", "lib", "pet_run_model")
+    if not args.no_configs and os.path.exists(run_model):
+        import subprocess
+        torch.cuda.synchronize()
+        for model in ("dilated:pet", "dilated", "resnet18", "bert", "resnet3d18"):
+            try:
+                res = subprocess.run([run_model, model, "--rounds", str(max(50, args.steps)),
+                                      "--warmup", "10"], capture_output=True, text=True,
+                                     timeout=300)
+                host_path[model] = (json.loads(res.stdout.strip().splitlines()[-1])
+                                    if res.returncode == 0 else {"error": res.stderr[-200:]})
+            except Exception as exc:
+                host_path[model] = {"error": str(exc)[:200]}
+
     dom_flop = conv_flop(DIL * DIL, 512, hs, hs, 512, 3, 3)
     dom_ms = conv_ms[0]
     achieved = dom_flop / dom_ms / 1e9
@@ -347,6 +364,7 @@ def main():
         "cpu_baseline": cpu,
         "per_op": per_op,
         "configs": other,
+        "host_layer_graphs": host_path,
     }
     print(json.dumps(out))
 

@@ -275,6 +275,83 @@ bool compile_chain(const ChainProgram &cp, ViewDesc &v) {
     return true;
 }
 
+// A chain without correction parameters only regroups and reorders extents: each
+// dim is a run of factors (extent, input stride), a split cuts a run, a reorder
+// moves runs, a fuse joins two. The output is then a plain strided view whose
+// dims are the factors in their final order, however many times a dim was fused.
+bool compile_pure_chain(const ChainProgram &cp, ViewDesc &v) {
+    struct Factor {
+        long long ext, stride;
+    };
+    std::vector<std::vector<Factor>> dims(cp.in_rank);
+    long long istr[PET_HIP_MAX_RANK];
+    row_major_strides(cp.dims[0], cp.in_rank, istr);
+    for (int i = 0; i < cp.in_rank; ++i) {
+        if (cp.dims[0][i] <= 0)
+            return false;
+        dims[i].push_back({cp.dims[0][i], istr[i]});
+    }
+    for (int o = 0; o < cp.nops; ++o) {
+        const ChainOp &op = cp.op[o];
+        if (op.kind == 0) {
+            if (op.c != 0 || op.d != 0 || cp.dims[o][op.a] % op.b != 0)
+                return false;
+            std::vector<Factor> &outer = dims[op.a], inner;
+            long long need = op.b;
+            while (need > 1) {
+                if (outer.empty())
+                    return false;
+                Factor last = outer.back();
+                if (last.ext <= need) {
+                    if (need % last.ext != 0)
+                        return false;
+                    inner.insert(inner.begin(), last);
+                    need /= last.ext;
+                    outer.pop_back();
+                } else {
+                    if (last.ext % need != 0)
+                        return false;
+                    inner.insert(inner.begin(), {need, last.stride});
+                    outer.back() = {last.ext / need, last.stride * need};
+                    need = 1;
+                }
+            }
+            dims.insert(dims.begin() + op.a + 1, inner);
+        } else if (op.kind == 1) {
+            std::vector<std::vector<Factor>> moved(dims.size());
+            for (size_t i = 0; i < dims.size(); ++i)
+                moved[i] = dims[op.perm[i]];
+            dims.swap(moved);
+        } else {
+            if (op.b != 0 || op.c != 0)
+                return false;
+            std::vector<Factor> &head = dims[op.a], &tail = dims[op.a + 1];
+            head.insert(head.end(), tail.begin(), tail.end());
+            dims.erase(dims.begin() + op.a + 1);
+        }
+    }
+    std::vector<Factor> flat;
+    for (auto &run : dims)
+        for (auto &f : run)
+            if (f.ext != 1)
+                flat.push_back(f);
+    if (flat.empty())
+        flat.push_back({1, 1});
+    if (flat.size() > (size_t)PET_HIP_MAX_RANK)
+        return false;
+    v.rank = (int)flat.size();
+    v.ibase = 0;
+    v.obase = 0;
+    long long os = 1;
+    for (int j = v.rank - 1; j >= 0; --j) {
+        if (flat[j].ext > 0x7fffffffll)
+            return false;
+        v.d[j] = plain_dim((int)flat[j].ext, os, flat[j].stride);
+        os *= flat[j].ext;
+    }
+    return true;
+}
+
 // Fallback: undo the chain per output element on the device.
 __global__ __launch_bounds__(256) void chain_interp_kernel(const float *__restrict__ x,
                                                            float *__restrict__ y,
@@ -394,7 +471,7 @@ int pet_hip_trans_chain(const float *x, float *y, const int *in_dims, int rank, 
     if (out_total == 0)
         return PET_HIP_OK;
     ViewDesc v;
-    if (compile_chain(cp, v))
+    if (compile_pure_chain(cp, v) || compile_chain(cp, v))
         return launch_view_copy(x, y, v, in_total, out_total, as_stream(stream));
     if (!x)
         return set_error(PET_HIP_ERR_INVALID, "null tensor pointer");

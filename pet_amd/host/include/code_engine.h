@@ -25,11 +25,13 @@ class GraphExec {
     double time(int warmup = 100, int rounds = 1000);
     size_t numKernelOps() const { return nLaunchOps; }
     size_t numAliasedOps() const { return nAliasOps; }
+    // Transposes that run as part of the transpose that follows them.
+    size_t numFoldedOps() const { return nFoldedOps; }
 
   private:
     friend class CodeEngine;
     pet_hip_graph_t graph = nullptr;
-    size_t nLaunchOps = 0, nAliasOps = 0;
+    size_t nLaunchOps = 0, nAliasOps = 0, nFoldedOps = 0;
 };
 
 class CodeEngine {

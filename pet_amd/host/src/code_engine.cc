@@ -61,6 +61,69 @@ bool weightOnly(const Operator *op) {
 
 size_t elems(const Tensor *t) { return t->size(); }
 
+// Transposes in a row become one kernel, as the reference's emitter collects a
+// transpose whose only successor is a transpose into that successor
+// (src/Graph/code_engine.cc:1428-1459): `folded` holds the operators that no
+// longer run by themselves, `chains` maps the last transpose of a row to the
+// whole row, first to last.
+struct TransposeChains {
+    std::set<const Operator *> folded;
+    std::map<const Operator *, std::vector<TransposeOp *>> chains;
+};
+
+TransposeChains planTransposeChains(const OpVec &order, const TensorVec &graphOutputs,
+                                    const std::set<const Operator *> &skipped) {
+    TransposeChains plan;
+    std::set<const Tensor *> outs(graphOutputs.begin(), graphOutputs.end());
+    std::map<const Operator *, std::vector<TransposeOp *>> open; // keyed by current last op
+    for (auto op : order) {
+        auto tr = dynamic_cast<TransposeOp *>(op);
+        if (!tr || skipped.count(op))
+            continue;
+        std::vector<TransposeOp *> row;
+        Operator *prev = op->getInputs()[0]->getOutputOf();
+        auto it = prev ? open.find(prev) : open.end();
+        if (it != open.end()) {
+            row = it->second;
+            open.erase(it);
+        }
+        row.push_back(tr);
+        Tensor *out = op->getOutputs()[0];
+        const OpVec &users = out->getInputOf();
+        bool continues = users.size() == 1 && dynamic_cast<TransposeOp *>(users[0]) != nullptr &&
+                         !skipped.count(users[0]) && !outs.count(out) &&
+                         weightOnly(op) == weightOnly(users[0]);
+        if (continues) {
+            open[op] = row;
+        } else if (row.size() > 1) {
+            for (size_t i = 0; i + 1 < row.size(); ++i)
+                plan.folded.insert(row[i]);
+            plan.chains[op] = row;
+        }
+    }
+    return plan;
+}
+
+// Micro-ops of a row of transposes, lowered on the first one's input.
+bool lowerChain(const std::vector<TransposeOp *> &row, TransProgram &prog) {
+    std::vector<std::shared_ptr<TransBasic>> all;
+    for (auto tr : row)
+        for (auto &m : tr->getTTParam())
+            all.push_back(m);
+    return TransposeEngine::getInstance().lower(all, row.front()->getInputs()[0]->getDims(), prog);
+}
+
+int launchChain(const std::vector<TransposeOp *> &row, pet_hip_stream_t s) {
+    TransProgram prog;
+    if (!lowerChain(row, prog))
+        return PET_HIP_ERR_INVALID;
+    int outDims[PET_HIP_MAX_RANK], outRank = 0;
+    return pet_hip_trans_chain(row.front()->getInputs()[0]->devicePtr(),
+                               row.back()->getOutputs()[0]->devicePtr(), prog.inDims.data(),
+                               (int)prog.inDims.size(), prog.ops.data(), prog.nops,
+                               prog.perms.data(), outDims, &outRank, s);
+}
+
 } // namespace
 
 // Storage sharing, decided before anything is captured:
@@ -148,6 +211,11 @@ std::unique_ptr<GraphExec> CodeEngine::instantiate(std::shared_ptr<SubGraph> &gr
                     t->devicePtr();
     }
     AliasPlan plan = planAliases(order);
+    TransposeChains rows = planTransposeChains(order, graph->getOutputs(), plan.skipped);
+    auto launchOp = [&](Operator *op, pet_hip_stream_t st) {
+        auto it = rows.chains.find(op);
+        return it == rows.chains.end() ? op->launch(st) : launchChain(it->second, st);
+    };
 
     std::unique_ptr<GraphExec> exec(new GraphExec());
     pet_hip_stream_t s = petStream();
@@ -155,8 +223,8 @@ std::unique_ptr<GraphExec> CodeEngine::instantiate(std::shared_ptr<SubGraph> &gr
     // (the reference's "Preprocess operators for weights" block,
     // src/Graph/code_engine.cc:183-190)
     for (auto op : order)
-        if (weightOnly(op) && !plan.skipped.count(op)) {
-            if (op->launch(s) != PET_HIP_OK)
+        if (weightOnly(op) && !plan.skipped.count(op) && !rows.folded.count(op)) {
+            if (launchOp(op, s) != PET_HIP_OK)
                 return nullptr;
             for (auto t : op->getOutputs())
                 t->deviceWritten();
@@ -178,7 +246,11 @@ std::unique_ptr<GraphExec> CodeEngine::instantiate(std::shared_ptr<SubGraph> &gr
         }
         if (weightOnly(op))
             continue;
-        if (op->launch(s) != PET_HIP_OK) {
+        if (rows.folded.count(op)) {
+            exec->nFoldedOps++;
+            continue;
+        }
+        if (launchOp(op, s) != PET_HIP_OK) {
             std::fprintf(stderr, "[pet] capture of %s failed: %s\n", op->toString().c_str(),
                          pet_hip_last_error());
             ok = false;
@@ -194,7 +266,7 @@ std::unique_ptr<GraphExec> CodeEngine::instantiate(std::shared_ptr<SubGraph> &gr
     }
     exec->graph = g;
     for (auto t : graph->getTensors())
-        if (t->getOutputOf() != nullptr) {
+        if (t->getOutputOf() != nullptr && !rows.folded.count(t->getOutputOf())) {
             t->deviceWritten();
             t->setComputed();
         }
@@ -305,10 +377,13 @@ std::string CodeEngine::genCode(std::shared_ptr<SubGraph> &graph) {
         }
         skipped.insert(op);
     }
+    TransposeChains rows = planTransposeChains(order, graph->getOutputs(), skipped);
     uint64_t seed = 1;
     for (auto t : all) {
         if (viewOf.count(t))
             continue;
+        if (t->getOutputOf() != nullptr && rows.folded.count(t->getOutputOf()))
+            continue; // inside a row of transposes: never materialised
         std::string n = e.name(t);
         e.line("    float *" + n + "; CHECK(pet_hip_malloc((void **)&" + n + ", " +
                std::to_string(std::max<size_t>(t->size(), 1)) + " * sizeof(float)));");
@@ -365,14 +440,17 @@ std::string CodeEngine::genCode(std::shared_ptr<SubGraph> &graph) {
               << nullable(e, mm->getBias()) << ", " << (int)mm->getAct() << ", s)";
         } else if (auto tr = dynamic_cast<TransposeOp *>(op)) {
             TransProgram prog;
-            if (!TransposeEngine::getInstance().lower(tr->getTTParam(),
-                                                      op->getInputs()[0]->getDims(), prog))
+            std::vector<TransposeOp *> row = {tr};
+            if (rows.chains.count(op))
+                row = rows.chains.at(op);
+            if (!lowerChain(row, prog))
                 return false;
             std::string id = std::to_string(op->getGuid());
+            std::string src = e.name(row.front()->getInputs()[0]);
             e.line("    static const int tin" + id + "[] = " + e.ints(prog.inDims) + ", tops" + id +
                    "[] = " + e.ints(prog.ops) + ", tperm" + id + "[] = " + e.ints(prog.perms) + ";");
             e.line("    // " + TransposeEngine::getInstance().describe(prog));
-            c << "pet_hip_trans_chain(" << in(0) << ", " << out(0) << ", tin" << id << ", "
+            c << "pet_hip_trans_chain(" << src << ", " << out(0) << ", tin" << id << ", "
               << prog.inDims.size() << ", tops" << id << ", " << prog.nops << ", tperm" << id
               << ", odims, &orank, s)";
         } else if (auto sp = dynamic_cast<SplitOp *>(op)) {
@@ -465,7 +543,7 @@ std::string CodeEngine::genCode(std::shared_ptr<SubGraph> &graph) {
     e.line("    int odims[PET_HIP_MAX_RANK], orank = 0; (void)odims; (void)orank;");
     e.line("    // operators that only touch weights run once");
     for (auto op : order)
-        if (weightOnly(op) && !skipped.count(op) && !emitOp(op))
+        if (weightOnly(op) && !skipped.count(op) && !rows.folded.count(op) && !emitOp(op))
             return "";
     e.line("    // constant 3-D filters: kt-major copy where the backend has that form");
     for (auto op : order) {
@@ -487,7 +565,7 @@ std::string CodeEngine::genCode(std::shared_ptr<SubGraph> &graph) {
     e.line("    // the rest is captured once and replayed as a HIP graph");
     e.line("    CHECK(pet_hip_graph_begin_capture(s));");
     for (auto op : order)
-        if (!weightOnly(op) && !skipped.count(op) && !emitOp(op))
+        if (!weightOnly(op) && !skipped.count(op) && !rows.folded.count(op) && !emitOp(op))
             return "";
     e.line("    pet_hip_graph_t g; CHECK(pet_hip_graph_end_capture(s, &g));");
     e.line("    pet_hip_event_t st, ed; CHECK(pet_hip_event_create(&st)); "

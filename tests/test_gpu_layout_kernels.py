@@ -152,6 +152,28 @@ def test_halo_chain_on_width(ops):
     assert got.shape == ref.shape and got.tobytes() == ref.tobytes()
 
 
+@pytest.mark.parametrize("n,c,h,w,d", [(1, 8, 16, 16, 2), (2, 3, 12, 18, 3), (1, 64, 64, 64, 2),
+                                        (3, 5, 8, 20, 4)])
+def test_chained_transposes_fold_into_one_view(ops, n, c, h, w, d):
+    """Space-to-batch written as two transposes in a row (rows, then columns, each
+    de-interleaved into the batch) and its inverse, each sent as one micro-op
+    chain: the output dim 0 is fused twice, which only the factor-wise chain
+    compiler turns into a strided view. Expected values from numpy."""
+    x = iota((n, c, h, w))
+    fwd = [("split", 2, d, 0, 0), ("reorder", [3, 0, 1, 2, 4]), ("fuse", 0, 0, 0),
+           ("split", 3, d, 0, 0), ("reorder", [4, 0, 1, 2, 3]), ("fuse", 0, 0, 0)]
+    ref = (x.reshape(n, c, h // d, d, w // d, d).transpose(5, 3, 0, 1, 2, 4)
+           .reshape(d * d * n, c, h // d, w // d))
+    assert oracle.trans_chain(x, fwd).tobytes() == ref.tobytes()
+    got = ops.trans_chain(dev(x), fwd)
+    assert host(got).shape == ref.shape and host(got).tobytes() == ref.tobytes()
+    # back: the column phase leaves the batch first, then the row phase
+    inv = [("split", 0, d * n, 0, 0), ("reorder", [1, 2, 3, 4, 0]), ("fuse", 3, 0, 0),
+           ("split", 0, n, 0, 0), ("reorder", [1, 2, 3, 0, 4]), ("fuse", 2, 0, 0)]
+    back = ops.trans_chain(got, inv)
+    assert host(back).shape == x.shape and host(back).tobytes() == x.tobytes()
+
+
 def test_random_permutes_pads_slices_against_numpy(ops):
     """300 seeded random cases across the kernel-selection boundaries: ranks 2-6,
     extents mixing multiples of 4, of 2 and odd numbers, any permutation; then a

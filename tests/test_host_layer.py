@@ -299,3 +299,27 @@ def test_generator_candidates_run_and_are_ranked_on_the_device(args):
     print(res.stdout[-6000:])
     print(res.stderr[-2000:])
     assert res.returncode == 0
+
+
+# ---- the benchmark networks through Graph -> SubGraph -> CodeEngine ---------------
+RUN_MODEL = os.path.join(LIB, "pet_run_model")
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("model", ["dilated", "dilated:pet", "resnet18", "bert", "resnet3d18"])
+def test_model_graph_replay_equals_operator_by_operator_run(model):
+    """pet_run_model --check: the captured HIP graph (storage sharing, transposes in a
+    row folded into one kernel, constant 3-D filters repacked) against
+    SubGraph::compute, which launches every operator by itself."""
+    import json
+    assert os.path.exists(RUN_MODEL), "run __graft_entry__.build() first"
+    res = subprocess.run([RUN_MODEL, model, "--check", "--rounds", "20", "--warmup", "3"],
+                         capture_output=True, text=True, timeout=300)
+    print(res.stdout)
+    print(res.stderr[-2000:])
+    assert res.returncode == 0
+    rec = json.loads(res.stdout.strip().splitlines()[-1])
+    assert rec["max_abs_diff_vs_eager"] <= 1e-4 * rec["max_abs_eager"]
+    assert rec["ms"] > 0
+    if model == "dilated:pet":
+        assert rec["folded"] == 2 and rec["kernels"] == 8
