@@ -136,6 +136,28 @@ PET_HIP_API int pet_hip_conv3d_f32(const float *x, const float *w, const float *
                        int pt, int ph, int pw, int st, int sh, int sw, int dt, int dh,
                        int dw, int groups, int act, pet_hip_stream_t stream);
 
+/* The three contractions with a residual operand: y = act(op(x, w) + bias +
+ * residual), residual laid out like y and not overlapping it. This is the z
+ * operand of cudnnConvolutionBiasActivationForward, which the reference passes
+ * with weight 0 (src/Graph/operator.cc:477-480, src/Graph/code_engine.cc:955-977);
+ * a graph runtime uses it to run "convolution, then Add with another tensor,
+ * then ReLU" (a ResNet block's tail) or "matmul, then Add" (a transformer
+ * block's residual) as one operator. All other arguments as in the entry points
+ * without _res; for the 3-D form w_is_packed says that w came from
+ * pet_hip_conv3d_pack_filters. */
+PET_HIP_API int pet_hip_conv2d_res_f32(const float *x, const float *w, const float *bias,
+                           const float *residual, float *y, int n, int c, int h, int wd, int f,
+                           int r, int s, int ph, int pw, int sh, int sw, int dh, int dw,
+                           int groups, int act, pet_hip_stream_t stream);
+PET_HIP_API int pet_hip_conv3d_res_f32(const float *x, const float *w, int w_is_packed,
+                           const float *bias, const float *residual, float *y, int n, int c,
+                           int t, int h, int wd, int f, int kt, int r, int s, int pt, int ph,
+                           int pw, int st, int sh, int sw, int dt, int dh, int dw, int groups,
+                           int act, pet_hip_stream_t stream);
+PET_HIP_API int pet_hip_bmm_res_f32(int transA, int transB, int b, int m, int n, int k, const float *A,
+                        const float *B, float *C, const float *bias, const float *residual,
+                        int act, pet_hip_stream_t stream);
+
 /* Constant 3-D filters, reordered once: [f][c/groups][kt][r][s] -> kt-major
  * [kt][f][c/groups][r][s] (same element count), so that each kt slice is a 2-D
  * filter bank the convolution kernel reads with 16-byte loads. This is a

@@ -46,6 +46,9 @@ SIGNATURES = {
     "pet_hip_conv_out_dim": [_i] * 5,
     "pet_hip_conv2d_f32": [_vp] * 4 + [_i] * 15 + [_vp],
     "pet_hip_conv3d_f32": [_vp] * 4 + [_i] * 20 + [_vp],
+    "pet_hip_conv2d_res_f32": [_vp] * 5 + [_i] * 15 + [_vp],
+    "pet_hip_conv3d_res_f32": [_vp, _vp, _i, _vp, _vp, _vp] + [_i] * 20 + [_vp],
+    "pet_hip_bmm_res_f32": [_i] * 6 + [_vp] * 5 + [_i, _vp],
     "pet_hip_conv3d_pack_filters": [_vp, _vp] + [_i] * 5 + [_vp],
     "pet_hip_conv3d_packed_f32": [_vp] * 4 + [_i] * 20 + [_vp],
     "pet_hip_bmm_f32": [_i] * 6 + [_vp] * 4 + [_i, _vp],

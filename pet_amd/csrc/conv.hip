@@ -20,6 +20,7 @@ namespace {
 
 struct ConvParams {
     const float *x, *w, *bias;
+    const float *res; // optional residual, laid out like y: y = act(conv + bias + res)
     float *y;
     int N, C, T, H, W, F;
     int KT, R, S;
@@ -255,7 +256,9 @@ __global__ __launch_bounds__(Cfg::NT) void conv_pipe_kernel(ConvParams p) {
             continue;
         unsigned n = fd_div(pix, p.fd_opix);
         unsigned rem = pix - n * p.OPIX;
-        float *__restrict__ yb = p.y + (((long long)n * p.F + (long long)g * p.M) * p.OPIX + rem);
+        const long long ybase = ((long long)n * p.F + (long long)g * p.M) * p.OPIX + rem;
+        float *__restrict__ yb = p.y + ybase;
+        const float *rb = p.res ? p.res + ybase : nullptr;
         const float *__restrict__ bias = p.bias ? p.bias + g * p.M : nullptr;
 #pragma unroll
         for (int tm = 0; tm < TM; ++tm) {
@@ -266,6 +269,8 @@ __global__ __launch_bounds__(Cfg::NT) void conv_pipe_kernel(ConvParams p) {
                     float v = acc[tm][tn][r];
                     if (bias)
                         v += bias[f];
+                    if (rb)
+                        v += rb[(unsigned)f * (unsigned)p.OPIX];
                     yb[(unsigned)f * (unsigned)p.OPIX] = apply_act(v, p.act);
                 }
             }
@@ -719,8 +724,9 @@ __global__ __launch_bounds__(Cfg::NT) void conv_plane_kernel(ConvParams p) {
         if (pix < p.NPIX) {
             const unsigned n = fd_div(pix, p.fd_opix);
             const unsigned rem = pix - n * p.OPIX;
-            float *__restrict__ yb =
-                p.y + (((long long)n * p.F + (long long)g * p.M) * p.OPIX + rem);
+            const long long ybase = ((long long)n * p.F + (long long)g * p.M) * p.OPIX + rem;
+            float *__restrict__ yb = p.y + ybase;
+            const float *rb = p.res ? p.res + ybase : nullptr;
             const float *__restrict__ bias =
                 (p.bias && p.bias_mode == 1) ? p.bias + g * p.M : nullptr;
             float cb[4] = {0.f, 0.f, 0.f, 0.f};
@@ -736,6 +742,14 @@ __global__ __launch_bounds__(Cfg::NT) void conv_plane_kernel(ConvParams p) {
                 if (f < p.M) {
                     float4 v = *reinterpret_cast<const float4 *>(lds + fl * C_LD + 4 * q);
                     const float bf = bias ? bias[f] : 0.f;
+                    if (rb) {
+                        const float4 rv =
+                            *reinterpret_cast<const float4 *>(rb + (unsigned)f * (unsigned)p.OPIX);
+                        v.x += rv.x;
+                        v.y += rv.y;
+                        v.z += rv.z;
+                        v.w += rv.w;
+                    }
                     v.x = apply_act(v.x + bf + cb[0], p.act);
                     v.y = apply_act(v.y + bf + cb[1], p.act);
                     v.z = apply_act(v.z + bf + cb[2], p.act);
@@ -755,7 +769,9 @@ __global__ __launch_bounds__(Cfg::NT) void conv_plane_kernel(ConvParams p) {
             continue;
         unsigned n = fd_div(pix, p.fd_opix);
         unsigned rem = pix - n * p.OPIX;
-        float *__restrict__ yb = p.y + (((long long)n * p.F + (long long)g * p.M) * p.OPIX + rem);
+        const long long ybase = ((long long)n * p.F + (long long)g * p.M) * p.OPIX + rem;
+        float *__restrict__ yb = p.y + ybase;
+        const float *rb = p.res ? p.res + ybase : nullptr;
         const float *__restrict__ bias =
             (p.bias && p.bias_mode == 1) ? p.bias + g * p.M : nullptr;
         const float colbias = (p.bias && p.bias_mode == 2) ? p.bias[rem] : 0.f;
@@ -780,6 +796,8 @@ __global__ __launch_bounds__(Cfg::NT) void conv_plane_kernel(ConvParams p) {
                         float v = acc[tm][tn][r];
                         if (bias)
                             v += bias[f];
+                        if (rb)
+                            v += rb[(unsigned)f * (unsigned)p.OPIX];
                         yb[(unsigned)f * (unsigned)p.OPIX] = apply_act(v + colbias, p.act);
                     }
                 }
@@ -836,11 +854,11 @@ int pick_tile(int M, int N, int batch) {
 }
 
 // Output initialisation for split-K launches: y = bias (per channel or per
-// column) or 0; the partial sums are then added atomically.
-__global__ __launch_bounds__(256) void splitk_init_kernel(float *__restrict__ y,
-                                                          const float *__restrict__ bias,
-                                                          int bias_mode, unsigned F, unsigned OPIX,
-                                                          size_t total) {
+// column) or 0, plus the residual if there is one (which may be y itself); the
+// partial sums are then added atomically.
+__global__ __launch_bounds__(256) void splitk_init_kernel(float *y, const float *__restrict__ bias,
+                                                          const float *res, int bias_mode,
+                                                          unsigned F, unsigned OPIX, size_t total) {
     size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
     const size_t step = (size_t)gridDim.x * 256;
     for (; i < total; i += step) {
@@ -850,6 +868,8 @@ __global__ __launch_bounds__(256) void splitk_init_kernel(float *__restrict__ y,
             unsigned f = (unsigned)((i / OPIX) % F);
             v = bias_mode == 2 ? bias[pix] : bias[f];
         }
+        if (res)
+            v += res[i];
         y[i] = v;
     }
 }
@@ -973,7 +993,7 @@ int launch_plane_cfg(ConvParams p, hipStream_t stream) {
         const size_t total = (size_t)p.NPIX * p.F;
         unsigned igrid = (unsigned)std::min<size_t>((total + 255) / 256, 4096);
         hipLaunchKernelGGL(splitk_init_kernel, dim3(igrid), dim3(256), 0, stream, p.y, p.bias,
-                           p.bias_mode, (unsigned)p.F, (unsigned)p.OPIX, total);
+                           p.res, p.bias_mode, (unsigned)p.F, (unsigned)p.OPIX, total);
         int rc = check_launch("splitk_init_kernel");
         if (rc)
             return rc;
@@ -981,7 +1001,7 @@ int launch_plane_cfg(ConvParams p, hipStream_t stream) {
     p.fd_splitk = make_fastdiv((unsigned)p.splitk);
     p.fd_mg = make_fastdiv((unsigned)p.xcd_mg);
     p.fd_band = make_fastdiv((unsigned)p.xcd_mg * grid.x);
-    p.vec_out = (p.OPIX % 4 == 0) && (((uintptr_t)p.y & 15) == 0);
+    p.vec_out = (p.OPIX % 4 == 0) && (((uintptr_t)p.y & 15) == 0) && (((uintptr_t)p.res & 15) == 0);
     if constexpr (has_streamk<Cfg>) {
         if (p.streamk) {
             grid = dim3(Cfg::BM * Cfg::BN >= 64 * 128 ? 256 : 512, 1, 1);
@@ -1097,7 +1117,7 @@ int launch_conv(ConvParams &p, hipStream_t stream) {
 int conv_common(const float *x, const float *w, const float *bias, float *y, int n, int c, int t,
                 int h, int wd, int f, int kt, int r, int s, int pt, int ph, int pw, int st, int sh,
                 int sw, int dt, int dh, int dw, int groups, int act, hipStream_t stream,
-                bool wpacked = false) {
+                bool wpacked = false, const float *res = nullptr) {
     if (n < 0 || c <= 0 || t <= 0 || h <= 0 || wd <= 0 || f <= 0 || kt <= 0 || r <= 0 || s <= 0 ||
         groups <= 0 || st <= 0 || sh <= 0 || sw <= 0 || dt <= 0 || dh <= 0 || dw <= 0 || pt < 0 ||
         ph < 0 || pw < 0)
@@ -1128,9 +1148,12 @@ int conv_common(const float *x, const float *w, const float *bias, float *y, int
         return set_error(PET_HIP_ERR_UNSUPPORTED, "convolution operands above 2^31 elements");
     if (!x || !w || !y)
         return set_error(PET_HIP_ERR_INVALID, "null tensor pointer");
+    if (res == y)
+        return set_error(PET_HIP_ERR_INVALID, "the residual must not be the output buffer");
     p.x = x;
     p.w = w;
     p.bias = bias;
+    p.res = res;
     p.y = y;
     p.N = n;
     p.C = c;
@@ -1182,8 +1205,8 @@ namespace mfma {
 // the batch is the group, B[b] ([k][n]) is that group's k-channel "image" of n
 // pixels, A[b] ([m][k]) its filters. Returns -1 when the plane kernel does not
 // apply (k not a multiple of 32, operands above 2 GiB, misaligned A).
-int bmm_as_grouped_1x1(const float *A, const float *B, float *C, const float *bias, int b, int m,
-                       int n, int k, int act, hipStream_t stream) {
+int bmm_as_grouped_1x1(const float *A, const float *B, float *C, const float *bias,
+                       const float *res, int b, int m, int n, int k, int act, hipStream_t stream) {
     if (k % 32 != 0 || b > 65535)
         return -1;
     ConvParams p;
@@ -1191,6 +1214,7 @@ int bmm_as_grouped_1x1(const float *A, const float *B, float *C, const float *bi
     p.x = B;
     p.w = A;
     p.bias = bias;
+    p.res = res;
     p.y = C;
     p.N = 1;
     p.C = b * k;
@@ -1240,6 +1264,25 @@ int pet_hip_conv3d_f32(const float *x, const float *w, const float *bias, float 
     PET_REQUIRE_INIT();
     return conv_common(x, w, bias, y, n, c, t, h, wd, f, kt, r, s, pt, ph, pw, st, sh, sw, dt, dh,
                        dw, groups, act, as_stream(stream));
+}
+
+int pet_hip_conv2d_res_f32(const float *x, const float *w, const float *bias,
+                           const float *residual, float *y, int n, int c, int h, int wd, int f,
+                           int r, int s, int ph, int pw, int sh, int sw, int dh, int dw, int groups,
+                           int act, pet_hip_stream_t stream) {
+    PET_REQUIRE_INIT();
+    return conv_common(x, w, bias, y, n, c, 1, h, wd, f, 1, r, s, 0, ph, pw, 1, sh, sw, 1, dh, dw,
+                       groups, act, as_stream(stream), false, residual);
+}
+
+int pet_hip_conv3d_res_f32(const float *x, const float *w, int w_is_packed, const float *bias,
+                           const float *residual, float *y, int n, int c, int t, int h, int wd,
+                           int f, int kt, int r, int s, int pt, int ph, int pw, int st, int sh,
+                           int sw, int dt, int dh, int dw, int groups, int act,
+                           pet_hip_stream_t stream) {
+    PET_REQUIRE_INIT();
+    return conv_common(x, w, bias, y, n, c, t, h, wd, f, kt, r, s, pt, ph, pw, st, sh, sw, dt, dh,
+                       dw, groups, act, as_stream(stream), w_is_packed != 0, residual);
 }
 
 int pet_hip_conv3d_pack_filters(const float *w, float *packed, int f, int cpg, int kt, int r,

@@ -150,12 +150,10 @@ int launch_bmm_t(const GemmParams &p, int batch, bool vec, hipStream_t stream) {
 
 } // namespace
 
-extern "C" {
+namespace {
 
-int pet_hip_bmm_f32(int transA, int transB, int b, int m, int n, int k, const float *A,
-                    const float *B, float *C, const float *bias, int act,
-                    pet_hip_stream_t stream) {
-    PET_REQUIRE_INIT();
+int bmm_common(int transA, int transB, int b, int m, int n, int k, const float *A, const float *B,
+               float *C, const float *bias, const float *res, int act, pet_hip_stream_t stream) {
     if (b < 0 || m < 0 || n < 0 || k < 0)
         return set_error(PET_HIP_ERR_INVALID, "negative matmul dims");
     if (act < PET_HIP_ACT_NONE || act > PET_HIP_ACT_GELU)
@@ -164,9 +162,13 @@ int pet_hip_bmm_f32(int transA, int transB, int b, int m, int n, int k, const fl
         return PET_HIP_OK;
     if (!C)
         return set_error(PET_HIP_ERR_INVALID, "null tensor pointer");
+    if (res == C)
+        return set_error(PET_HIP_ERR_INVALID, "the residual must not be the output buffer");
+    const size_t cn = (size_t)b * m * n;
     if (k == 0) {
-        // empty contraction: C = act(bias)
-        int rc = pet_hip_fill_f32(C, 0.f, (size_t)b * m * n, stream);
+        // empty contraction: C = act(bias + residual)
+        int rc = res ? pet_hip_memcpy_d2d(C, res, cn * sizeof(float), stream)
+                     : pet_hip_fill_f32(C, 0.f, cn, stream);
         if (rc == PET_HIP_OK && (bias || act != PET_HIP_ACT_NONE))
             rc = pet_hip_bias_act(C, bias, C, (size_t)b * m, (size_t)n, 1, act, stream);
         return rc;
@@ -187,12 +189,24 @@ int pet_hip_bmm_f32(int transA, int transB, int b, int m, int n, int k, const fl
     p.sA = (long long)m * k;
     p.sB = (long long)k * n;
     p.sC = (long long)m * n;
-    p.act = act;
+    p.act = res ? PET_HIP_ACT_NONE : act;
     if (!transA && !transB) {
-        int rc = bmm_as_grouped_1x1(A, B, C, bias, b, m, n, k, act, as_stream(stream));
+        int rc = bmm_as_grouped_1x1(A, B, C, bias, res, b, m, n, k, act, as_stream(stream));
         if (rc >= 0)
             return rc;
     }
+    // the general kernel has no residual operand: add it, and apply the activation,
+    // in two small launches afterwards
+    auto finish = [&](int rc) {
+        if (rc != PET_HIP_OK || !res)
+            return rc;
+        const float *ins[2] = {C, res};
+        const size_t sizes[2] = {cn, cn};
+        rc = pet_hip_eltwise(PET_HIP_ADD, ins, sizes, 2, C, cn, stream);
+        if (rc == PET_HIP_OK && act != PET_HIP_ACT_NONE)
+            rc = pet_hip_activation(C, C, cn, act, stream);
+        return rc;
+    };
     // float4 loads need every row start 16-byte aligned on both operands
     long long lda = transA ? m : k, ldb = transB ? k : n;
     bool vec = lda % 4 == 0 && ldb % 4 == 0 && p.sA % 4 == 0 && p.sB % 4 == 0 &&
@@ -200,10 +214,28 @@ int pet_hip_bmm_f32(int transA, int transB, int b, int m, int n, int k, const fl
                (transA ? m % 4 == 0 : k % 4 == 0) && (transB ? k % 4 == 0 : n % 4 == 0);
     hipStream_t s = as_stream(stream);
     if (transA)
-        return transB ? launch_bmm_t<true, true>(p, b, vec, s)
-                      : launch_bmm_t<true, false>(p, b, vec, s);
-    return transB ? launch_bmm_t<false, true>(p, b, vec, s)
-                  : launch_bmm_t<false, false>(p, b, vec, s);
+        return finish(transB ? launch_bmm_t<true, true>(p, b, vec, s)
+                             : launch_bmm_t<true, false>(p, b, vec, s));
+    return finish(transB ? launch_bmm_t<false, true>(p, b, vec, s)
+                         : launch_bmm_t<false, false>(p, b, vec, s));
+}
+
+} // namespace
+
+extern "C" {
+
+int pet_hip_bmm_f32(int transA, int transB, int b, int m, int n, int k, const float *A,
+                    const float *B, float *C, const float *bias, int act,
+                    pet_hip_stream_t stream) {
+    PET_REQUIRE_INIT();
+    return bmm_common(transA, transB, b, m, n, k, A, B, C, bias, nullptr, act, stream);
+}
+
+int pet_hip_bmm_res_f32(int transA, int transB, int b, int m, int n, int k, const float *A,
+                        const float *B, float *C, const float *bias, const float *residual,
+                        int act, pet_hip_stream_t stream) {
+    PET_REQUIRE_INIT();
+    return bmm_common(transA, transB, b, m, n, k, A, B, C, bias, residual, act, stream);
 }
 
 } // extern "C"

@@ -33,8 +33,10 @@ def conv_out_dim(i, k, p, s, d):
     return (i - (k - s) * d + 2 * p) // s if (i - (k - s) * d + 2 * p) >= 0 else -1
 
 
-def conv2d(x, w, ph, pw, sh=1, sw=1, dh=1, dw=1, bias=None, act="none", out=None):
-    _chk(x, w, bias, out)
+def conv2d(x, w, ph, pw, sh=1, sw=1, dh=1, dw=1, bias=None, act="none", out=None,
+           residual=None):
+    """act(conv(x, w) + bias + residual); residual has the output's shape."""
+    _chk(x, w, bias, out, residual)
     n, c, h, wd = x.shape
     f, cpg, r, s = w.shape
     if cpg <= 0 or c % cpg:
@@ -43,6 +45,12 @@ def conv2d(x, w, ph, pw, sh=1, sw=1, dh=1, dw=1, bias=None, act="none", out=None
     oh, ow = conv_out_dim(h, r, ph, sh, dh), conv_out_dim(wd, s, pw, sw, dw)
     if out is None:
         out = torch.empty((n, f, max(oh, 0), max(ow, 0)), device=x.device, dtype=torch.float32)
+    if residual is not None:
+        if tuple(residual.shape) != tuple(out.shape):
+            raise abi.PetHipError(1, "residual shape differs from the output's")
+        abi.call("pet_hip_conv2d_res_f32", _ptr(x), _ptr(w), _ptr(bias), _ptr(residual), _ptr(out),
+                 n, c, h, wd, f, r, s, ph, pw, sh, sw, dh, dw, groups, abi.ACT[act], _stream())
+        return out
     abi.call("pet_hip_conv2d_f32", _ptr(x), _ptr(w), _ptr(bias), _ptr(out), n, c, h, wd, f, r, s,
              ph, pw, sh, sw, dh, dw, groups, abi.ACT[act], _stream())
     return out
@@ -71,14 +79,15 @@ def conv3d_pack_filters(w):
     return PackedFilters(packed, w.shape)
 
 
-def conv3d(x, w, pad, stride=(1, 1, 1), dil=(1, 1, 1), bias=None, act="none", out=None):
+def conv3d(x, w, pad, stride=(1, 1, 1), dil=(1, 1, 1), bias=None, act="none", out=None,
+           residual=None):
     """w: filters [f, c/g, kt, r, s], or a PackedFilters made from them."""
     entry = "pet_hip_conv3d_f32"
     if isinstance(w, PackedFilters):
         entry, wshape, w = "pet_hip_conv3d_packed_f32", w.shape, w.data
     else:
         wshape = w.shape
-    _chk(x, w, bias, out)
+    _chk(x, w, bias, out, residual)
     n, c, t, h, wd = x.shape
     f, cpg, kt, r, s = wshape
     if cpg <= 0 or c % cpg:
@@ -89,14 +98,22 @@ def conv3d(x, w, pad, stride=(1, 1, 1), dil=(1, 1, 1), bias=None, act="none", ou
     ow = conv_out_dim(wd, s, pad[2], stride[2], dil[2])
     if out is None:
         out = torch.empty((n, f, ot, oh, ow), device=x.device, dtype=torch.float32)
+    if residual is not None:
+        if tuple(residual.shape) != tuple(out.shape):
+            raise abi.PetHipError(1, "residual shape differs from the output's")
+        abi.call("pet_hip_conv3d_res_f32", _ptr(x), _ptr(w),
+                 int(entry == "pet_hip_conv3d_packed_f32"), _ptr(bias), _ptr(residual), _ptr(out),
+                 n, c, t, h, wd, f, kt, r, s, *pad, *stride, *dil, groups, abi.ACT[act], _stream())
+        return out
     abi.call(entry, _ptr(x), _ptr(w), _ptr(bias), _ptr(out), n, c, t, h, wd, f, kt,
              r, s, *pad, *stride, *dil, groups, abi.ACT[act], _stream())
     return out
 
 
-def matmul(A, B, transA=False, transB=False, bias=None, act="none", out=None):
-    """MatmulOp on [b, ., .] tensors (MatmulOp::computeShape, operator.cc:717-726)."""
-    _chk(A, B, bias, out)
+def matmul(A, B, transA=False, transB=False, bias=None, act="none", out=None, residual=None):
+    """MatmulOp on [b, ., .] tensors (MatmulOp::computeShape, operator.cc:717-726);
+    with residual: act(A @ B + bias + residual)."""
+    _chk(A, B, bias, out, residual)
     b = A.shape[0]
     m = A.shape[2] if transA else A.shape[1]
     k = A.shape[1] if transA else A.shape[2]
@@ -106,6 +123,12 @@ def matmul(A, B, transA=False, transB=False, bias=None, act="none", out=None):
         raise abi.PetHipError(1, "matmul shapes do not agree")
     if out is None:
         out = torch.empty((b, m, n), device=A.device, dtype=torch.float32)
+    if residual is not None:
+        if residual.numel() != out.numel():
+            raise abi.PetHipError(1, "residual size differs from the output's")
+        abi.call("pet_hip_bmm_res_f32", int(transA), int(transB), b, m, n, k, _ptr(A), _ptr(B),
+                 _ptr(out), _ptr(bias), _ptr(residual), abi.ACT[act], _stream())
+        return out
     abi.call("pet_hip_bmm_f32", int(transA), int(transB), b, m, n, k, _ptr(A), _ptr(B), _ptr(out),
              _ptr(bias), abi.ACT[act], _stream())
     return out

@@ -327,6 +327,81 @@ def test_matmul_float_tier_and_bias_gelu(ops):
     assert max_rel_err(got2, ref2, mag + np.abs(bias)) <= REL_TOL
 
 
+RESIDUAL_CONV_CASES = [
+    # n, c, h, w, f, cpg, r, pad, stride    what the shape exercises
+    (1, 64, 14, 14, 64, 64, 3, 1, 1),       # few tiles: split K (init kernel carries the residual)
+    (2, 16, 32, 32, 64, 16, 3, 1, 1),       # no split, pixel count % 4 == 0: 16-byte epilogue
+    (1, 8, 9, 7, 24, 8, 3, 1, 1),           # odd pixel count: scalar epilogue
+    (1, 3, 20, 20, 16, 3, 7, 3, 2),         # general kernel (7x7, three channels)
+    (1, 64, 12, 12, 32, 64, 1, 0, 1),       # 1x1 plane kernel, 32-row tiles
+]
+
+
+@pytest.mark.parametrize("case", RESIDUAL_CONV_CASES)
+@pytest.mark.parametrize("deterministic", [0, 1])
+def test_conv2d_with_residual_bit_exact(ops, case, deterministic):
+    """pet_hip_conv2d_res_f32: relu(conv + bias + residual) in one call equals the
+    oracle's conv, bias, Add and ReLU applied one after the other."""
+    from pet_amd import abi
+    n, c, h, w, f, cpg, r, pad, st = case
+    rng = np.random.default_rng(21)
+    x, wt = ints(rng, (n, c, h, w), -2, 3), ints(rng, (f, cpg, r, r), -2, 3)
+    b = ints(rng, (f,), -3, 4)
+    conv = oracle.conv2d(x, wt, pad, pad, st, st)
+    res = ints(rng, conv.shape, -9, 10)
+    ref = oracle.activation(oracle.eltwise("add", [oracle.bias_act(conv, b, "none"), res],
+                                           conv.shape), "relu")
+    abi.call("pet_hip_set_deterministic", deterministic)
+    try:
+        got = host(ops.conv2d(dev(x), dev(wt), pad, pad, st, st, bias=dev(b), act="relu",
+                              residual=dev(res)))
+    finally:
+        abi.call("pet_hip_set_deterministic", 0)
+    np.testing.assert_array_equal(got, ref)
+
+
+def test_conv2d_residual_must_not_be_the_output(ops):
+    from pet_amd import abi
+    x = torch.zeros((1, 8, 8, 8), device="cuda")
+    w = torch.zeros((8, 8, 3, 3), device="cuda")
+    y = torch.zeros((1, 8, 8, 8), device="cuda")
+    with pytest.raises(abi.PetHipError) as e:
+        ops.conv2d(x, w, 1, 1, out=y, residual=y)
+    assert e.value.status == 1
+
+
+@pytest.mark.parametrize("packed", [False, True])
+def test_conv3d_with_residual_bit_exact(ops, packed):
+    rng = np.random.default_rng(22)
+    x, wt = ints(rng, (1, 16, 6, 10, 10), -2, 3), ints(rng, (32, 16, 3, 3, 3), -2, 3)
+    b = ints(rng, (32,), -3, 4)
+    conv = oracle.conv3d(x, wt, (1, 1, 1), (1, 1, 1), (1, 1, 1))
+    res = ints(rng, conv.shape, -9, 10)
+    ref = oracle.activation(oracle.eltwise("add", [oracle.bias_act(conv, b, "none"), res],
+                                           conv.shape), "relu")
+    filt = ops.conv3d_pack_filters(dev(wt)) if packed else dev(wt)
+    got = host(ops.conv3d(dev(x), filt, (1, 1, 1), bias=dev(b), act="relu", residual=dev(res)))
+    np.testing.assert_array_equal(got, ref)
+
+
+@pytest.mark.parametrize("tB", [False, True])
+@pytest.mark.parametrize("shape", [(1, 128, 96, 64), (3, 20, 36, 32), (2, 5, 7, 4)])
+def test_matmul_with_residual_bit_exact(ops, shape, tB):
+    """Plane-kernel path (no transposes, k % 32 == 0) and the general kernel, whose
+    residual is added by a following launch."""
+    b, m, n, k = shape
+    rng = np.random.default_rng(23)
+    A = ints(rng, (b, m, k))
+    B = ints(rng, (b, n, k) if tB else (b, k, n))
+    bias, res = ints(rng, (n,), -3, 4), ints(rng, (b, m, n), -9, 10)
+    ref = oracle.activation(
+        oracle.eltwise("add", [oracle.bias_act(oracle.matmul(A, B, False, tB), bias, "none",
+                                               ch_axis=2), res], res.shape), "relu")
+    got = host(ops.matmul(dev(A), dev(B), False, tB, bias=dev(bias), act="relu",
+                          residual=dev(res)))
+    np.testing.assert_array_equal(got, ref)
+
+
 def test_batch_gemm_merge_identity(ops):
     # src/Test/batch_gemm_test.cc: concat lhs, concat rhs, bmm, split == two matmuls
     m, n, k = 8, 8, 4
