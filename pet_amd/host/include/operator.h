@@ -122,6 +122,14 @@ class Operator {
     virtual Dim computeShape() = 0;
     virtual bool computeShape(const TensorVec &ins, const TensorVec &outs);
 
+    // Contractions only (Conv, Conv3d, Matmul): one launch of
+    // out = finalAct(op(inputs) + bias + residual), residual and out laid out like
+    // the operator's output. The graph runtime uses it to run "contraction, Add,
+    // activation" as one operator. PET_HIP_ERR_UNSUPPORTED elsewhere.
+    virtual int launchFused(pet_hip_stream_t stream, const float *residual, ActType finalAct,
+                            float *out);
+    virtual bool canTakeResidual() const { return false; }
+
     virtual int numInputs() = 0;
     virtual int numOutputs() = 0;
     void print() const { std::cout << toString() << std::endl; }
@@ -181,6 +189,9 @@ class ConvOp : public Operator {
     Dim computeOutputPenalty(const Dim &p);
     double perf(PerfEngine *pe, int rounds = 200, int warmupRounds = 200) override;
     int launch(pet_hip_stream_t stream) override;
+    int launchFused(pet_hip_stream_t stream, const float *residual, ActType finalAct,
+                    float *out) override;
+    bool canTakeResidual() const override { return act == None; }
     std::string toString() const override;
     int numInputs() override { return 2; }
     int numOutputs() override { return 1; }
@@ -230,6 +241,9 @@ class Conv3dOp : public Operator {
     Dim computeShape() override;
     double perf(PerfEngine *pe, int rounds = 200, int warmupRounds = 200) override;
     int launch(pet_hip_stream_t stream) override;
+    int launchFused(pet_hip_stream_t stream, const float *residual, ActType finalAct,
+                    float *out) override;
+    bool canTakeResidual() const override { return act == None; }
     std::string toString() const override;
     int numInputs() override { return 2; }
     int numOutputs() override { return 1; }
@@ -270,6 +284,9 @@ class MatmulOp : public Operator {
     Dim computeShape() override;
     double perf(PerfEngine *pe, int rounds = 200, int warmupRounds = 200) override;
     int launch(pet_hip_stream_t stream) override;
+    int launchFused(pet_hip_stream_t stream, const float *residual, ActType finalAct,
+                    float *out) override;
+    bool canTakeResidual() const override { return act == None; }
     std::string toString() const override;
     int numInputs() override { return 2; }
     int numOutputs() override { return 1; }

@@ -2,6 +2,7 @@
 
 #include <algorithm>
 #include <fstream>
+#include <functional>
 #include <map>
 #include <set>
 #include <sstream>
@@ -100,6 +101,74 @@ TransposeChains planTransposeChains(const OpVec &order, const TensorVec &graphOu
                 plan.folded.insert(row[i]);
             plan.chains[op] = row;
         }
+    }
+    return plan;
+}
+
+// "Contraction, Add with another tensor, activation" as one operator: the
+// contraction's residual operand takes the other tensor and its epilogue the
+// activation (cuDNN's fused convolution has the same z operand; the reference
+// passes it with weight 0, src/Graph/code_engine.cc:955-977). The fused operator
+// runs where the Add stood, when both of its inputs exist.
+struct FusedTail {
+    Operator *contraction = nullptr;
+    Tensor *residual = nullptr;
+    Operator::ActType act = Operator::None;
+    Tensor *out = nullptr;
+};
+
+struct FusedTails {
+    std::set<const Operator *> absorbed;          // contractions and activations that moved
+    std::map<const Operator *, FusedTail> atAdd;  // keyed by the Add they run in place of
+};
+
+FusedTails planFusedTails(const OpVec &order, const TensorVec &graphOutputs,
+                          const std::set<const Operator *> &skipped,
+                          const std::function<bool(const FusedTail &)> &storageOk) {
+    FusedTails plan;
+    std::set<const Tensor *> outs(graphOutputs.begin(), graphOutputs.end());
+    std::map<const Operator *, size_t> pos;
+    for (size_t i = 0; i < order.size(); ++i)
+        pos[order[i]] = i;
+    for (auto op : order) {
+        if (op->getType() != Operator::Add || op->getInputs().size() != 2 || skipped.count(op))
+            continue;
+        Tensor *sum = op->getOutputs()[0];
+        Operator *pick = nullptr;
+        Tensor *other = nullptr;
+        for (int side = 0; side < 2; ++side) {
+            Tensor *a = op->getInputs()[side], *b = op->getInputs()[1 - side];
+            Operator *prod = a->getOutputOf();
+            if (prod == nullptr || !prod->canTakeResidual() || skipped.count(prod) ||
+                plan.absorbed.count(prod) || weightOnly(prod) || a == b ||
+                a->getInputOf().size() != 1 || outs.count(a) || a->size() != sum->size() ||
+                b->size() != sum->size() || prod->getOutputs().size() != 1)
+                continue;
+            if (pick == nullptr || pos[prod] > pos[pick]) { // the later one: its partner exists
+                pick = prod;
+                other = b;
+            }
+        }
+        if (pick == nullptr)
+            continue;
+        FusedTail tail;
+        tail.contraction = pick;
+        tail.residual = other;
+        tail.out = sum;
+        const OpVec &users = sum->getInputOf();
+        ActivationOp *actOp = nullptr;
+        if (users.size() == 1 && !outs.count(sum) && !skipped.count(users[0]))
+            actOp = dynamic_cast<ActivationOp *>(users[0]);
+        if (actOp) {
+            tail.act = actOp->getActType();
+            tail.out = actOp->getOutputs()[0];
+        }
+        if (!storageOk(tail)) // residual and result share a buffer: keep the operators apart
+            continue;
+        if (actOp)
+            plan.absorbed.insert(actOp);
+        plan.absorbed.insert(pick);
+        plan.atAdd[op] = tail;
     }
     return plan;
 }
@@ -212,7 +281,17 @@ std::unique_ptr<GraphExec> CodeEngine::instantiate(std::shared_ptr<SubGraph> &gr
     }
     AliasPlan plan = planAliases(order);
     TransposeChains rows = planTransposeChains(order, graph->getOutputs(), plan.skipped);
-    auto launchOp = [&](Operator *op, pet_hip_stream_t st) {
+    FusedTails tails = planFusedTails(order, graph->getOutputs(), plan.skipped,
+                                      [](const FusedTail &f) {
+                                          return f.residual->devicePtr() != f.out->devicePtr();
+                                      });
+    auto launchOp = [&](Operator *op, pet_hip_stream_t st) -> int {
+        auto tail = tails.atAdd.find(op);
+        if (tail != tails.atAdd.end()) {
+            const FusedTail &f = tail->second;
+            return f.contraction->launchFused(st, f.residual->devicePtr(), f.act,
+                                              f.out->devicePtr());
+        }
         auto it = rows.chains.find(op);
         return it == rows.chains.end() ? op->launch(st) : launchChain(it->second, st);
     };
@@ -246,7 +325,7 @@ std::unique_ptr<GraphExec> CodeEngine::instantiate(std::shared_ptr<SubGraph> &gr
         }
         if (weightOnly(op))
             continue;
-        if (rows.folded.count(op)) {
+        if (rows.folded.count(op) || tails.absorbed.count(op)) {
             exec->nFoldedOps++;
             continue;
         }
@@ -267,6 +346,14 @@ std::unique_ptr<GraphExec> CodeEngine::instantiate(std::shared_ptr<SubGraph> &gr
     exec->graph = g;
     for (auto t : graph->getTensors())
         if (t->getOutputOf() != nullptr && !rows.folded.count(t->getOutputOf())) {
+            // what a fused tail absorbed is not materialised either, except its last tensor
+            const Operator *prod = t->getOutputOf();
+            bool inside = tails.absorbed.count(prod) && dynamic_cast<const ActivationOp *>(prod) == nullptr;
+            auto tail = tails.atAdd.find(prod);
+            if (tail != tails.atAdd.end() && tail->second.out != t)
+                inside = true;
+            if (inside)
+                continue;
             t->deviceWritten();
             t->setComputed();
         }
@@ -397,34 +484,55 @@ std::string CodeEngine::genCode(std::shared_ptr<SubGraph> &graph) {
         e.line(l);
 
     std::map<const Operator *, std::string> packedName; // Conv3d -> its kt-major filter copy
-    auto emitOp = [&](Operator *op) -> bool {
+    FusedTails tails = planFusedTails(order, graph->getOutputs(), skipped, [&](const FusedTail &f) {
+        return !viewOf.count(f.residual) && !viewOf.count(f.out);
+    });
+    // set while a contraction is emitted in place of the Add that follows it
+    const FusedTail *tail = nullptr;
+    std::function<bool(Operator *)> emitOp = [&](Operator *op) -> bool {
         std::ostringstream c;
         auto in = [&](size_t i) { return e.name(op->getInputs()[i]); };
-        auto out = [&](size_t i) { return e.name(op->getOutputs()[i]); };
+        auto out = [&](size_t i) {
+            return tail ? e.name(tail->out) : e.name(op->getOutputs()[i]);
+        };
+        const std::string res = tail ? e.name(tail->residual) + ", " : "";
+        auto actOf = [&](Operator::ActType own) { return (int)(tail ? tail->act : own); };
+        if (tails.atAdd.count(op) && tail == nullptr) {
+            tail = &tails.atAdd.at(op);
+            bool ok = emitOp(tail->contraction);
+            tail = nullptr;
+            return ok;
+        }
         if (auto conv = dynamic_cast<ConvOp *>(op)) {
             auto d = op->getInputs()[0]->getDims(), w = op->getInputs()[1]->getDims();
-            c << "pet_hip_conv2d_f32(" << in(0) << ", " << in(1) << ", "
-              << nullable(e, conv->getBias()) << ", " << out(0) << ", " << d[0] << ", " << d[1]
+            c << (tail ? "pet_hip_conv2d_res_f32(" : "pet_hip_conv2d_f32(") << in(0) << ", " << in(1)
+              << ", " << nullable(e, conv->getBias()) << ", " << res << out(0) << ", " << d[0]
+              << ", " << d[1]
               << ", " << d[2] << ", " << d[3] << ", " << w[0] << ", " << w[2] << ", " << w[3]
               << ", " << conv->getPh() << ", " << conv->getPw() << ", " << conv->getSh() << ", "
               << conv->getSw() << ", " << conv->getDh() << ", " << conv->getDw() << ", "
-              << d[1] / w[1] << ", " << (int)conv->getAct() << ", s)";
+              << d[1] / w[1] << ", " << actOf(conv->getAct()) << ", s)";
         } else if (auto c3 = dynamic_cast<Conv3dOp *>(op)) {
             auto d = op->getInputs()[0]->getDims(), w = op->getInputs()[1]->getDims();
             // filters with a kt-major copy (made before capture, below) use it
-            if (packedName.count(op))
+            const bool pk = packedName.count(op) != 0;
+            const std::string filt =
+                pk ? packedName[op] + "_ok ? " + packedName[op] + " : " + in(1) : in(1);
+            if (tail)
+                c << "pet_hip_conv3d_res_f32(" << in(0) << ", " << filt << ", "
+                  << (pk ? packedName[op] + "_ok" : std::string("0")) << ", ";
+            else if (pk)
                 c << "(" << packedName[op] << "_ok ? pet_hip_conv3d_packed_f32 : "
-                  << "pet_hip_conv3d_f32)(" << in(0) << ", " << packedName[op] << "_ok ? "
-                  << packedName[op] << " : " << in(1) << ", ";
+                  << "pet_hip_conv3d_f32)(" << in(0) << ", " << filt << ", ";
             else
                 c << "pet_hip_conv3d_f32(" << in(0) << ", " << in(1) << ", ";
-            c << nullable(e, c3->getBias()) << ", " << out(0);
+            c << nullable(e, c3->getBias()) << ", " << res << out(0);
             for (int v : {d[0], d[1], d[2], d[3], d[4], w[0], w[2], w[3], w[4]})
                 c << ", " << v;
             for (const Dim *v : {&c3->getPad(), &c3->getStride(), &c3->getDilation()})
                 for (int x : *v)
                     c << ", " << x;
-            c << ", " << d[1] / w[1] << ", " << (int)c3->getAct() << ", s)";
+            c << ", " << d[1] / w[1] << ", " << actOf(c3->getAct()) << ", s)";
         } else if (auto ln = dynamic_cast<LayerNormOp *>(op)) {
             size_t cols = (size_t)op->getInputs()[0]->getDims().back();
             c << "pet_hip_layernorm(" << in(0) << ", " << nullable(e, ln->getGamma()) << ", "
@@ -435,9 +543,11 @@ std::string CodeEngine::genCode(std::shared_ptr<SubGraph> &graph) {
             bool ta, tb;
             int b, m, n, k;
             std::tie(ta, tb, b, m, n, k) = mm->getArgs();
-            c << "pet_hip_bmm_f32(" << ta << ", " << tb << ", " << b << ", " << m << ", " << n
-              << ", " << k << ", " << in(0) << ", " << in(1) << ", " << out(0) << ", "
-              << nullable(e, mm->getBias()) << ", " << (int)mm->getAct() << ", s)";
+            c << (tail ? "pet_hip_bmm_res_f32(" : "pet_hip_bmm_f32(") << ta << ", " << tb << ", " << b
+              << ", " << m << ", " << n << ", " << k << ", " << in(0) << ", " << in(1) << ", "
+              << out(0) << ", " << nullable(e, mm->getBias()) << ", "
+              << (tail ? e.name(tail->residual) + ", " : std::string()) << actOf(mm->getAct())
+              << ", s)";
         } else if (auto tr = dynamic_cast<TransposeOp *>(op)) {
             TransProgram prog;
             std::vector<TransposeOp *> row = {tr};
@@ -543,7 +653,8 @@ std::string CodeEngine::genCode(std::shared_ptr<SubGraph> &graph) {
     e.line("    int odims[PET_HIP_MAX_RANK], orank = 0; (void)odims; (void)orank;");
     e.line("    // operators that only touch weights run once");
     for (auto op : order)
-        if (weightOnly(op) && !skipped.count(op) && !rows.folded.count(op) && !emitOp(op))
+        if (weightOnly(op) && !skipped.count(op) && !rows.folded.count(op) &&
+            !tails.absorbed.count(op) && !emitOp(op))
             return "";
     e.line("    // constant 3-D filters: kt-major copy where the backend has that form");
     for (auto op : order) {
@@ -565,7 +676,8 @@ std::string CodeEngine::genCode(std::shared_ptr<SubGraph> &graph) {
     e.line("    // the rest is captured once and replayed as a HIP graph");
     e.line("    CHECK(pet_hip_graph_begin_capture(s));");
     for (auto op : order)
-        if (!weightOnly(op) && !skipped.count(op) && !rows.folded.count(op) && !emitOp(op))
+        if (!weightOnly(op) && !skipped.count(op) && !rows.folded.count(op) &&
+            !tails.absorbed.count(op) && !emitOp(op))
             return "";
     e.line("    pet_hip_graph_t g; CHECK(pet_hip_graph_end_capture(s, &g));");
     e.line("    pet_hip_event_t st, ed; CHECK(pet_hip_event_create(&st)); "

@@ -63,6 +63,10 @@ Tensor *Operator::compute() {
     return outputs[0];
 }
 
+int Operator::launchFused(pet_hip_stream_t, const float *, ActType, float *) {
+    return PET_HIP_ERR_UNSUPPORTED;
+}
+
 std::pair<std::vector<DimRange>, std::function<bool()>> Operator::compute(DimRange dr) {
     if (dr.notValid())
         return {};
@@ -302,6 +306,18 @@ int ConvOp::launch(pet_hip_stream_t stream) {
                               groups, (int)act, stream);
 }
 
+int ConvOp::launchFused(pet_hip_stream_t stream, const float *residual, ActType finalAct,
+                        float *out) {
+    auto in = inputs[0]->getDims(), wt = inputs[1]->getDims();
+    int groups = in[1] / wt[1];
+    if (groups <= 0 || wt[0] % groups != 0 || act != None)
+        return PET_HIP_ERR_INVALID;
+    return pet_hip_conv2d_res_f32(inputs[0]->devicePtr(), inputs[1]->devicePtr(),
+                                  bias ? bias->devicePtr() : nullptr, residual, out, in[0], in[1],
+                                  in[2], in[3], wt[0], wt[2], wt[3], ph, pw, sh, sw, dh, dw, groups,
+                                  (int)finalAct, stream);
+}
+
 double ConvOp::perf(PerfEngine *pe, int rounds, int warmupRounds) {
     ConvArgs args = getArgs(pe->withPenalty());
     if (pe->checkOpPerf(Conv, args))
@@ -444,6 +460,21 @@ int Conv3dOp::launch(pet_hip_stream_t stream) {
                  dilation[1], dilation[2], groups, (int)act, stream);
 }
 
+int Conv3dOp::launchFused(pet_hip_stream_t stream, const float *residual, ActType finalAct,
+                          float *out) {
+    auto in = inputs[0]->getDims(), wt = inputs[1]->getDims();
+    int groups = in[1] / wt[1];
+    if (groups <= 0 || wt[0] % groups != 0 || act != None)
+        return PET_HIP_ERR_INVALID;
+    const bool usePacked = usesPackedFilters();
+    return pet_hip_conv3d_res_f32(inputs[0]->devicePtr(), usePacked ? packed : inputs[1]->devicePtr(),
+                                  usePacked, bias ? bias->devicePtr() : nullptr, residual, out,
+                                  in[0], in[1], in[2], in[3], in[4], wt[0], wt[2], wt[3], wt[4],
+                                  pad[0], pad[1], pad[2], stride[0], stride[1], stride[2],
+                                  dilation[0], dilation[1], dilation[2], groups, (int)finalAct,
+                                  stream);
+}
+
 double Conv3dOp::perf(PerfEngine *, int rounds, int warmupRounds) {
     return timeLaunches(rounds, warmupRounds);
 }
@@ -536,6 +567,18 @@ int MatmulOp::launch(pet_hip_stream_t stream) {
     return pet_hip_bmm_f32(ta, tb, b, m, n, k, inputs[0]->devicePtr(), inputs[1]->devicePtr(),
                            outputs[0]->devicePtr(), bias ? bias->devicePtr() : nullptr, (int)act,
                            stream);
+}
+
+int MatmulOp::launchFused(pet_hip_stream_t stream, const float *residual, ActType finalAct,
+                          float *out) {
+    if (act != None)
+        return PET_HIP_ERR_INVALID;
+    bool ta, tb;
+    int b, m, n, k;
+    std::tie(ta, tb, b, m, n, k) = getArgs();
+    return pet_hip_bmm_res_f32(ta, tb, b, m, n, k, inputs[0]->devicePtr(), inputs[1]->devicePtr(),
+                               out, bias ? bias->devicePtr() : nullptr, residual, (int)finalAct,
+                               stream);
 }
 
 double MatmulOp::perf(PerfEngine *pe, int rounds, int warmupRounds) {

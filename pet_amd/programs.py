@@ -36,11 +36,16 @@ class GpuNS:
         self.t.cuda.synchronize()
         return t.cpu().numpy()
 
-    def conv2d(self, x, w, ph, pw, sh=1, sw=1, dh=1, dw=1, bias=None, act="none"):
-        return self._k(self.ops.conv2d(x, w, ph, pw, sh, sw, dh, dw, bias=bias, act=act))
+    # residual: a tensor of the output's shape added before the activation (the
+    # contraction, the Add and the activation of a block's tail as one operator)
+    def conv2d(self, x, w, ph, pw, sh=1, sw=1, dh=1, dw=1, bias=None, act="none", residual=None):
+        return self._k(self.ops.conv2d(x, w, ph, pw, sh, sw, dh, dw, bias=bias, act=act,
+                                       residual=residual))
 
-    def conv3d(self, x, w, pad, stride=(1, 1, 1), dil=(1, 1, 1), bias=None, act="none"):
-        return self._k(self.ops.conv3d(x, w, pad, stride, dil, bias=bias, act=act))
+    def conv3d(self, x, w, pad, stride=(1, 1, 1), dil=(1, 1, 1), bias=None, act="none",
+               residual=None):
+        return self._k(self.ops.conv3d(x, w, pad, stride, dil, bias=bias, act=act,
+                                       residual=residual))
 
     def filters3d(self, w):
         """Constant 3-D filters in the form conv3d reads fastest (kt-major where
@@ -48,8 +53,9 @@ class GpuNS:
         packed = self.ops.conv3d_pack_filters(w)
         return w if packed is None else packed
 
-    def matmul(self, A, B, transA=False, transB=False, bias=None, act="none"):
-        return self._k(self.ops.matmul(A, B, transA, transB, bias=bias, act=act))
+    def matmul(self, A, B, transA=False, transB=False, bias=None, act="none", residual=None):
+        return self._k(self.ops.matmul(A, B, transA, transB, bias=bias, act=act,
+                                       residual=residual))
 
     def permute_flat(self, x, flat, perm):
         return self._k(self.ops.permute_flat(x, flat, perm))
@@ -235,8 +241,8 @@ def run_c3(ns, p, transformed=False, T=None):
                 idn = x
                 if has_ds:
                     idn = ns.conv2d(x, T[pre + ".ds.w"], 0, 0, 2, 2, bias=T[pre + ".ds.b"])
-            y = ns.conv2d(y, T[pre + ".c2.w"], 1, 1, bias=T[pre + ".c2.b"])
-            x = ns.act(ns.add([y, idn]), "relu")
+            x = ns.conv2d(y, T[pre + ".c2.w"], 1, 1, bias=T[pre + ".c2.b"], residual=idn,
+                          act="relu")
     n, c, h, w = tuple(x.shape)
     x = ns.pool2d(x, h, w, 0, 0, 1, 1, mode="avg")
     x = ns.reshape(x, (1, 1, c))
@@ -303,11 +309,11 @@ def run_c4(ns, p, transformed=False, T=None):
         s = ns.softmax(ns.mul([s, scale]))
         ctx = ns.matmul(s, vh)                             # [heads, seq, dh]
         ctx = ns.reshape(ns.transpose(ctx, -1, [1, 0, 2]), (1, seq, hidden))
-        att = ns.matmul(ctx, T[pre + "o.w"], bias=T[pre + "o.b"])
-        x = ns.layernorm(ns.add([x, att]), T[pre + "ln1.g"], T[pre + "ln1.b"])
+        att = ns.matmul(ctx, T[pre + "o.w"], bias=T[pre + "o.b"], residual=x)
+        x = ns.layernorm(att, T[pre + "ln1.g"], T[pre + "ln1.b"])
         h = ns.matmul(x, T[pre + "f1.w"], bias=T[pre + "f1.b"], act="gelu")
-        h = ns.matmul(h, T[pre + "f2.w"], bias=T[pre + "f2.b"])
-        x = ns.layernorm(ns.add([x, h]), T[pre + "ln2.g"], T[pre + "ln2.b"])
+        h = ns.matmul(h, T[pre + "f2.w"], bias=T[pre + "f2.b"], residual=x)
+        x = ns.layernorm(h, T[pre + "ln2.g"], T[pre + "ln2.b"])
     return x
 
 
@@ -370,11 +376,10 @@ def run_c5(ns, p, transformed=False, T=None):
                     z = ns.conv3d(ys, T[pre + ".c2.w"], (1, 1, 1), bias=T[pre + ".c2.b"])
                     y = ns.trans_chain(z, [("split", 0, 2, 0, 0),
                                            ("reorder", [0, 2, 1, 3, 4, 5]), ("fuse", 2, 0, 1)])
-                else:
-                    y = ns.conv3d(y, T[pre + ".c2.w"], (1, 1, 1), bias=T[pre + ".c2.b"])
-            else:
-                y = ns.conv3d(y, T[pre + ".c2.w"], (1, 1, 1), bias=T[pre + ".c2.b"])
-            x = ns.act(ns.add([y, idn]), "relu")
+                    x = ns.act(ns.add([y, idn]), "relu")
+                    continue
+            x = ns.conv3d(y, T[pre + ".c2.w"], (1, 1, 1), bias=T[pre + ".c2.b"], residual=idn,
+                          act="relu")
     n, c, t, h, w = tuple(x.shape)
     x = ns.pool2d(ns.reshape(x, (1, c, t, h * w)), t, h * w, 0, 0, 1, 1, mode="avg")
     x = ns.reshape(x, (1, 1, c))

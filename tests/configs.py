@@ -20,17 +20,23 @@ class OracleNS:
     def numpy(self, t):
         return t
 
-    def conv2d(self, x, w, ph, pw, sh=1, sw=1, dh=1, dw=1, bias=None, act="none"):
-        y = self.o.conv2d(x, w, ph, pw, sh, sw, dh, dw)
-        return self.o.bias_act(y, bias, act) if (bias is not None or act != "none") else y
+    def _tail(self, y, bias, act, residual, ch_axis=1):
+        """bias, then the residual Add, then the activation: operator by operator."""
+        if bias is not None:
+            y = self.o.bias_act(y, bias, "none", ch_axis=ch_axis)
+        if residual is not None:
+            y = self.o.eltwise("add", [y, residual.reshape(y.shape)], y.shape)
+        return self.o.activation(y, act) if act != "none" else y
 
-    def conv3d(self, x, w, pad, stride=(1, 1, 1), dil=(1, 1, 1), bias=None, act="none"):
-        y = self.o.conv3d(x, w, pad, stride, dil)
-        return self.o.bias_act(y, bias, act) if (bias is not None or act != "none") else y
+    def conv2d(self, x, w, ph, pw, sh=1, sw=1, dh=1, dw=1, bias=None, act="none", residual=None):
+        return self._tail(self.o.conv2d(x, w, ph, pw, sh, sw, dh, dw), bias, act, residual)
 
-    def matmul(self, A, B, transA=False, transB=False, bias=None, act="none"):
-        y = self.o.matmul(A, B, transA, transB)
-        return self.o.bias_act(y, bias, act, ch_axis=2) if (bias is not None or act != "none") else y
+    def conv3d(self, x, w, pad, stride=(1, 1, 1), dil=(1, 1, 1), bias=None, act="none",
+               residual=None):
+        return self._tail(self.o.conv3d(x, w, pad, stride, dil), bias, act, residual)
+
+    def matmul(self, A, B, transA=False, transB=False, bias=None, act="none", residual=None):
+        return self._tail(self.o.matmul(A, B, transA, transB), bias, act, residual, ch_axis=2)
 
     def permute_flat(self, x, flat, perm):
         return self.o.permute_flat(x, flat, perm)

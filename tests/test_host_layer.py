@@ -323,3 +323,32 @@ def test_model_graph_replay_equals_operator_by_operator_run(model):
     assert rec["ms"] > 0
     if model == "dilated:pet":
         assert rec["folded"] == 2 and rec["kernels"] == 8
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("model", ["resnet18", "resnet3d18", "bert"])
+def test_emitted_model_program_compiles_and_agrees_with_the_runtime(model, tmp_path):
+    """CodeEngine::genCode for a whole network (fused block tails, kt-major filters,
+    storage sharing): the emitted C++ builds against pet_hip.h alone, runs, and its
+    time per iteration is that of the in-process graph."""
+    import json
+    import re
+    src = tmp_path / "net.cpp"
+    res = subprocess.run([RUN_MODEL, model, "--rounds", "50", "--warmup", "5", "--emit", str(src)],
+                         capture_output=True, text=True, timeout=300)
+    assert res.returncode == 0, res.stderr[-2000:]
+    rec = json.loads(res.stdout.strip().splitlines()[-1])
+    text = src.read_text()
+    if model != "bert":
+        assert "_res_f32(" in text               # a block tail became one call
+    else:
+        assert "pet_hip_bmm_res_f32(" in text
+    if model == "resnet3d18":
+        assert "pet_hip_conv3d_pack_filters(" in text
+    exe = tmp_path / "net"
+    subprocess.run(["g++", "-O1", str(src), "-I", os.path.join(ROOT, "include"), "-L", LIB,
+                    "-lpet_hip", "-Wl,-rpath," + LIB, "-o", str(exe)], check=True)
+    run = subprocess.run([str(exe)], capture_output=True, text=True, timeout=300)
+    assert run.returncode == 0, run.stdout + run.stderr
+    ms = float(re.search(r"Time\(ms\)\D*([0-9.eE+-]+)", run.stdout).group(1))
+    assert 0.7 * rec["ms"] <= ms <= 1.4 * rec["ms"], (ms, rec["ms"])
