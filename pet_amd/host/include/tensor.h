@@ -86,6 +86,11 @@ class Tensor {
     void aliasDevice(float *ptr);
     // Marks the device copy as just written by a kernel.
     void deviceWritten();
+    // A caller that took getDataPtr() before the tensor was computed keeps reading
+    // through that pointer afterwards (the reference's tests do: there the pointer
+    // is the data). If a host mirror of the right size exists, bring it up to date
+    // in place; Operator::compute() calls this for its outputs.
+    void refreshHostMirrorInPlace();
     // Counts the writes to this tensor's values (dataRand, setData, a kernel's
     // output, a host pointer handed out): lets a holder of derived data, such as
     // repacked filters, see that it is out of date.

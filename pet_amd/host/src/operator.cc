@@ -59,6 +59,7 @@ Tensor *Operator::compute() {
     for (auto t : outputs) {
         t->deviceWritten();
         t->setComputed();
+        t->refreshHostMirrorInPlace();
     }
     return outputs[0];
 }

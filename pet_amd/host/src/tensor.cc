@@ -84,6 +84,9 @@ void Tensor::clear() {
     splittingPoints.clear();
     hash = generateHash();
     dimPenalty.clear();
+    // a recycled tensor starts without a host mirror (the device buffer stays)
+    std::vector<VType>().swap(host);
+    hostFresh = false;
 }
 
 const Dim &Tensor::getPenalty() {
@@ -202,6 +205,15 @@ void Tensor::aliasDevice(float *ptr) {
     ownsDev = false;
     devFresh = true;
     hostFresh = false;
+}
+
+void Tensor::refreshHostMirrorInPlace() {
+    if (host.size() != size() || host.empty() || hostFresh || !dev || !devFresh)
+        return;
+    pet_hip_stream_sync(petStream());
+    if (petOk(pet_hip_memcpy_d2h(host.data(), dev, size() * sizeof(float), petStream()),
+              "pet_hip_memcpy_d2h"))
+        hostFresh = true;
 }
 
 void Tensor::deviceWritten() {
