@@ -402,6 +402,81 @@ def test_matmul_with_residual_bit_exact(ops, shape, tB):
     np.testing.assert_array_equal(got, ref)
 
 
+def test_random_contractions_with_residual_and_packed_filters(ops):
+    """120 seeded random cases over the three contractions with bias, ReLU, and at
+    random a residual operand, grouped filters, strides, dilations, transposed matmul
+    operands and kt-major 3-D filters; small integers, so every result must equal the
+    oracle's conv / matmul, bias, Add, ReLU applied one after the other bit for bit."""
+    rng = np.random.default_rng(4242)
+
+    def tail(y, b, res, ch_axis=1):
+        y = oracle.bias_act(y, b, "none", ch_axis=ch_axis)
+        if res is not None:
+            y = oracle.eltwise("add", [y, res], y.shape)
+        return oracle.activation(y, "relu")
+
+    done = 0
+    while done < 120:
+        kind = rng.choice(["conv2d", "conv3d", "bmm"])
+        use_res = rng.random() < 0.5
+        if kind == "conv2d":
+            g = int(rng.choice([1, 1, 2, 4]))
+            cpg = int(rng.choice([1, 3, 8, 16, 32, 64]))
+            f = g * int(rng.choice([1, 2, 5, 8, 16, 33, 64]))
+            r = int(rng.choice([1, 3, 3, 5]))
+            s = int(rng.choice([r, 1, 3]))
+            h, w = int(rng.integers(max(r, 3), 36)), int(rng.integers(max(s, 3), 36))
+            n = int(rng.choice([1, 2, 4]))
+            ph, pw = int(rng.integers(0, 3)), int(rng.integers(0, 3))
+            sh, sw = int(rng.choice([1, 1, 2])), int(rng.choice([1, 1, 2]))
+            dh, dw = int(rng.choice([1, 1, 2])), int(rng.choice([1, 1, 2]))
+            if min(oracle.conv_out_dim(h, r, ph, sh, dh), oracle.conv_out_dim(w, s, pw, sw, dw)) <= 0:
+                continue
+            x, wt = ints(rng, (n, cpg * g, h, w), -2, 3), ints(rng, (f, cpg, r, s), -2, 3)
+            b = ints(rng, (f,), -3, 4)
+            conv = oracle.conv2d(x, wt, ph, pw, sh, sw, dh, dw)
+            res = ints(rng, conv.shape, -9, 10) if use_res else None
+            got = host(ops.conv2d(dev(x), dev(wt), ph, pw, sh, sw, dh, dw, bias=dev(b), act="relu",
+                                  residual=dev(res) if use_res else None))
+            ref = tail(conv, b, res)
+        elif kind == "conv3d":
+            g = int(rng.choice([1, 1, 2]))
+            cpg = int(rng.choice([2, 8, 16, 32]))
+            f = g * int(rng.choice([2, 8, 16, 40]))
+            kt, r = int(rng.choice([1, 3, 3])), int(rng.choice([1, 3, 3]))
+            t, h, w = int(rng.integers(kt, 8)), int(rng.integers(3, 16)), int(rng.integers(3, 16))
+            pad = tuple(int(v) for v in rng.integers(0, 2, 3))
+            st = (int(rng.choice([1, 1, 2])),) * 3
+            dl = (int(rng.choice([1, 1, 2])), 1, 1)
+            if min(oracle.conv_out_dim(t, kt, pad[0], st[0], dl[0]),
+                   oracle.conv_out_dim(h, r, pad[1], st[1], 1),
+                   oracle.conv_out_dim(w, r, pad[2], st[2], 1)) <= 0:
+                continue
+            x, wt = ints(rng, (1, cpg * g, t, h, w), -2, 3), ints(rng, (f, cpg, kt, r, r), -2, 3)
+            b = ints(rng, (f,), -3, 4)
+            conv = oracle.conv3d(x, wt, pad, st, dl)
+            res = ints(rng, conv.shape, -9, 10) if use_res else None
+            filt = dev(wt)
+            packed = ops.conv3d_pack_filters(filt) if rng.random() < 0.6 else None
+            got = host(ops.conv3d(dev(x), packed if packed is not None else filt, pad, st, dl,
+                                  bias=dev(b), act="relu", residual=dev(res) if use_res else None))
+            ref = tail(conv, b, res)
+        else:
+            bb, m, n = int(rng.choice([1, 2, 3, 12])), int(rng.integers(1, 150)), int(rng.integers(1, 150))
+            k = int(rng.choice([4, 32, 64, 96, 100, 768]))
+            tA, tB = bool(rng.integers(0, 2)), bool(rng.integers(0, 2))
+            A = ints(rng, (bb, k, m) if tA else (bb, m, k))
+            B = ints(rng, (bb, n, k) if tB else (bb, k, n))
+            b = ints(rng, (n,), -3, 4)
+            res = ints(rng, (bb, m, n), -9, 10) if use_res else None
+            got = host(ops.matmul(dev(A), dev(B), tA, tB, bias=dev(b), act="relu",
+                                  residual=dev(res) if use_res else None))
+            ref = tail(oracle.matmul(A, B, tA, tB), b, res, ch_axis=2)
+        assert got.shape == ref.shape
+        np.testing.assert_array_equal(got, ref)
+        done += 1
+
+
 def test_batch_gemm_merge_identity(ops):
     # src/Test/batch_gemm_test.cc: concat lhs, concat rhs, bmm, split == two matmuls
     m, n, k = 8, 8, 4
