@@ -313,6 +313,98 @@ static bool test_conv3d_prepacked_graph() {
     return true;
 }
 
+// Seeded random graphs through both executors: SubGraph::compute launches every
+// operator by itself, CodeEngine::instantiate plans storage sharing, folds rows of
+// transposes and fuses "contraction, Add, activation" tails. Small integers keep
+// every value exact, so the two must agree bit for bit whatever the plan.
+static bool test_random_graphs_replay_equals_eager() {
+    unsigned state = 12345;
+    auto rnd = [&](int n) {
+        state = state * 1664525u + 1013904223u;
+        return (int)((state >> 16) % (unsigned)n);
+    };
+    size_t folded = 0, aliased = 0;
+    for (int trial = 0; trial < 24; ++trial) {
+        Graph g;
+        const int c = 8, hw = 8 + 4 * rnd(3);
+        std::vector<Tensor *> live = {g.tensor({1, c, hw, hw})}; // same-shape tensors so far
+        std::vector<int> depth = {0};                            // convolutions behind each
+        int nops = 4 + rnd(5);
+        for (int i = 0; i < nops; ++i) {
+            int pick = rnd((int)live.size());
+            Tensor *x = live[pick];
+            int kind = rnd(5);
+            if (kind == 0 && depth[pick] < 2) { // convolution, sometimes with its own ReLU
+                auto op = static_cast<ConvOp *>(g.conv(x, g.tensor({c, c, 3, 3}), 1, 1));
+                if (rnd(2))
+                    op->setAct(Operator::Relu);
+                live.push_back(op->getOutputs()[0]);
+                depth.push_back(depth[pick] + 1);
+            } else if (kind == 1 && live.size() > 1) { // Add with another tensor
+                int other = rnd((int)live.size());
+                live.push_back(g.add({x, live[other]})->getOutputs()[0]);
+                depth.push_back(std::max(depth[pick], depth[other]));
+            } else if (kind == 2) {
+                live.push_back(g.relu(x)->getOutputs()[0]);
+                depth.push_back(depth[pick]);
+            } else if (kind == 3) { // rows de-interleaved into the batch and back: a row of two
+                auto a = g.transpose(x, 2, {{-1, 0}, 1, 2, 3}, 2);
+                auto b = g.transpose(a->getOutputs()[0], 0, {-1, 1, {2, 0}, 3}, -2);
+                live.push_back(b->getOutputs()[0]);
+                depth.push_back(depth[pick]);
+            } else { // split on the batch axis of a doubled tensor, then use one half
+                auto cat = g.concat({x, x}, 0);
+                auto sp = g.split(cat->getOutputs()[0], 0, 2);
+                live.push_back(sp->getOutputs()[rnd(2)]);
+                depth.push_back(depth[pick]);
+            }
+        }
+        // one sink so that every branch matters: the sum of all tensors nobody consumed
+        g.updateConnection();
+        TensorVec loose;
+        for (auto t : g.getTensors())
+            if (t->getInputOf().empty() && (t->getOutputOf() != nullptr || t == live[0]))
+                loose.push_back(t);
+        while (loose.size() > 1) {
+            Tensor *a = loose.back();
+            loose.pop_back();
+            Tensor *b = loose.back();
+            loose.pop_back();
+            loose.push_back(g.add({a, b})->getOutputs()[0]);
+        }
+        g.updateConnection();
+        auto s1 = std::make_shared<SubGraph>(g.getOperators());
+        auto s2 = std::make_shared<SubGraph>(g.getOperators());
+        EXPECT(s1->getInputs().size() == s2->getInputs().size());
+        for (size_t i = 0; i < s1->getInputs().size(); ++i) {
+            s1->getInputs()[i]->dataRand(100 * trial + (int)i + 1);
+            s2->getInputs()[i]->setData(s1->getInputs()[i]->getDataPtr());
+        }
+        EXPECT(s1->compute());
+        CodeEngine ce;
+        auto exec = ce.instantiate(s2);
+        EXPECT(exec != nullptr);
+        EXPECT(exec->launch() && exec->sync());
+        EXPECT(s1->getOutputs().size() == 1 && s2->getOutputs().size() == 1);
+        Tensor *o1 = s1->getOutputs()[0], *o2 = s2->getOutputs()[0];
+        o2->deviceWritten();
+        if (!equalArrays(o1->getDataPtr(), o2->getDataPtr(), o1->size())) {
+            std::printf("  trial %d: %zu operators, %zu kernels, %zu folded, %zu aliased\n", trial,
+                        s2->getOperators().size(), exec->numKernelOps(), exec->numFoldedOps(),
+                        exec->numAliasedOps());
+            for (auto op : s2->getOperators())
+                std::printf("    %s\n", op->toString().c_str());
+            return false;
+        }
+        folded += exec->numFoldedOps();
+        aliased += exec->numAliasedOps();
+    }
+    std::printf("  24 graphs: %zu operators folded into neighbours, %zu without a kernel\n", folded,
+                aliased);
+    EXPECT(folded >= 10 && aliased >= 5); // the plans were exercised, not bypassed
+    return true;
+}
+
 // Writes the emitted program of the config-1 transformed graph to argv[2]; the
 // python test compiles and runs it.
 static std::string g_emit_path;
@@ -489,6 +581,7 @@ int main(int argc, char **argv) {
         {"dilated_space_to_batch_program", test_dilated_space_to_batch_program},
         {"code_engine_graph_runtime", test_code_engine_graph_runtime},
         {"conv3d_prepacked_graph", test_conv3d_prepacked_graph},
+        {"random_graphs_replay_equals_eager", test_random_graphs_replay_equals_eager},
         {"emit_program", test_emit_program},
         {"perf_engine_memo", test_perf_engine_memo},
         {"split_ratio_and_eltwise", test_split_ratio_and_eltwise},
