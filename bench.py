@@ -141,6 +141,13 @@ def main():
             ops.permute_flat(big_out, [2, 2, 1, 4096, 128, 128], [2, 3, 4, 0, 5, 1], out=big)
             ops.permute_flat(big, [1, 4096, 2, 128, 256], [0, 2, 1, 3, 4], out=big_out)
             ops.trans_chain(big, halo_chain, out=halo_out)
+        del big_out, halo_out
+        # odd rows: zero-pad 126x126 planes to 128x128 and crop them back
+        odd = big.reshape(-1)[:64 * 256 * 126 * 126].reshape(64, 256, 126, 126)
+        padded = torch.empty((64, 256, 128, 128), device=dev)
+        for _ in range(args.layout_only):
+            ops.pad(odd, [0, 0, 1, 1], [0, 0, 1, 1], out=padded)
+            ops.slice_(padded, [0, 0, 1, 1], [0, 0, 1, 1], out=odd)
         torch.cuda.synchronize()
         return
 
@@ -250,7 +257,19 @@ def main():
     ms = time_kernel(lambda: ops.trans_chain(big, halo_chain, out=halo_out), reps=10, warm=2)
     per_op.append({"op": "H2N with 1-row halo, same tensor", "ms": ms,
                    "GB/s": halo_bytes / ms / 1e6, "frac_hbm": halo_bytes / ms / 1e6 / HBM_PEAK_GBS})
-    del big, halo_out
+    del halo_out
+    # rows at odd dword alignment: zero-pad 126x126 planes to 128x128 and crop them back
+    odd = big.reshape(-1)[:64 * 256 * 126 * 126].reshape(64, 256, 126, 126)
+    padded = torch.empty((64, 256, 128, 128), device=dev)
+    odd_bytes = 4.0 * (odd.numel() + padded.numel())
+    ms = time_kernel(lambda: ops.pad(odd, [0, 0, 1, 1], [0, 0, 1, 1], out=padded), reps=10, warm=2)
+    per_op.append({"op": "pad 64x256x126x126 -> 64x256x128x128", "ms": ms,
+                   "GB/s": odd_bytes / ms / 1e6, "frac_hbm": odd_bytes / ms / 1e6 / HBM_PEAK_GBS})
+    ms = time_kernel(lambda: ops.slice_(padded, [0, 0, 1, 1], [0, 0, 1, 1], out=odd), reps=10,
+                     warm=2)
+    per_op.append({"op": "slice 64x256x128x128 -> 64x256x126x126", "ms": ms,
+                   "GB/s": odd_bytes / ms / 1e6, "frac_hbm": odd_bytes / ms / 1e6 / HBM_PEAK_GBS})
+    del big, odd, padded
 
     # ---- the other configurations: batch-1 latency of the original network and of
     # its PET-transformed program, each replayed as one HIP graph

@@ -137,17 +137,16 @@ __global__ __launch_bounds__(256) void view_direct_kernel(const float *__restric
 // split into the innermost dim and the rest so that neighbours along a row reuse
 // the outer part. 32-bit wrap-around arithmetic: both buffers hold fewer than
 // 2^31 elements, so the offset of every valid element is exact modulo 2^32.
-__device__ __forceinline__ void decode_outer(const DirectParams &p, unsigned e, unsigned &inner,
-                                             unsigned &io, bool &ok) {
+// Row index (all dims but the innermost, flattened) -> input offset of the row's
+// element 0 and whether the row lies inside every outer window.
+__device__ __forceinline__ void decode_row(const DirectParams &p, unsigned e, unsigned &io,
+                                           bool &ok) {
     io = (unsigned)p.ibase;
     const int L = p.rank - 1;
-    unsigned q = fd_div(e, p.ext[L]);
-    inner = e - q * p.ext[L].d;
-    e = q;
 #pragma unroll
     for (int d = PET_HIP_MAX_RANK - 2; d >= 0; --d) {
         if (d < L) {
-            q = fd_div(e, p.ext[d]);
+            unsigned q = fd_div(e, p.ext[d]);
             unsigned r = e - q * p.ext[d].d;
             e = q;
             if (p.has_div[d]) {
@@ -159,6 +158,14 @@ __device__ __forceinline__ void decode_outer(const DirectParams &p, unsigned e, 
             ok = ok && ((int)r >= p.lo[d]) && ((int)r < p.hi[d]);
         }
     }
+}
+
+__device__ __forceinline__ void decode_outer(const DirectParams &p, unsigned e, unsigned &inner,
+                                             unsigned &io, bool &ok) {
+    const int L = p.rank - 1;
+    unsigned q = fd_div(e, p.ext[L]);
+    inner = e - q * p.ext[L].d;
+    decode_row(p, q, io, ok);
 }
 
 __device__ __forceinline__ void eval_inner(const DirectParams &p, unsigned r, unsigned &io,
@@ -226,6 +233,102 @@ __global__ __launch_bounds__(256) void view_gather4_kernel(const float *__restri
         const unsigned t = base + u * 256u;
         if (t < p.total)
             st4<NT>(y + p.obase + 4ll * t, (vf4){v[u][0], v[u][1], v[u][2], v[u][3]});
+    }
+}
+
+// Dense, 16-byte aligned output whose rows are contiguous pieces of the input at
+// any dword alignment (a cropped or zero-padded innermost dim, an odd row length):
+// a workgroup produces ROWSTAGE_TILE consecutive output elements in LDS and
+// stores them as aligned 16-byte words. The rows that meet the tile are fetched
+// as the ALIGNED 16-byte input words that cover them, one word per work item,
+// and scattered element-wise into the LDS tile at their output position, so
+// that both global sides move whole aligned words however the two row lengths
+// relate. An aligned word that holds one valid element lies inside that
+// element's page, so the up to three neighbours it brings along are always
+// readable; they are dropped. Elements outside the windows keep the zeros the
+// tile is cleared to (only views that have such elements clear it).
+constexpr unsigned ROWSTAGE_TILE = 4096;
+struct RowStageParams {
+    FastDiv cpr;        // upper bound of the aligned input words one row needs inside a tile
+    int zero;           // some window is narrower than its dim
+    unsigned total;     // output elements
+};
+
+template <bool NT>
+__global__ __launch_bounds__(256) void view_rowstage_kernel(const float *__restrict__ x,
+                                                            float *__restrict__ y,
+                                                            DirectParams p, RowStageParams rs) {
+    constexpr unsigned T = ROWSTAGE_TILE;
+    constexpr int UN = 4;
+    __shared__ __attribute__((aligned(16))) float tile[T];
+    const unsigned tid = threadIdx.x;
+    const unsigned E0 = blockIdx.x * T;
+    const unsigned E1 = min(E0 + T, rs.total);
+    const int L = p.rank - 1;
+    const unsigned ext_inner = p.ext[L].d;
+    const int lo = p.lo[L], hi = p.hi[L];
+    const unsigned r0 = fd_div(E0, p.ext[L]);
+    const unsigned r1 = fd_div(E1 - 1u, p.ext[L]);
+    const unsigned items = (r1 - r0 + 1u) * rs.cpr.d;
+    if (rs.zero) {
+#pragma unroll
+        for (unsigned u = 0; u < T / 1024u; ++u)
+            *reinterpret_cast<vf4 *>(&tile[(u * 256u + tid) * 4u]) = (vf4){0.f, 0.f, 0.f, 0.f};
+        __syncthreads();
+    }
+    for (unsigned it0 = 0; it0 < items; it0 += 256u * UN) {
+        vf4 w[UN];
+        int first[UN], a[UN], b[UN], rel[UN];
+#pragma unroll
+        for (int u = 0; u < UN; ++u) {
+            const unsigned it = it0 + u * 256u + tid;
+            a[u] = 0;
+            b[u] = 0;
+            first[u] = 0;
+            rel[u] = 0;
+            w[u] = (vf4){0.f, 0.f, 0.f, 0.f};
+            if (it < items) {
+                const unsigned rl = fd_div(it, rs.cpr);
+                const unsigned ch = it - rl * rs.cpr.d;
+                const unsigned row = r0 + rl;
+                unsigned io_row;
+                bool ok = true;
+                decode_row(p, row, io_row, ok);
+                const unsigned row_start = row * ext_inner;
+                // the part of this row inside the tile and the window, as inner indices
+                const int aa = max((int)(E0 > row_start ? E0 - row_start : 0u), lo);
+                const int bb = min((int)(min(E1, row_start + ext_inner) - row_start), hi);
+                if (ok && aa < bb) {
+                    const unsigned g = io_row + (unsigned)aa; // input offset of inner index aa
+                    const unsigned mis = g & 3u;
+                    const int ii = aa - (int)mis + 4 * (int)ch;
+                    if (ii < bb) {
+                        w[u] = ld4<NT>(x + ((g - mis) + 4u * ch));
+                        a[u] = aa;
+                        b[u] = bb;
+                        first[u] = ii;
+                        rel[u] = (int)(row_start - E0); // wraps to the negative offset of a row that began before the tile
+                    }
+                }
+            }
+        }
+#pragma unroll
+        for (int u = 0; u < UN; ++u) {
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const int i = first[u] + j;
+                if (i >= a[u] && i < b[u])
+                    tile[rel[u] + i] = w[u][j];
+            }
+        }
+    }
+    __syncthreads();
+#pragma unroll
+    for (unsigned u = 0; u < T / 1024u; ++u) {
+        const unsigned idx = (u * 256u + tid) * 4u;
+        if (E0 + idx < E1)
+            st4<NT>(y + p.obase + (long long)(E0 + idx),
+                    *reinterpret_cast<const vf4 *>(&tile[idx]));
     }
 }
 
@@ -992,6 +1095,25 @@ int launch_view_copy(const float *x, float *y, ViewDesc v, long long in_elems,
             p.inner_contig = c.d[L].sr == 1 && c.d[L].m >= c.d[L].ext;
             p.total = (unsigned)(total / 4);
             const bool nt = stream_sized(total);
+            if (p.inner_contig && c.d[L].ext >= 16 && (uintptr_t)x % 16 == 0) {
+                RowStageParams rs;
+                const long long words =
+                    std::min<long long>((c.d[L].ext + 3) / 4 + 1, ROWSTAGE_TILE / 4 + 1);
+                rs.cpr = make_fastdiv((unsigned)words);
+                rs.zero = 0;
+                for (int i = 0; i < c.rank; ++i)
+                    if (c.d[i].lo > 0 || c.d[i].hi < std::min(c.d[i].ext, c.d[i].m))
+                        rs.zero = 1;
+                rs.total = (unsigned)total;
+                const dim3 rgrid((unsigned)((total + ROWSTAGE_TILE - 1) / ROWSTAGE_TILE));
+                if (nt)
+                    hipLaunchKernelGGL(view_rowstage_kernel<true>, rgrid, dim3(256), 0, stream, x,
+                                       y, p, rs);
+                else
+                    hipLaunchKernelGGL(view_rowstage_kernel<false>, rgrid, dim3(256), 0, stream,
+                                       x, y, p, rs);
+                return check_launch("view_rowstage_kernel");
+            }
             const dim3 grid((unsigned)((p.total + 1023) / 1024)), block(256);
             if (nt)
                 hipLaunchKernelGGL(view_gather4_kernel<true>, grid, block, 0, stream, x, y, p);

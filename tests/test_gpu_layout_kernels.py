@@ -136,6 +136,55 @@ def test_pad_then_slice_back(ops, shape, begin, end):
     assert host(back).tobytes() == x.tobytes()
 
 
+@pytest.mark.parametrize("shape,begin,end", [
+    ((8, 16, 30), (0, 0, 1), (0, 0, 1)),                 # rows of 30 -> 32: one row per 8 words
+    ((8, 16, 33), (0, 0, 0), (0, 0, -1)),                # crop the last column: rows of 32 from 33
+    ((4, 7, 9, 19), (0, 1, 2, -1), (1, 0, -1, -2)),      # pad and crop mixed, odd rows of 16
+    ((3, 4100), (0, 2), (1, 2)),                         # rows longer than a staging tile
+    ((2, 9001), (0, -1), (0, 0)),                        # ... and odd, cropped in front
+    ((5, 3, 126, 126), (0, 0, 1, 1), (0, 0, 1, 1)),
+    ((5, 3, 128, 128), (0, 0, -1, -1), (0, 0, -1, -1)),
+    ((2, 2, 64, 130), (1, 0, 0, -3), (0, 1, 0, -3)),     # whole zero planes around cropped rows
+    ((33, 257, 129), (0, 0, -1), (0, 0, 0)),             # > 1 Mi outputs
+])
+def test_row_staged_windows(ops, shape, begin, end):
+    """Dense output whose rows are pieces of input rows at any dword alignment: the
+    LDS-staged kernel (aligned 16-byte words on both global sides). Negative
+    amounts crop. Also through an input that starts 4 bytes into its buffer,
+    which must take the element-wise kernel and give the same bytes."""
+    x = iota(shape)
+    ref = x
+    for d, (b, e) in enumerate(zip(begin, end)):
+        idx = [slice(None)] * ref.ndim
+        idx[d] = slice(max(0, -b), ref.shape[d] - max(0, -e))
+        ref = ref[tuple(idx)]
+        widths = [(0, 0)] * ref.ndim
+        widths[d] = (max(0, b), max(0, e))
+        ref = np.pad(ref, widths)
+    ref = np.ascontiguousarray(ref)
+
+    def run(xd):
+        cb, ce = [max(0, -b) for b in begin], [max(0, -e) for e in end]
+        pb, pe = [max(0, b) for b in begin], [max(0, e) for e in end]
+        t = ops.slice_(xd, cb, ce) if any(cb) or any(ce) else xd
+        return ops.pad(t, pb, pe) if any(pb) or any(pe) else t
+
+    assert host(run(dev(x))).tobytes() == ref.tobytes()
+    shifted = torch.empty(x.size + 1, dtype=torch.float32, device="cuda")
+    shifted[1:] = dev(x).reshape(-1)
+    assert host(run(shifted[1:].reshape(shape))).tobytes() == ref.tobytes()
+
+
+def test_row_staged_streaming_variant(ops):
+    x = iota((64, 64, 126, 126))                         # 65 Mi elements: non-temporal variant
+    p = ops.pad(dev(x), [0, 0, 1, 1], [0, 0, 1, 1])
+    back = ops.slice_(p, [0, 0, 1, 1], [0, 0, 1, 1])
+    assert host(back).tobytes() == x.tobytes()
+    ph = host(p)
+    assert not ph[:, :, 0, :].any() and not ph[:, :, :, 127].any()
+    assert ph[:, :, 1:127, 1:127].tobytes() == x.tobytes()
+
+
 @pytest.mark.parametrize("shape,dim,num", [((2, 6, 7, 7), 1, 2), ((4, 8, 16), 0, 1), ((3, 5, 12), 2, 3)])
 def test_extend(ops, shape, dim, num):
     x = iota(shape)
