@@ -930,16 +930,21 @@ int launch_plane_cfg(ConvParams p, hipStream_t stream) {
     // Stream-K instead: 256 (64x128 tiles) or 512 workgroups share the tiles * nit K
     // steps evenly, so no CU waits for a last, partly filled round of tiles. All
     // sums go into y as float atomics (initialising launch before, activation after).
-    // Taken when the model sees a tenth less work on the busiest CU.
+    // Taken when the model sees 5 % less work on the busiest CU (its workgroups also sit two
+    // to a CU where a short grid of tiles leaves one: measured, a margin of 10 % left the
+    // 128->128 and 256->256 3x3x3 layers of R3D-18 on split K, 18 % and 9 % slower; at
+    // no margin the 512->512 layers of the dilated block turn 3 % slower).
     p.streamk = 0;
     {
         static const int sk_env = getenv("PET_HIP_STREAMK") ? atoi(getenv("PET_HIP_STREAMK")) : -1;
         const long long units = tiles * nit;
         const int wgs = Cfg::BM * Cfg::BN >= 64 * 128 ? 256 : 512;
         const double cost_sk = (double)units / 256 + 2 * c_fixed + c_launches;
+        static const double sk_margin =
+            getenv("PET_HIP_STREAMK_MARGIN") ? atof(getenv("PET_HIP_STREAMK_MARGIN")) : 0.95;
         const bool fits = p.G == 1 && units * (wgs + 1) < (1ll << 31) && units >= 2 * wgs &&
                           has_streamk<Cfg> && !deterministic();
-        if (fits && forced <= 0 && (sk_env == 1 || (sk_env != 0 && cost_sk < 0.9 * best))) {
+        if (fits && forced <= 0 && (sk_env == 1 || (sk_env != 0 && cost_sk < sk_margin * best))) {
             p.streamk = 1;
             splitk = 1;
             p.sk_units = (int)units;
@@ -1027,13 +1032,10 @@ int launch_plane(const ConvParams &p, bool is3d, hipStream_t stream) {
     // barrier waits), measured equal or better than one 64x128 workgroup per CU up to
     // a few rounds of tiles; beyond that 64x128 wins through its lower LDS traffic per
     // MFMA (2048 tiles of 64x128 with 8 steps: 212 vs 230 us). 32x64 for M <= 32.
-    // The 3-D kernel carries more registers and is the exception: it keeps 64x128 once
-    // those tiles fill the chip and the K loop is long (R3D-18 layer 1: 152 vs 165 us).
+    // The 3-D kernel stays with 64x64: with kt-major filters R3D-18 layer 1 takes 117 us
+    // against 121 us with 64x128 tiles.
     int tile = p.M > 32 ? 1 : 2;
-    const int nit = (p.cpg / CB) * p.KT;
     if (p.M > 32 && !is3d && tiles_for(p.M, p.NPIX, 64, 64, p.G) > 2048)
-        tile = 0;
-    if (p.M > 32 && is3d && tiles_for(p.M, p.NPIX, 64, 128, p.G) >= 200 && nit > 16)
         tile = 0;
     if (forced_tile() >= 0)
         tile = forced_tile() % 3;
