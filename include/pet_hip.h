@@ -49,7 +49,9 @@ typedef enum pet_hip_act {
 typedef enum pet_hip_eltwise_op {
     PET_HIP_ADD = 0, /* AddOp::compute, src/Graph/operator.cc:2983-3002 */
     PET_HIP_SUB = 1, /* SubOp::compute, src/Graph/operator.cc:3074-3090 */
-    PET_HIP_MUL = 2  /* MulOp::compute, src/Graph/operator.cc:3157-3176 */
+    PET_HIP_MUL = 2, /* MulOp::compute, src/Graph/operator.cc:3157-3176 */
+    PET_HIP_DIV = 3  /* DivOp, shape rule src/Graph/operator.cc:3306-3313; a / b (the
+                        reference's CPU body at :3259 subtracts) */
 } pet_hip_eltwise_op;
 
 /* Opaque handles (a hipStream_t / hipEvent_t / hipGraphExec_t underneath). */
@@ -240,12 +242,25 @@ PET_HIP_API int pet_hip_extend(const float *x, float *y, const int *in_dims, int
 
 /* ---- element-wise ---------------------------------------------------------*/
 
-/* k-ary Add / Mul, binary Sub with flat-modulo broadcast in[i % sizes[j]]
+/* k-ary Add / Mul, binary Sub / Div with flat-modulo broadcast in[i % sizes[j]]
  * (src/Graph/operator.cc:2983-3002, 3074-3090, 3157-3176); replaces
  * cublasSaxpy / cudnnOpTensor (src/Graph/code_engine.cc:1335-1348, 1377-1422).
  * k <= 8. y may alias ins[j] only when sizes[j] == n. */
 PET_HIP_API int pet_hip_eltwise(int op, const float *const *ins, const size_t *sizes, int k, float *y,
                     size_t n, pet_hip_stream_t stream);
+
+/* PowOp::compute, src/Graph/operator.cc:3330-3343 with powVType
+ * (include/common.h:157-162): y = 1 * x * x ... (`pow` factors, each product rounded
+ * to fp32; pow <= 0 gives 1). pow <= 1024. x == y is allowed. */
+PET_HIP_API int pet_hip_pow(const float *x, float *y, size_t n, int pow, pet_hip_stream_t stream);
+
+/* BatchNormOp::compute, src/Graph/operator.cc:2660-2681, on an [outer, ch, inner]
+ * view (channel = dim 1 of the tensor): y = (x - mean[ch]) * scale[ch] /
+ * sqrt(var[ch] + eps) + bias[ch]. The reference emits nothing for it on the GPU
+ * (src/Graph/code_engine.cc:1848-1850). x == y is allowed. */
+PET_HIP_API int pet_hip_batchnorm(const float *x, const float *scale, const float *bias,
+                      const float *mean, const float *var, float *y, size_t outer, size_t ch,
+                      size_t inner, float eps, pet_hip_stream_t stream);
 
 /* y = act(x); replaces cudnnActivationForward (src/Graph/code_engine.cc:1260-1274).
  * The reference has no CPU compute for it (include/operator.h:1968-1977). */

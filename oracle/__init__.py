@@ -290,6 +290,37 @@ def eltwise(op, xs, out_shape):
     return None if rc else y
 
 
+def pow_(x, power):
+    """PowOp::compute (operator.cc:3330-3343): `power` copies multiplied up from 1."""
+    x = _c(x)
+    t = _tier(x)
+    y = np.empty_like(x)
+    getattr(lib(), "oracle_pow_" + t)(_p(x), _p(y), ctypes.c_size_t(x.size), int(power))
+    return y
+
+
+def div(a, b, out_shape):
+    a = _c(a.astype(np.float32, copy=False))
+    b = _c(b.astype(np.float32, copy=False))
+    y = np.empty(out_shape, dtype=np.float32)
+    lib().oracle_div_f32(_p(a), ctypes.c_size_t(a.size), _p(b), ctypes.c_size_t(b.size),
+                         _p(y), ctypes.c_size_t(y.size))
+    return y
+
+
+def batchnorm(x, scale, bias, mean, var, eps=1e-5):
+    """BatchNormOp::compute (operator.cc:2660-2681); channel axis 1."""
+    x = _c(x.astype(np.float32, copy=False))
+    ch = x.shape[1]
+    inner = int(np.prod(x.shape[2:], dtype=np.int64))
+    y = np.empty_like(x)
+    vs = [_c(v.astype(np.float32, copy=False)) for v in (scale, bias, mean, var)]
+    lib().oracle_batchnorm_f32(_p(x), _p(vs[0]), _p(vs[1]), _p(vs[2]), _p(vs[3]), _p(y),
+                               ctypes.c_size_t(x.shape[0]), ctypes.c_size_t(ch),
+                               ctypes.c_size_t(inner), ctypes.c_float(eps))
+    return y
+
+
 SPLIT, REORDER, FUSE = 0, 1, 2
 
 

@@ -25,6 +25,13 @@
  *   split_one, concat_one, pad, slice, extend : numpy split / concatenate / pad /
  *       slicing / tile.
  *   eltwise : numpy with explicit flat-modulo broadcast on hand-built cases.
+ *   pow : Python integers modulo 2^32 (u32 tier) and numpy integer powers of small
+ *       integers, exact in fp32 (f32 tier); pow 0 and 1 by definition.
+ *   div : numpy true division. The reference's DivOp::compute body subtracts
+ *       (src/Graph/operator.cc:3259) and nothing upstream runs Div on a GPU, so
+ *       division itself is parity unpinned by the reference.
+ *   batchnorm : torch.nn.functional.batch_norm (CPU, inference mode) and the
+ *       identity statistics (mean 0, var 1 - eps, scale 1, bias 0 -> y = x).
  *   trans_chain : numpy constructions of halo split / drop fuse / pad fuse /
  *       extr split on iota inputs, and conv equivalence (split+conv+fuse == conv).
  *   relu/sigmoid/tanh/gelu, bias_act, maxpool, avgpool, softmax, layernorm :
@@ -120,6 +127,31 @@ PET_ORACLE_EXPORT void oracle_activation_f32(const float *x, float *y, size_t n,
 #pragma omp parallel for
     for (size_t i = 0; i < n; ++i)
         y[i] = act_apply(act, x[i]);
+}
+
+/* DivOp with the flat-modulo broadcast of the other binary operators
+ * (shape rule src/Graph/operator.cc:3306-3313). The reference's compute body
+ * at :3259 subtracts; this is division. */
+PET_ORACLE_EXPORT void oracle_div_f32(const float *a, size_t na, const float *b, size_t nb,
+                                      float *y, size_t n) {
+#pragma omp parallel for
+    for (size_t i = 0; i < n; ++i)
+        y[i] = a[i % na] / b[i % nb];
+}
+
+/* BatchNormOp::compute, src/Graph/operator.cc:2660-2681: channel = dim 1,
+ * factor[c] = scale[c] / sqrt(var[c] + eps) in double, y = (x - mean[c]) *
+ * factor[c] + bias[c]. */
+PET_ORACLE_EXPORT void oracle_batchnorm_f32(const float *x, const float *scale,
+                                            const float *bias, const float *mean,
+                                            const float *var, float *y, size_t outer,
+                                            size_t ch, size_t inner, float eps) {
+#pragma omp parallel for
+    for (size_t i = 0; i < outer * ch * inner; ++i) {
+        size_t c = (i / inner) % ch;
+        double factor = (double)scale[c] / sqrt((double)var[c] + (double)eps);
+        y[i] = (float)(((double)x[i] - (double)mean[c]) * factor + (double)bias[c]);
+    }
 }
 
 /* y[o, ch, inner] = act(x + bias[ch]): the epilogue the GPU path fuses

@@ -11,7 +11,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "lib", "libpet_hip.so")
 
 ACT = {"none": 0, "relu": 1, "sigmoid": 2, "tanh": 3, "gelu": 4, None: 0}
-ELT = {"add": 0, "sub": 1, "mul": 2}
+ELT = {"add": 0, "sub": 1, "mul": 2, "div": 3}
 
 _c_int_p = ctypes.POINTER(ctypes.c_int)
 _vp = ctypes.c_void_p
@@ -61,6 +61,8 @@ SIGNATURES = {
     "pet_hip_extend": [_vp, _vp, _c_int_p, _i, _i, _i, _vp],
     "pet_hip_eltwise": [_i, ctypes.POINTER(_vp), ctypes.POINTER(_sz), _i, _vp, _sz, _vp],
     "pet_hip_activation": [_vp, _vp, _sz, _i, _vp],
+    "pet_hip_pow": [_vp, _vp, _sz, _i, _vp],
+    "pet_hip_batchnorm": [_vp] * 6 + [_sz, _sz, _sz, ctypes.c_float, _vp],
     "pet_hip_bias_act": [_vp, _vp, _vp, _sz, _sz, _sz, _i, _vp],
     "pet_hip_pool2d": [_vp, _vp] + [_i] * 13 + [_vp],
     "pet_hip_softmax": [_vp, _vp, _sz, _sz, _vp],

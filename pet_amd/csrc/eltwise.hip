@@ -60,8 +60,10 @@ __global__ __launch_bounds__(256) void eltwise_kernel(EltParams p, float *__rest
                         acc[v] += val[v];
                     else if (p.op == PET_HIP_MUL)
                         acc[v] *= val[v];
-                    else
+                    else if (p.op == PET_HIP_SUB)
                         acc[v] = j == 0 ? val[v] : acc[v] - val[v];
+                    else
+                        acc[v] = j == 0 ? val[v] : acc[v] / val[v];
                 }
             }
         }
@@ -89,6 +91,72 @@ __global__ __launch_bounds__(256) void activation_kernel(const float *__restrict
             *reinterpret_cast<float4 *>(y + i) = v;
         } else {
             y[i] = apply_act(x[i], act);
+        }
+    }
+}
+
+// y = x multiplied up `pow` times from 1, every product rounded to fp32 (the order
+// of PowOp's CPU loop, so small integers and exact products agree bit for bit).
+template <int VEC>
+__global__ __launch_bounds__(256) void pow_kernel(const float *__restrict__ x,
+                                                  float *__restrict__ y, size_t n, int pow) {
+    size_t i = ((size_t)blockIdx.x * 256 + threadIdx.x) * VEC;
+    const size_t step = (size_t)gridDim.x * 256 * VEC;
+    for (; i < n; i += step) {
+        float v[VEC], r[VEC];
+        if (VEC == 4) {
+            float4 t = *reinterpret_cast<const float4 *>(x + i);
+            v[0] = t.x;
+            v[1 % VEC] = t.y;
+            v[2 % VEC] = t.z;
+            v[3 % VEC] = t.w;
+        } else {
+            v[0] = x[i];
+        }
+#pragma unroll
+        for (int e = 0; e < VEC; ++e)
+            r[e] = 1.f;
+        for (int j = 0; j < pow; ++j)
+#pragma unroll
+            for (int e = 0; e < VEC; ++e)
+                r[e] *= v[e];
+        if (VEC == 4)
+            *reinterpret_cast<float4 *>(y + i) = make_float4(r[0], r[1 % VEC], r[2 % VEC],
+                                                             r[3 % VEC]);
+        else
+            y[i] = r[0];
+    }
+}
+
+// Inference batch normalisation over [outer, ch, inner]: one (outer, ch) row of
+// `inner` elements per workgroup pass, so the channel's factor and shift are
+// computed once per row and the row moves as 16-byte words when it can.
+__global__ __launch_bounds__(256) void batchnorm_kernel(const float *__restrict__ x,
+                                                        const float *__restrict__ scale,
+                                                        const float *__restrict__ bias,
+                                                        const float *__restrict__ mean,
+                                                        const float *__restrict__ var,
+                                                        float *__restrict__ y, size_t rows,
+                                                        unsigned ch, size_t inner, float eps,
+                                                        int vec) {
+    for (size_t row = blockIdx.x; row < rows; row += gridDim.x) {
+        const unsigned c = (unsigned)(row % ch);
+        const float factor = scale[c] / sqrtf(var[c] + eps);
+        const float shift = bias[c] - mean[c] * factor;
+        const float *xr = x + row * inner;
+        float *yr = y + row * inner;
+        if (vec) {
+            for (size_t i = threadIdx.x * 4; i < inner; i += 1024) {
+                float4 v = *reinterpret_cast<const float4 *>(xr + i);
+                v.x = v.x * factor + shift;
+                v.y = v.y * factor + shift;
+                v.z = v.z * factor + shift;
+                v.w = v.w * factor + shift;
+                *reinterpret_cast<float4 *>(yr + i) = v;
+            }
+        } else {
+            for (size_t i = threadIdx.x; i < inner; i += 256)
+                yr[i] = xr[i] * factor + shift;
         }
     }
 }
@@ -310,12 +378,12 @@ extern "C" {
 int pet_hip_eltwise(int op, const float *const *ins, const size_t *sizes, int k, float *y,
                     size_t n, pet_hip_stream_t stream) {
     PET_REQUIRE_INIT();
-    if (op != PET_HIP_ADD && op != PET_HIP_SUB && op != PET_HIP_MUL)
+    if (op != PET_HIP_ADD && op != PET_HIP_SUB && op != PET_HIP_MUL && op != PET_HIP_DIV)
         return set_error(PET_HIP_ERR_INVALID, "unknown element-wise op %d", op);
     if (k < 1 || k > kMaxEltIn || !ins || !sizes)
         return set_error(PET_HIP_ERR_INVALID, "element-wise ops take 1..%d inputs", kMaxEltIn);
-    if (op == PET_HIP_SUB && k != 2)
-        return set_error(PET_HIP_ERR_INVALID, "Sub is binary");
+    if ((op == PET_HIP_SUB || op == PET_HIP_DIV) && k != 2)
+        return set_error(PET_HIP_ERR_INVALID, "Sub and Div are binary");
     if (n == 0)
         return PET_HIP_OK;
     if (!y)
@@ -327,7 +395,10 @@ int pet_hip_eltwise(int op, const float *const *ins, const size_t *sizes, int k,
     p.k = k;
     p.op = op;
     p.n = n;
-    bool vec = (n % 4 == 0) && aligned16(y);
+    // Div takes one element per thread: in the four-wide instance the compiler's
+    // expansion of the division delivered elements 0 and 1 of every word into slots 2
+    // and 3 and zeros into 0 and 1 (measured on gfx950 with ROCm 7.2).
+    bool vec = (n % 4 == 0) && aligned16(y) && op != PET_HIP_DIV;
     for (int j = 0; j < k; ++j) {
         if (!ins[j] || sizes[j] == 0)
             return set_error(PET_HIP_ERR_INVALID, "input %d is empty", j);
@@ -375,6 +446,41 @@ int pet_hip_activation(const float *x, float *y, size_t n, int act, pet_hip_stre
         hipLaunchKernelGGL(activation_kernel<1>, dim3(grid_for(n)), dim3(256), 0,
                            as_stream(stream), x, y, n, act);
     return check_launch("activation_kernel");
+}
+
+int pet_hip_pow(const float *x, float *y, size_t n, int pow, pet_hip_stream_t stream) {
+    PET_REQUIRE_INIT();
+    if (pow > 1024)
+        return set_error(PET_HIP_ERR_UNSUPPORTED, "power %d is beyond 1024", pow);
+    if (n == 0)
+        return PET_HIP_OK;
+    if (!x || !y)
+        return set_error(PET_HIP_ERR_INVALID, "null pointer");
+    if (n % 4 == 0 && aligned16(x) && aligned16(y))
+        hipLaunchKernelGGL(pow_kernel<4>, dim3(grid_for(n / 4)), dim3(256), 0, as_stream(stream), x,
+                           y, n, pow);
+    else
+        hipLaunchKernelGGL(pow_kernel<1>, dim3(grid_for(n)), dim3(256), 0, as_stream(stream), x, y,
+                           n, pow);
+    return check_launch("pow_kernel");
+}
+
+int pet_hip_batchnorm(const float *x, const float *scale, const float *bias, const float *mean,
+                      const float *var, float *y, size_t outer, size_t ch, size_t inner, float eps,
+                      pet_hip_stream_t stream) {
+    PET_REQUIRE_INIT();
+    const size_t rows = outer * ch;
+    if (rows == 0 || inner == 0)
+        return PET_HIP_OK;
+    if (!x || !y || !scale || !bias || !mean || !var)
+        return set_error(PET_HIP_ERR_INVALID, "null pointer");
+    if (ch >= (1ull << 31))
+        return set_error(PET_HIP_ERR_UNSUPPORTED, "too many channels");
+    const int vec = inner % 4 == 0 && aligned16(x) && aligned16(y);
+    const unsigned grid = (unsigned)std::min<size_t>(rows, 65536);
+    hipLaunchKernelGGL(batchnorm_kernel, dim3(grid), dim3(256), 0, as_stream(stream), x, scale,
+                       bias, mean, var, y, rows, (unsigned)ch, inner, eps, vec);
+    return check_launch("batchnorm_kernel");
 }
 
 int pet_hip_bias_act(const float *x, const float *bias, float *y, size_t outer, size_t ch,

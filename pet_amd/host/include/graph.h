@@ -84,6 +84,14 @@ class Graph : public GraphBase {
     Operator *sub(Tensor *a, Tensor *b, Tensor *output);
     Operator *mul(const TensorVec &inputs, Tensor *output);
     Operator *mul(const TensorVec &inputs);
+    Operator *div(Tensor *input0, Tensor *input1, Tensor *output);
+    Operator *div(Tensor *input0, Tensor *input1);
+    Operator *pow(Tensor *input, Tensor *output, int pow);
+    Operator *pow(Tensor *input, int pow);
+    Operator *batchnorm(Tensor *input, Tensor *scale, Tensor *bias, Tensor *mean, Tensor *var,
+                        Tensor *output, float epsilon = 1e-05, float momentum = 0.9);
+    Operator *batchnorm(Tensor *input, Tensor *scale, Tensor *bias, Tensor *mean, Tensor *var,
+                        float epsilon = 1e-05, float momentum = 0.9);
     Operator *reshape(Tensor *input, Tensor *output);
     Operator *identity(Tensor *input, Tensor *output);
     Operator *relu(Tensor *input, Tensor *output);

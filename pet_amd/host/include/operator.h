@@ -603,7 +603,7 @@ class ExtendOp : public Operator {
     int dim, num;
 };
 
-// ---- element-wise: Add / Sub / Mul (flat-modulo broadcast) ------------------------
+// ---- element-wise: Add / Sub / Mul / Div (flat-modulo broadcast) ------------------
 class EltwiseOp : public Operator {
   public:
     EltwiseOp(OpType type, TensorVec inputs, Tensor *output);
@@ -613,7 +613,7 @@ class EltwiseOp : public Operator {
     double perf(PerfEngine *pe, int rounds = 200, int warmupRounds = 200) override;
     int launch(pet_hip_stream_t stream) override;
     std::string toString() const override;
-    int numInputs() override { return type == Sub ? 2 : (int)inputs.size(); }
+    int numInputs() override { return type == Sub || type == Div ? 2 : (int)inputs.size(); }
     int numOutputs() override { return 1; }
     // One output point -> the input points it depends on; the closure runs the
     // whole operator on the device.
@@ -647,6 +647,75 @@ class MulOp : public EltwiseOp {
     explicit MulOp(TensorVec inputs) : EltwiseOp(Mul, std::move(inputs), nullptr) {}
     MulOp() : EltwiseOp(Mul) {}
     MulOp *clone() override { return new MulOp(*this); }
+};
+
+// Division proper: the reference's CPU body subtracts (src/Graph/operator.cc:3259)
+// and it has no GPU emitter for Div.
+class DivOp : public EltwiseOp {
+  public:
+    DivOp(TensorVec inputs, Tensor *output) : EltwiseOp(Div, std::move(inputs), output) {}
+    explicit DivOp(TensorVec inputs) : EltwiseOp(Div, std::move(inputs), nullptr) {}
+    DivOp() : EltwiseOp(Div) {}
+    DivOp *clone() override { return new DivOp(*this); }
+};
+
+// x multiplied up `pow` times from 1 (src/Graph/operator.cc:3315-3343).
+class PowOp : public Operator {
+  public:
+    PowOp(Tensor *input, Tensor *output, int pow);
+    PowOp(Tensor *input, int pow);
+    explicit PowOp(int pow);
+    PowOp(const PowOp &rhs) : Operator(rhs), pow(rhs.pow) {}
+    PowOp *clone() override { return new PowOp(*this); }
+    Dim computeShape() override;
+    double perf(PerfEngine *pe, int rounds = 200, int warmupRounds = 200) override;
+    int launch(pet_hip_stream_t stream) override;
+    std::string toString() const override;
+    int numInputs() override { return 1; }
+    int numOutputs() override { return 1; }
+    int getPow() const { return pow; }
+    std::pair<std::vector<DimRange>, std::function<bool()>> compute(DimRange dr) override;
+    using Operator::compute;
+
+  private:
+    bool checkValid(const TensorVec &ins) override { return ins.size() == 1 && ins[0]; }
+    void initHash() override;
+    int pow;
+};
+
+// Inference batch normalisation, channel = dim 1 (src/Graph/operator.cc:2660-2715).
+// scale / bias / mean / var are side tensors of [channels], like a conv bias.
+class BatchNormOp : public Operator {
+  public:
+    BatchNormOp(Tensor *input, Tensor *scale, Tensor *bias, Tensor *mean, Tensor *var,
+                Tensor *output, float epsilon = 1e-05, float momentum = 0.9);
+    BatchNormOp(Tensor *input, Tensor *scale, Tensor *bias, Tensor *mean, Tensor *var,
+                float epsilon = 1e-05, float momentum = 0.9);
+    BatchNormOp(Tensor *scale, Tensor *bias, Tensor *mean, Tensor *var, float epsilon = 1e-05,
+                float momentum = 0.9);
+    BatchNormOp(const BatchNormOp &rhs)
+        : Operator(rhs), epsilon(rhs.epsilon), momentum(rhs.momentum), scale(rhs.scale),
+          bias(rhs.bias), mean(rhs.mean), var(rhs.var) {}
+    BatchNormOp *clone() override { return new BatchNormOp(*this); }
+    Dim computeShape() override;
+    double perf(PerfEngine *pe, int rounds = 200, int warmupRounds = 200) override;
+    int launch(pet_hip_stream_t stream) override;
+    std::string toString() const override;
+    int numInputs() override { return 1; }
+    int numOutputs() override { return 1; }
+    Tensor *getScale() const { return scale; }
+    Tensor *getBias() const { return bias; }
+    Tensor *getMean() const { return mean; }
+    Tensor *getVar() const { return var; }
+    float getEpsilon() const { return epsilon; }
+    std::pair<std::vector<DimRange>, std::function<bool()>> compute(DimRange dr) override;
+    using Operator::compute;
+
+  private:
+    bool checkValid(const TensorVec &ins) override;
+    void initHash() override;
+    float epsilon, momentum;
+    Tensor *scale, *bias, *mean, *var;
 };
 
 // ---- single-input ops without a reference CPU compute ----------------------------

@@ -278,6 +278,9 @@ std::unique_ptr<GraphExec> CodeEngine::instantiate(std::shared_ptr<SubGraph> &gr
             for (Tensor *t : {ln->getGamma(), ln->getBeta()})
                 if (t)
                     t->devicePtr();
+        if (auto bn = dynamic_cast<BatchNormOp *>(op))
+            for (Tensor *t : {bn->getScale(), bn->getBias(), bn->getMean(), bn->getVar()})
+                t->devicePtr();
     }
     AliasPlan plan = planAliases(order);
     TransposeChains rows = planTransposeChains(order, graph->getOutputs(), plan.skipped);
@@ -422,6 +425,9 @@ std::string CodeEngine::genCode(std::shared_ptr<SubGraph> &graph) {
             for (Tensor *t : {ln->getGamma(), ln->getBeta()})
                 if (t)
                     all.push_back(t);
+        if (auto bn = dynamic_cast<BatchNormOp *>(op))
+            for (Tensor *t : {bn->getScale(), bn->getBias(), bn->getMean(), bn->getVar()})
+                all.push_back(t);
     }
     std::set<const Tensor *> viewOf;
     std::set<const Operator *> skipped;
@@ -621,10 +627,27 @@ std::string CodeEngine::genCode(std::shared_ptr<SubGraph> &graph) {
             }
             e.line("    const float *eins" + id + "[] = " + ptrs + "}; static const size_t esz" + id +
                    "[] = " + sizes + "};");
-            int code = op->getType() == Operator::Add ? 0 : (op->getType() == Operator::Sub ? 1 : 2);
+            int code = op->getType() == Operator::Add   ? PET_HIP_ADD
+                       : op->getType() == Operator::Sub ? PET_HIP_SUB
+                       : op->getType() == Operator::Div ? PET_HIP_DIV
+                                                        : PET_HIP_MUL;
             c << "pet_hip_eltwise(" << code << ", eins" << id << ", esz" << id << ", "
               << op->getInputs().size() << ", " << out(0) << ", " << op->getOutputs()[0]->size()
               << ", s)";
+        } else if (auto pw = dynamic_cast<PowOp *>(op)) {
+            c << "pet_hip_pow(" << in(0) << ", " << out(0) << ", " << op->getInputs()[0]->size()
+              << ", " << pw->getPow() << ", s)";
+        } else if (auto bn = dynamic_cast<BatchNormOp *>(op)) {
+            const Dim &d = op->getInputs()[0]->getDims();
+            size_t inner = 1;
+            for (size_t i = 2; i < d.size(); ++i)
+                inner *= (size_t)d[i];
+            char eps[32];
+            snprintf(eps, sizeof eps, "%.9gf", bn->getEpsilon());
+            c << "pet_hip_batchnorm(" << in(0) << ", " << e.name(bn->getScale()) << ", "
+              << e.name(bn->getBias()) << ", " << e.name(bn->getMean()) << ", "
+              << e.name(bn->getVar()) << ", " << out(0) << ", " << d[0] << ", " << d[1] << ", "
+              << inner << ", " << eps << ", s)";
         } else if (auto act = dynamic_cast<ActivationOp *>(op)) {
             c << "pet_hip_activation(" << in(0) << ", " << out(0) << ", "
               << op->getInputs()[0]->size() << ", " << (int)act->getActType() << ", s)";

@@ -190,6 +190,22 @@ Operator *Graph::add(const TensorVec &ins) { return own(new AddOp(ins)); }
 Operator *Graph::sub(Tensor *a, Tensor *b, Tensor *output) { return own(new SubOp(a, b, output)); }
 Operator *Graph::mul(const TensorVec &ins, Tensor *output) { return own(new MulOp(ins, output)); }
 Operator *Graph::mul(const TensorVec &ins) { return own(new MulOp(ins)); }
+Operator *Graph::div(Tensor *a, Tensor *b, Tensor *output) {
+    return own(new DivOp({a, b}, output));
+}
+Operator *Graph::div(Tensor *a, Tensor *b) { return own(new DivOp({a, b})); }
+Operator *Graph::pow(Tensor *input, Tensor *output, int pow) {
+    return own(new PowOp(input, output, pow));
+}
+Operator *Graph::pow(Tensor *input, int pow) { return own(new PowOp(input, pow)); }
+Operator *Graph::batchnorm(Tensor *input, Tensor *scale, Tensor *bias, Tensor *mean, Tensor *var,
+                           Tensor *output, float epsilon, float momentum) {
+    return own(new BatchNormOp(input, scale, bias, mean, var, output, epsilon, momentum));
+}
+Operator *Graph::batchnorm(Tensor *input, Tensor *scale, Tensor *bias, Tensor *mean, Tensor *var,
+                           float epsilon, float momentum) {
+    return own(new BatchNormOp(input, scale, bias, mean, var, epsilon, momentum));
+}
 Operator *Graph::reshape(Tensor *input, Tensor *output) {
     return own(new ReshapeOp(input, output));
 }

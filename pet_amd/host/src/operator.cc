@@ -1220,7 +1220,7 @@ EltwiseOp::EltwiseOp(OpType type, TensorVec ins, Tensor *output)
 void EltwiseOp::initHash() { hash = hashPack(type); }
 
 bool EltwiseOp::checkValid(const TensorVec &ins) {
-    if (ins.empty() || ins.size() > 8 || (type == Sub && ins.size() != 2))
+    if (ins.empty() || ins.size() > 8 || ((type == Sub || type == Div) && ins.size() != 2))
         return false;
     for (auto t : ins)
         if (t == nullptr || t->size() == 0)
@@ -1257,7 +1257,10 @@ int EltwiseOp::launch(pet_hip_stream_t stream) {
         ptrs.push_back(t->devicePtr());
         sizes.push_back(t->size());
     }
-    int op = type == Add ? PET_HIP_ADD : (type == Sub ? PET_HIP_SUB : PET_HIP_MUL);
+    int op = type == Add   ? PET_HIP_ADD
+             : type == Sub ? PET_HIP_SUB
+             : type == Div ? PET_HIP_DIV
+                           : PET_HIP_MUL;
     return pet_hip_eltwise(op, ptrs.data(), sizes.data(), (int)ptrs.size(),
                            outputs[0]->devicePtr(), outputs[0]->size(), stream);
 }
@@ -1268,6 +1271,92 @@ double EltwiseOp::perf(PerfEngine *, int rounds, int warmupRounds) {
 
 std::string EltwiseOp::toString() const {
     return getOpName(type) + "(n=" + std::to_string(inputs.size()) + ")";
+}
+
+// ---- Pow / BatchNorm ------------------------------------------------------------------
+
+PowOp::PowOp(Tensor *input, Tensor *output, int pow) : Operator(Pow, {input}, {output}), pow(pow) {
+    assert(checkValid(inputs));
+    computeShape();
+    initHash();
+}
+PowOp::PowOp(Tensor *input, int pow) : PowOp(input, new Tensor(), pow) {}
+PowOp::PowOp(int pow) : Operator(Pow), pow(pow) { initHash(); }
+
+void PowOp::initHash() { hash = hashPack(hashAppend(type, pow)); }
+
+Dim PowOp::computeShape() {
+    outputs[0]->setDims(inputs[0]->getDims());
+    outputs[0]->setType(inputs[0]->getType());
+    return inputs[0]->getDims();
+}
+
+int PowOp::launch(pet_hip_stream_t stream) {
+    return pet_hip_pow(inputs[0]->devicePtr(), outputs[0]->devicePtr(), inputs[0]->size(), pow,
+                       stream);
+}
+
+double PowOp::perf(PerfEngine *, int rounds, int warmupRounds) {
+    return timeLaunches(std::min(rounds, 50), std::min(warmupRounds, 10));
+}
+
+std::string PowOp::toString() const { return "Pow(pow=" + std::to_string(pow) + ")"; }
+
+BatchNormOp::BatchNormOp(Tensor *input, Tensor *scale, Tensor *bias, Tensor *mean, Tensor *var,
+                         Tensor *output, float epsilon, float momentum)
+    : Operator(BatchNorm, {input}, {output}), epsilon(epsilon), momentum(momentum), scale(scale),
+      bias(bias), mean(mean), var(var) {
+    assert(checkValid(inputs));
+    computeShape();
+    initHash();
+}
+BatchNormOp::BatchNormOp(Tensor *input, Tensor *scale, Tensor *bias, Tensor *mean, Tensor *var,
+                         float epsilon, float momentum)
+    : BatchNormOp(input, scale, bias, mean, var, new Tensor(), epsilon, momentum) {}
+BatchNormOp::BatchNormOp(Tensor *scale, Tensor *bias, Tensor *mean, Tensor *var, float epsilon,
+                         float momentum)
+    : Operator(BatchNorm), epsilon(epsilon), momentum(momentum), scale(scale), bias(bias),
+      mean(mean), var(var) {
+    initHash();
+}
+
+void BatchNormOp::initHash() { hash = hashPack(type); }
+
+// every per-channel vector has as many elements as the input has channels
+bool BatchNormOp::checkValid(const TensorVec &ins) {
+    if (ins.size() != 1 || ins[0] == nullptr || ins[0]->getDims().size() < 2)
+        return false;
+    size_t c = (size_t)ins[0]->getDims()[1];
+    for (Tensor *t : {scale, bias, mean, var})
+        if (t == nullptr || t->size() != c)
+            return false;
+    return true;
+}
+
+Dim BatchNormOp::computeShape() {
+    outputs[0]->setDims(inputs[0]->getDims());
+    outputs[0]->setType(Tensor::Input);
+    return inputs[0]->getDims();
+}
+
+int BatchNormOp::launch(pet_hip_stream_t stream) {
+    const Dim &d = inputs[0]->getDims();
+    size_t inner = 1;
+    for (size_t i = 2; i < d.size(); ++i)
+        inner *= (size_t)d[i];
+    return pet_hip_batchnorm(inputs[0]->devicePtr(), scale->devicePtr(), bias->devicePtr(),
+                             mean->devicePtr(), var->devicePtr(), outputs[0]->devicePtr(),
+                             (size_t)d[0], (size_t)d[1], inner, epsilon, stream);
+}
+
+double BatchNormOp::perf(PerfEngine *, int rounds, int warmupRounds) {
+    return timeLaunches(std::min(rounds, 50), std::min(warmupRounds, 10));
+}
+
+std::string BatchNormOp::toString() const {
+    std::ostringstream os;
+    os << "BatchNorm(in=" << inputs[0]->getHash() << ",out=" << outputs[0]->getHash() << ")";
+    return os.str();
 }
 
 // ---- Activation / Pool / Softmax / LayerNorm / Reshape -----------------------------
@@ -1642,6 +1731,26 @@ PointDeps ExtendOp::compute(DimRange dr) {
         return {};
     src[dim] %= inputs[0]->getDims()[dim];
     return {{DimRange(src)}, [this]() { return compute() != nullptr; }};
+}
+
+// Pow and BatchNorm read the input at the output's own position
+// (src/Graph/operator.cc:3345-3357, 2683-2694).
+PointDeps PowOp::compute(DimRange dr) {
+    PointDeps ret;
+    if (symbolicRange(this, dr, inputs.size(), ret))
+        return ret;
+    if (!insideDims(dr.getBegin(), outputs[0]->getDims()))
+        return {};
+    return {{DimRange(dr.getBegin())}, [this]() { return compute() != nullptr; }};
+}
+
+PointDeps BatchNormOp::compute(DimRange dr) {
+    PointDeps ret;
+    if (symbolicRange(this, dr, inputs.size(), ret))
+        return ret;
+    if (!insideDims(dr.getBegin(), outputs[0]->getDims()))
+        return {};
+    return {{DimRange(dr.getBegin())}, [this]() { return compute() != nullptr; }};
 }
 
 PointDeps EltwiseOp::compute(DimRange dr) {

@@ -311,6 +311,31 @@ def activation(x, act, out=None):
     return out
 
 
+def pow_(x, power, out=None):
+    """PowOp (operator.cc:3330-3343): `power` copies of x multiplied up from 1."""
+    _chk(x, out)
+    if out is None:
+        out = torch.empty_like(x)
+    abi.call("pet_hip_pow", _ptr(x), _ptr(out), x.numel(), int(power), _stream())
+    return out
+
+
+def batchnorm(x, scale, bias, mean, var, eps=1e-5, out=None):
+    """BatchNormOp (operator.cc:2660-2681): inference statistics, channel axis 1."""
+    _chk(x, scale, bias, mean, var, out)
+    ch = x.shape[1]
+    if any(t.numel() != ch for t in (scale, bias, mean, var)):
+        raise abi.PetHipError(1, "per-channel vectors must have %d elements" % ch)
+    inner = 1
+    for d in x.shape[2:]:
+        inner *= d
+    if out is None:
+        out = torch.empty_like(x)
+    abi.call("pet_hip_batchnorm", _ptr(x), _ptr(scale), _ptr(bias), _ptr(mean), _ptr(var),
+             _ptr(out), x.shape[0], ch, inner, float(eps), _stream())
+    return out
+
+
 def bias_act(x, bias, act="none", ch_axis=1, out=None):
     _chk(x, bias, out)
     outer = 1

@@ -496,6 +496,72 @@ static bool test_split_ratio_and_eltwise() {
     return true;
 }
 
+// BatchNormOp / PowOp / DivOp (src/Graph/operator.cc:2660-2681, 3330-3343, 3246-3262;
+// Div divides here, see the class): operator by operator against the formulas on
+// the host, then the same graph through the graph runtime and the emitter.
+static bool test_batchnorm_pow_div() {
+    Graph g;
+    auto x = g.tensor({2, 6, 5, 7}), d = g.tensor({5, 7});
+    Tensor scale({6}, Tensor::Weight), bias({6}, Tensor::Weight), mean({6}, Tensor::Weight),
+        var({6}, Tensor::Weight);
+    auto bn = g.batchnorm(x, &scale, &bias, &mean, &var, 1e-3f);
+    auto pw = g.pow(bn->getOutputs()[0], 3);
+    auto dv = g.div(pw->getOutputs()[0], d);
+    EXPECT(dv->getOutputs()[0]->getDims() == (Dim{2, 6, 5, 7}));
+    g.updateConnection();
+    auto s1 = std::make_shared<SubGraph>(g.getOperators());
+    auto s2 = std::make_shared<SubGraph>(g.getOperators());
+    scale.dataRand(21);
+    bias.dataRand(22);
+    mean.dataRand(23);
+    var.dataRand(24);
+    for (size_t i = 0; i < s1->getInputs().size(); ++i) {
+        Tensor *t = s1->getInputs()[i];
+        t->dataRand((int)i + 31);
+        if (t->getDims().size() == 2) { // the divisor: keep away from zero
+            std::vector<float> v(t->getDataPtr(), t->getDataPtr() + t->size());
+            for (auto &e : v)
+                e += 1.f;
+            t->setData(v.data());
+        }
+        s2->getInputs()[i]->setData(t->getDataPtr());
+    }
+    EXPECT(s1->compute());
+    Tensor *xin = nullptr, *din = nullptr;
+    for (auto t : s1->getInputs())
+        (t->getDims().size() == 4 ? xin : din) = t;
+    EXPECT(xin && din);
+    Tensor *out = s1->getOutputs()[0];
+    const float *xp = xin->getDataPtr(), *dp = din->getDataPtr(), *op = out->getDataPtr();
+    for (size_t i = 0; i < out->size(); ++i) {
+        size_t c = (i / 35) % 6;
+        double f = (double)scale.getData(c) / std::sqrt((double)var.getData(c) + 1e-3);
+        double b = ((double)xp[i] - (double)mean.getData(c)) * f + (double)bias.getData(c);
+        double want = b * b * b / (double)dp[i % 35];
+        if (std::fabs((double)op[i] - want) > 1e-4 * std::max(1.0, std::fabs(want))) {
+            std::printf("  element %zu: %g, expected %g\n", i, (double)op[i], want);
+            return false;
+        }
+    }
+    CodeEngine ce;
+    auto exec = ce.instantiate(s2);
+    EXPECT(exec != nullptr);
+    for (int rep = 0; rep < 2; ++rep) {
+        EXPECT(exec->launch() && exec->sync());
+        Tensor *o2 = s2->getOutputs()[0];
+        o2->deviceWritten();
+        EXPECT(equalArrays(out->getDataPtr(), o2->getDataPtr(), out->size()));
+    }
+    std::string code = ce.genCode(s2);
+    EXPECT(code.find("pet_hip_batchnorm(") != std::string::npos);
+    EXPECT(code.find("pet_hip_pow(") != std::string::npos);
+    EXPECT(code.find("pet_hip_eltwise(3,") != std::string::npos);
+    // one output point depends on the same point of the input
+    auto deps = pw->compute(DimRange(Dim{1, 2, 3, 4}));
+    EXPECT(deps.first.size() == 1 && deps.first[0].getBegin() == (Dim{1, 2, 3, 4}));
+    return true;
+}
+
 // src/Mutant/generator.cc:1327-1381: two convolutions of one input become one
 // (weights concatenated on dim 0, result split on dim 1); :1159-1234: two
 // convolutions of different inputs and filter counts 8 and 12 become one
@@ -585,6 +651,7 @@ int main(int argc, char **argv) {
         {"emit_program", test_emit_program},
         {"perf_engine_memo", test_perf_engine_memo},
         {"split_ratio_and_eltwise", test_split_ratio_and_eltwise},
+        {"batchnorm_pow_div", test_batchnorm_pow_div},
         {"conv_merge_programs", test_conv_merge_programs},
     };
     std::string only = argc > 1 ? argv[1] : "";

@@ -653,6 +653,44 @@ def test_eltwise_bit_exact(ops):
     assert got.tobytes() == oracle.eltwise("add", [r0, r1], r0.shape).tobytes()
 
 
+def test_pow_div_batchnorm(ops):
+    """PowOp: bit-exact (the same chain of fp32 products as the CPU loop). Div:
+    division proper, correctly rounded like numpy's. BatchNorm: 1e-5 relative
+    (fp32 factor and shift against the oracle's double)."""
+    rng = np.random.default_rng(12)
+    for shape in [(2, 3, 8), (5, 7), (1, 64, 56, 56), (3,)]:
+        x = rng.standard_normal(shape).astype(np.float32)
+        xi = rng.integers(-7, 8, shape).astype(np.float32)
+        for p in (0, 1, 2, 3, 5):
+            assert host(ops.pow_(dev(x), p)).tobytes() == oracle.pow_(x, p).tobytes(), (shape, p)
+            assert host(ops.pow_(dev(xi), p)).tobytes() == oracle.pow_(xi, p).tobytes()
+    assert host(ops.pow_(dev(x), -1)).tobytes() == np.ones_like(x).tobytes()
+    with pytest.raises(Exception):
+        ops.pow_(dev(x), 5000)
+
+    a = rng.standard_normal((2, 6, 8)).astype(np.float32)
+    for b in [rng.uniform(0.5, 2.0, (8,)).astype(np.float32),
+              rng.uniform(0.5, 2.0, (6, 8)).astype(np.float32),
+              rng.uniform(-3.0, -1.0, (2, 6, 8)).astype(np.float32),
+              np.array([4.0], dtype=np.float32)]:
+        ref = oracle.div(a, b, a.shape)
+        got = host(ops.eltwise("div", [dev(a), dev(b)], a.shape))
+        np.testing.assert_array_max_ulp(got, ref, maxulp=1)
+    with pytest.raises(Exception):
+        ops.eltwise("div", [dev(a), dev(a), dev(a)], a.shape)
+
+    for shape in [(2, 5, 3, 4), (1, 64, 56, 56), (4, 7, 9), (3, 6), (1, 8, 2, 5, 5)]:
+        x = rng.standard_normal(shape).astype(np.float32)
+        ch = shape[1]
+        sc, bi, me = (rng.standard_normal(ch).astype(np.float32) for _ in range(3))
+        va = rng.uniform(0.25, 4.0, ch).astype(np.float32)
+        ref = oracle.batchnorm(x, sc, bi, me, va, 1e-3)
+        got = host(ops.batchnorm(dev(x), dev(sc), dev(bi), dev(me), dev(va), 1e-3))
+        np.testing.assert_allclose(got, ref, rtol=1e-5, atol=1e-5)
+    with pytest.raises(Exception):
+        ops.batchnorm(dev(x), dev(sc[:-1]), dev(bi), dev(me), dev(va))
+
+
 def test_activation_pool_softmax_layernorm(ops):
     rng = np.random.default_rng(10)
     x = rng.standard_normal((2, 3, 9, 9)).astype(np.float32)

@@ -292,6 +292,47 @@ def test_eltwise_flat_modulo_broadcast():
     np.testing.assert_array_equal(oracle.eltwise("add", [a, d], (2, 3, 4)), ref)
 
 
+def test_pow_div_batchnorm_pins():
+    """PowOp (operator.cc:3330-3343 + powVType, common.h:157-162): against Python
+    integers modulo 2^32 and exact small-integer powers. Div: numpy true division.
+    BatchNorm (operator.cc:2660-2681): torch's inference batch_norm and the identity
+    statistics."""
+    import torch
+    xu = np.array([0, 1, 2, 3, 7, 65536, 65537, 4294967295, 123456789], dtype=np.uint32)
+    for p in (0, 1, 2, 3, 5, 9):
+        want = np.array([pow(int(v), p, 1 << 32) for v in xu], dtype=np.uint32)
+        assert np.array_equal(oracle.pow_(xu, p), want), p
+    assert np.array_equal(oracle.pow_(xu, -2), np.ones_like(xu))     # the loop never runs
+    xf = np.arange(-9, 10, dtype=np.float32)
+    for p in (0, 1, 2, 3, 4, 6):
+        assert np.array_equal(oracle.pow_(xf, p), (xf.astype(np.int64) ** p).astype(np.float32))
+    # a dropped factor or an off-by-one in the loop count would show here
+    assert oracle.pow_(np.array([1.5], dtype=np.float32), 3)[0] == np.float32(3.375)
+
+    rng = np.random.default_rng(3)
+    a = rng.standard_normal((2, 3, 4)).astype(np.float32)
+    b = np.array([2.0, -4.0, 0.5, 8.0], dtype=np.float32)
+    assert np.array_equal(oracle.div(a, b, a.shape), a / b)          # trailing-dim broadcast
+    assert np.array_equal(oracle.div(b, a, a.shape), b / a)
+
+    x = rng.standard_normal((2, 5, 3, 4)).astype(np.float32)
+    sc, bi, me = (rng.standard_normal(5).astype(np.float32) for _ in range(3))
+    va = rng.uniform(0.25, 4.0, 5).astype(np.float32)
+    want = torch.nn.functional.batch_norm(
+        torch.from_numpy(x), torch.from_numpy(me), torch.from_numpy(va), torch.from_numpy(sc),
+        torch.from_numpy(bi), False, 0.1, 1e-3).numpy()
+    np.testing.assert_allclose(oracle.batchnorm(x, sc, bi, me, va, 1e-3), want, rtol=1e-5,
+                               atol=1e-6)
+    ident = oracle.batchnorm(x, np.ones(5, np.float32), np.zeros(5, np.float32),
+                             np.zeros(5, np.float32), np.ones(5, np.float32), 0.0)
+    assert np.array_equal(ident, x)
+    # channel axis is 1: a per-channel shift moves whole [h, w] planes
+    shifted = oracle.batchnorm(x, np.ones(5, np.float32), np.arange(5, dtype=np.float32),
+                               np.zeros(5, np.float32), np.ones(5, np.float32), 0.0)
+    np.testing.assert_allclose(shifted - x, np.arange(5, dtype=np.float32)[None, :, None, None]
+                               * np.ones_like(x), atol=1e-6)
+
+
 def test_trans_chain_plain_equals_transpose():
     x = rng.integers(0, 1000, (2, 3, 8, 5)).astype(np.uint32)
     # H2N as micro-ops (TransposeOp::getTTParam, operator.cc:2436-2455)
