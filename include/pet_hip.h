@@ -262,6 +262,23 @@ PET_HIP_API int pet_hip_batchnorm(const float *x, const float *scale, const floa
                       const float *mean, const float *var, float *y, size_t outer, size_t ch,
                       size_t inner, float eps, pet_hip_stream_t stream);
 
+/* GatherOp: out[j..., p..., q...] = x[p..., indices[j...], q...], the index dims
+ * leading the output (GatherOp::computeShape, src/Graph/operator.cc:3420-3428, and
+ * the lambda of CodeEngine::genGatherCompute, src/Graph/code_engine.cc:1465-1498,
+ * which this replaces). pre / post: products of the dims of x before / after the
+ * axis, dim: the axis extent, nidx: number of indices. indices: int32, or fp32
+ * values holding integers when index_is_float != 0. Negative indices count from the
+ * end; indices outside the axis give zeros. The reference has no CPU compute for it
+ * (src/Graph/operator.cc:3409-3412). */
+PET_HIP_API int pet_hip_gather(const float *x, const void *indices, int index_is_float, float *y,
+                   size_t pre, size_t dim, size_t post, size_t nidx, pet_hip_stream_t stream);
+
+/* ReduceMeanOp: y[o, 0, i] = mean over d of x[o, d, i] (shape rule
+ * ReduceMeanOp::computeShape, src/Graph/operator.cc:3454-3458; no CPU compute and no
+ * GPU emitter upstream, :3443-3446). */
+PET_HIP_API int pet_hip_reduce_mean(const float *x, float *y, size_t outer, size_t dim, size_t inner,
+                        pet_hip_stream_t stream);
+
 /* y = act(x); replaces cudnnActivationForward (src/Graph/code_engine.cc:1260-1274).
  * The reference has no CPU compute for it (include/operator.h:1968-1977). */
 PET_HIP_API int pet_hip_activation(const float *x, float *y, size_t n, int act, pet_hip_stream_t stream);

@@ -321,6 +321,31 @@ def batchnorm(x, scale, bias, mean, var, eps=1e-5):
     return y
 
 
+def gather(x, indices, axis):
+    """GatherOp (operator.cc:3420-3428, code_engine.cc:1465-1498): index dims first."""
+    x = _c(x.astype(np.float32, copy=False))
+    idx = _c(np.asarray(indices).astype(np.int32))
+    pre = int(np.prod(x.shape[:axis], dtype=np.int64))
+    post = int(np.prod(x.shape[axis + 1:], dtype=np.int64))
+    y = np.empty(tuple(idx.shape) + x.shape[:axis] + x.shape[axis + 1:], dtype=np.float32)
+    lib().oracle_gather_f32(_p(x), _p(idx), _p(y), ctypes.c_size_t(pre),
+                            ctypes.c_size_t(x.shape[axis]), ctypes.c_size_t(post),
+                            ctypes.c_size_t(idx.size))
+    return y
+
+
+def reduce_mean(x, axis):
+    x = _c(x.astype(np.float32, copy=False))
+    outer = int(np.prod(x.shape[:axis], dtype=np.int64))
+    inner = int(np.prod(x.shape[axis + 1:], dtype=np.int64))
+    shp = list(x.shape)
+    shp[axis] = 1
+    y = np.empty(shp, dtype=np.float32)
+    lib().oracle_reduce_mean_f32(_p(x), _p(y), ctypes.c_size_t(outer),
+                                 ctypes.c_size_t(x.shape[axis]), ctypes.c_size_t(inner))
+    return y
+
+
 SPLIT, REORDER, FUSE = 0, 1, 2
 
 

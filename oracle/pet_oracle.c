@@ -30,6 +30,8 @@
  *   div : numpy true division. The reference's DivOp::compute body subtracts
  *       (src/Graph/operator.cc:3259) and nothing upstream runs Div on a GPU, so
  *       division itself is parity unpinned by the reference.
+ *   gather, reduce_mean : numpy.take + moveaxis / numpy.mean(keepdims). The reference
+ *       holds shape rules only (src/Graph/operator.cc:3409-3458): parity unpinned by it.
  *   batchnorm : torch.nn.functional.batch_norm (CPU, inference mode) and the
  *       identity statistics (mean 0, var 1 - eps, scale 1, bias 0 -> y = x).
  *   trans_chain : numpy constructions of halo split / drop fuse / pad fuse /
@@ -152,6 +154,36 @@ PET_ORACLE_EXPORT void oracle_batchnorm_f32(const float *x, const float *scale,
         double factor = (double)scale[c] / sqrt((double)var[c] + (double)eps);
         y[i] = (float)(((double)x[i] - (double)mean[c]) * factor + (double)bias[c]);
     }
+}
+
+/* GatherOp as the reference's shape rule and GPU lambda define it
+ * (src/Graph/operator.cc:3420-3428, src/Graph/code_engine.cc:1465-1498):
+ * out[j, p, q] = x[p, idx[j], q]; negative indices count from the end, indices
+ * outside the axis give 0. */
+PET_ORACLE_EXPORT void oracle_gather_f32(const float *x, const int *idx, float *y, size_t pre,
+                                         size_t dim, size_t post, size_t nidx) {
+    for (size_t j = 0; j < nidx; ++j) {
+        long long id = idx[j];
+        if (id < 0)
+            id += (long long)dim;
+        for (size_t p = 0; p < pre; ++p)
+            for (size_t q = 0; q < post; ++q)
+                y[(j * pre + p) * post + q] =
+                    (id >= 0 && id < (long long)dim) ? x[(p * dim + (size_t)id) * post + q] : 0.f;
+    }
+}
+
+/* ReduceMeanOp (shape rule src/Graph/operator.cc:3454-3458): mean over the axis in
+ * double. */
+PET_ORACLE_EXPORT void oracle_reduce_mean_f32(const float *x, float *y, size_t outer, size_t dim,
+                                              size_t inner) {
+    for (size_t o = 0; o < outer; ++o)
+        for (size_t i = 0; i < inner; ++i) {
+            double s = 0.0;
+            for (size_t d = 0; d < dim; ++d)
+                s += (double)x[(o * dim + d) * inner + i];
+            y[o * inner + i] = (float)(s / (double)dim);
+        }
 }
 
 /* y[o, ch, inner] = act(x + bias[ch]): the epilogue the GPU path fuses

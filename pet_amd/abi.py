@@ -62,6 +62,8 @@ SIGNATURES = {
     "pet_hip_eltwise": [_i, ctypes.POINTER(_vp), ctypes.POINTER(_sz), _i, _vp, _sz, _vp],
     "pet_hip_activation": [_vp, _vp, _sz, _i, _vp],
     "pet_hip_pow": [_vp, _vp, _sz, _i, _vp],
+    "pet_hip_gather": [_vp, _vp, _i, _vp, _sz, _sz, _sz, _sz, _vp],
+    "pet_hip_reduce_mean": [_vp, _vp, _sz, _sz, _sz, _vp],
     "pet_hip_batchnorm": [_vp] * 6 + [_sz, _sz, _sz, ctypes.c_float, _vp],
     "pet_hip_bias_act": [_vp, _vp, _vp, _sz, _sz, _sz, _i, _vp],
     "pet_hip_pool2d": [_vp, _vp] + [_i] * 13 + [_vp],

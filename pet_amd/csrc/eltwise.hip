@@ -161,6 +161,62 @@ __global__ __launch_bounds__(256) void batchnorm_kernel(const float *__restrict_
     }
 }
 
+// out[j, p, q] = x[p, idx[j], q]: the index dims lead the output, as in the
+// reference's shape rule. Negative indices count from the end; an index outside
+// the axis gives zeros.
+template <bool FIDX>
+__global__ __launch_bounds__(256) void gather_kernel(const float *__restrict__ x,
+                                                     const void *__restrict__ indices,
+                                                     float *__restrict__ y, size_t total,
+                                                     size_t pre, long long dim, size_t post) {
+    size_t o = (size_t)blockIdx.x * 256 + threadIdx.x;
+    const size_t step = (size_t)gridDim.x * 256;
+    const size_t slab = pre * post;
+    for (; o < total; o += step) {
+        const size_t j = o / slab, r = o - j * slab;
+        const size_t pi = r / post, q = r - pi * post;
+        long long id = FIDX ? (long long)rintf(static_cast<const float *>(indices)[j])
+                            : (long long)static_cast<const int *>(indices)[j];
+        if (id < 0)
+            id += dim;
+        y[o] = (id >= 0 && id < dim) ? x[(pi * (size_t)dim + (size_t)id) * post + q] : 0.f;
+    }
+}
+
+// y[o, i] = mean over d of x[o, d, i]. A thread owns one output and walks d
+// (neighbouring threads read neighbouring i); with inner == 1 a wave owns one row
+// and sums it across lanes.
+__global__ __launch_bounds__(256) void reduce_mean_kernel(const float *__restrict__ x,
+                                                          float *__restrict__ y, size_t outer,
+                                                          size_t dim, size_t inner) {
+    if (inner == 1) {
+        const size_t wave = ((size_t)blockIdx.x * 256 + threadIdx.x) >> 6;
+        const size_t nwaves = ((size_t)gridDim.x * 256) >> 6;
+        const unsigned lane = threadIdx.x & 63;
+        for (size_t row = wave; row < outer; row += nwaves) {
+            float s = 0.f;
+            for (size_t d = lane; d < dim; d += 64)
+                s += x[row * dim + d];
+#pragma unroll
+            for (int off = 32; off > 0; off >>= 1)
+                s += __shfl_xor(s, off);
+            if (lane == 0)
+                y[row] = s / (float)dim;
+        }
+        return;
+    }
+    size_t o = (size_t)blockIdx.x * 256 + threadIdx.x;
+    const size_t step = (size_t)gridDim.x * 256, total = outer * inner;
+    for (; o < total; o += step) {
+        const size_t ou = o / inner, i = o - ou * inner;
+        const float *src = x + ou * dim * inner + i;
+        float s = 0.f;
+        for (size_t d = 0; d < dim; ++d)
+            s += src[d * inner];
+        y[o] = s / (float)dim;
+    }
+}
+
 __global__ __launch_bounds__(256) void bias_act_kernel(const float *__restrict__ x,
                                                        const float *__restrict__ bias,
                                                        float *__restrict__ y, size_t total,
@@ -481,6 +537,42 @@ int pet_hip_batchnorm(const float *x, const float *scale, const float *bias, con
     hipLaunchKernelGGL(batchnorm_kernel, dim3(grid), dim3(256), 0, as_stream(stream), x, scale,
                        bias, mean, var, y, rows, (unsigned)ch, inner, eps, vec);
     return check_launch("batchnorm_kernel");
+}
+
+int pet_hip_gather(const float *x, const void *indices, int index_is_float, float *y, size_t pre,
+                   size_t dim, size_t post, size_t nidx, pet_hip_stream_t stream) {
+    PET_REQUIRE_INIT();
+    const size_t total = nidx * pre * post;
+    if (total == 0)
+        return PET_HIP_OK;
+    if (!x || !indices || !y)
+        return set_error(PET_HIP_ERR_INVALID, "null pointer");
+    if (dim == 0)
+        return set_error(PET_HIP_ERR_INVALID, "gather along an empty axis");
+    if (total >= (1ull << 40) || dim >= (1ull << 31))
+        return set_error(PET_HIP_ERR_UNSUPPORTED, "gather is limited to 2^40 outputs");
+    if (index_is_float)
+        hipLaunchKernelGGL(gather_kernel<true>, dim3(grid_for(total)), dim3(256), 0,
+                           as_stream(stream), x, indices, y, total, pre, (long long)dim, post);
+    else
+        hipLaunchKernelGGL(gather_kernel<false>, dim3(grid_for(total)), dim3(256), 0,
+                           as_stream(stream), x, indices, y, total, pre, (long long)dim, post);
+    return check_launch("gather_kernel");
+}
+
+int pet_hip_reduce_mean(const float *x, float *y, size_t outer, size_t dim, size_t inner,
+                        pet_hip_stream_t stream) {
+    PET_REQUIRE_INIT();
+    if (outer * inner == 0)
+        return PET_HIP_OK;
+    if (!x || !y)
+        return set_error(PET_HIP_ERR_INVALID, "null pointer");
+    if (dim == 0)
+        return set_error(PET_HIP_ERR_INVALID, "mean over an empty axis");
+    const size_t threads = inner == 1 ? outer * 64 : outer * inner;
+    hipLaunchKernelGGL(reduce_mean_kernel, dim3(grid_for(threads)), dim3(256), 0, as_stream(stream),
+                       x, y, outer, dim, inner);
+    return check_launch("reduce_mean_kernel");
 }
 
 int pet_hip_bias_act(const float *x, const float *bias, float *y, size_t outer, size_t ch,

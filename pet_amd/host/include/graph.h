@@ -88,6 +88,10 @@ class Graph : public GraphBase {
     Operator *div(Tensor *input0, Tensor *input1);
     Operator *pow(Tensor *input, Tensor *output, int pow);
     Operator *pow(Tensor *input, int pow);
+    Operator *gather(Tensor *data, Tensor *indices, Tensor *output, int axis);
+    Operator *gather(Tensor *data, Tensor *indices, int axis);
+    Operator *reduceMean(Tensor *input, Tensor *output, int axis);
+    Operator *reduceMean(Tensor *input, int axis);
     Operator *batchnorm(Tensor *input, Tensor *scale, Tensor *bias, Tensor *mean, Tensor *var,
                         Tensor *output, float epsilon = 1e-05, float momentum = 0.9);
     Operator *batchnorm(Tensor *input, Tensor *scale, Tensor *bias, Tensor *mean, Tensor *var,

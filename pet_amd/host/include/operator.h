@@ -718,6 +718,52 @@ class BatchNormOp : public Operator {
     Tensor *scale, *bias, *mean, *var;
 };
 
+// out[j..., p..., q...] = data[p..., indices[j...], q...]: the index dims lead the
+// output (src/Graph/operator.cc:3396-3428). Indices travel as fp32 values holding
+// integers, like every tensor of this host layer.
+class GatherOp : public Operator {
+  public:
+    GatherOp(Tensor *data, Tensor *indices, Tensor *output, int axis);
+    GatherOp(Tensor *data, Tensor *indices, int axis);
+    GatherOp() : Operator(Gather), axis(0) { initHash(); }
+    GatherOp(const GatherOp &rhs) : Operator(rhs), axis(rhs.axis) {}
+    GatherOp *clone() override { return new GatherOp(*this); }
+    Dim computeShape() override;
+    double perf(PerfEngine *pe, int rounds = 200, int warmupRounds = 200) override;
+    int launch(pet_hip_stream_t stream) override;
+    std::string toString() const override;
+    int numInputs() override { return 2; }
+    int numOutputs() override { return 1; }
+    int getAxis() const { return axis; }
+
+  private:
+    bool checkValid(const TensorVec &ins) override;
+    void initHash() override;
+    int axis;
+};
+
+// Mean over one axis, which stays in the shape as 1 (src/Graph/operator.cc:3430-3458).
+class ReduceMeanOp : public Operator {
+  public:
+    ReduceMeanOp(Tensor *input, Tensor *output, int axis);
+    ReduceMeanOp(Tensor *input, int axis);
+    ReduceMeanOp() : Operator(ReduceMean), axis(0) { initHash(); }
+    ReduceMeanOp(const ReduceMeanOp &rhs) : Operator(rhs), axis(rhs.axis) {}
+    ReduceMeanOp *clone() override { return new ReduceMeanOp(*this); }
+    Dim computeShape() override;
+    double perf(PerfEngine *pe, int rounds = 200, int warmupRounds = 200) override;
+    int launch(pet_hip_stream_t stream) override;
+    std::string toString() const override;
+    int numInputs() override { return 1; }
+    int numOutputs() override { return 1; }
+    int getAxis() const { return axis; }
+
+  private:
+    bool checkValid(const TensorVec &ins) override;
+    void initHash() override;
+    int axis;
+};
+
 // ---- single-input ops without a reference CPU compute ----------------------------
 class ActivationOp : public Operator {
   public:

@@ -634,6 +634,25 @@ std::string CodeEngine::genCode(std::shared_ptr<SubGraph> &graph) {
             c << "pet_hip_eltwise(" << code << ", eins" << id << ", esz" << id << ", "
               << op->getInputs().size() << ", " << out(0) << ", " << op->getOutputs()[0]->size()
               << ", s)";
+        } else if (auto ga = dynamic_cast<GatherOp *>(op)) {
+            const Dim &d = op->getInputs()[0]->getDims();
+            size_t pre = 1, post = 1;
+            for (int i = 0; i < ga->getAxis(); ++i)
+                pre *= (size_t)d[i];
+            for (size_t i = ga->getAxis() + 1; i < d.size(); ++i)
+                post *= (size_t)d[i];
+            c << "pet_hip_gather(" << in(0) << ", " << in(1) << ", 1, " << out(0) << ", " << pre
+              << ", " << d[ga->getAxis()] << ", " << post << ", " << op->getInputs()[1]->size()
+              << ", s)";
+        } else if (auto rm = dynamic_cast<ReduceMeanOp *>(op)) {
+            const Dim &d = op->getInputs()[0]->getDims();
+            size_t outer = 1, inner = 1;
+            for (int i = 0; i < rm->getAxis(); ++i)
+                outer *= (size_t)d[i];
+            for (size_t i = rm->getAxis() + 1; i < d.size(); ++i)
+                inner *= (size_t)d[i];
+            c << "pet_hip_reduce_mean(" << in(0) << ", " << out(0) << ", " << outer << ", "
+              << d[rm->getAxis()] << ", " << inner << ", s)";
         } else if (auto pw = dynamic_cast<PowOp *>(op)) {
             c << "pet_hip_pow(" << in(0) << ", " << out(0) << ", " << op->getInputs()[0]->size()
               << ", " << pw->getPow() << ", s)";

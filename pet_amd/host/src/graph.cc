@@ -198,6 +198,18 @@ Operator *Graph::pow(Tensor *input, Tensor *output, int pow) {
     return own(new PowOp(input, output, pow));
 }
 Operator *Graph::pow(Tensor *input, int pow) { return own(new PowOp(input, pow)); }
+Operator *Graph::gather(Tensor *data, Tensor *indices, Tensor *output, int axis) {
+    return own(new GatherOp(data, indices, output, axis));
+}
+Operator *Graph::gather(Tensor *data, Tensor *indices, int axis) {
+    return own(new GatherOp(data, indices, axis));
+}
+Operator *Graph::reduceMean(Tensor *input, Tensor *output, int axis) {
+    return own(new ReduceMeanOp(input, output, axis));
+}
+Operator *Graph::reduceMean(Tensor *input, int axis) {
+    return own(new ReduceMeanOp(input, axis));
+}
 Operator *Graph::batchnorm(Tensor *input, Tensor *scale, Tensor *bias, Tensor *mean, Tensor *var,
                            Tensor *output, float epsilon, float momentum) {
     return own(new BatchNormOp(input, scale, bias, mean, var, output, epsilon, momentum));

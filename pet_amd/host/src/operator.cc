@@ -1359,6 +1359,99 @@ std::string BatchNormOp::toString() const {
     return os.str();
 }
 
+// ---- Gather / ReduceMean --------------------------------------------------------------
+
+GatherOp::GatherOp(Tensor *data, Tensor *indices, Tensor *output, int axis)
+    : Operator(Gather, {data, indices}, {output}), axis(axis) {
+    assert(checkValid(inputs));
+    computeShape();
+    initHash();
+}
+GatherOp::GatherOp(Tensor *data, Tensor *indices, int axis)
+    : GatherOp(data, indices, new Tensor(), axis) {}
+
+void GatherOp::initHash() { hash = hashPack(hashAppend(type, axis)); }
+
+bool GatherOp::checkValid(const TensorVec &ins) {
+    return ins.size() == 2 && ins[0] && ins[1] && axis >= 0 &&
+           axis < (int)ins[0]->getDims().size();
+}
+
+Dim GatherOp::computeShape() {
+    Dim dim = inputs[1]->getDims();
+    const Dim &data = inputs[0]->getDims();
+    for (size_t i = 0; i < data.size(); ++i)
+        if ((int)i != axis)
+            dim.push_back(data[i]);
+    outputs[0]->setDims(dim);
+    outputs[0]->setType(Tensor::Input);
+    return dim;
+}
+
+int GatherOp::launch(pet_hip_stream_t stream) {
+    const Dim &d = inputs[0]->getDims();
+    size_t pre = 1, post = 1;
+    for (int i = 0; i < axis; ++i)
+        pre *= (size_t)d[i];
+    for (size_t i = axis + 1; i < d.size(); ++i)
+        post *= (size_t)d[i];
+    return pet_hip_gather(inputs[0]->devicePtr(), inputs[1]->devicePtr(), 1,
+                          outputs[0]->devicePtr(), pre, (size_t)d[axis], post, inputs[1]->size(),
+                          stream);
+}
+
+double GatherOp::perf(PerfEngine *, int rounds, int warmupRounds) {
+    return timeLaunches(std::min(rounds, 50), std::min(warmupRounds, 10));
+}
+
+std::string GatherOp::toString() const {
+    std::ostringstream os;
+    os << "Gather(data=" << inputs[0]->getHash() << ",indices=" << inputs[1]->getHash()
+       << ",out=" << outputs[0]->getHash() << ",axis=" << axis << ")";
+    return os.str();
+}
+
+ReduceMeanOp::ReduceMeanOp(Tensor *input, Tensor *output, int axis)
+    : Operator(ReduceMean, {input}, {output}), axis(axis) {
+    assert(checkValid(inputs));
+    computeShape();
+    initHash();
+}
+ReduceMeanOp::ReduceMeanOp(Tensor *input, int axis) : ReduceMeanOp(input, new Tensor(), axis) {}
+
+void ReduceMeanOp::initHash() { hash = hashPack(hashAppend(type, axis)); }
+
+bool ReduceMeanOp::checkValid(const TensorVec &ins) {
+    return ins.size() == 1 && ins[0] && axis >= 0 && axis < (int)ins[0]->getDims().size();
+}
+
+Dim ReduceMeanOp::computeShape() {
+    Dim dim = inputs[0]->getDims();
+    dim[axis] = 1;
+    outputs[0]->setDims(dim);
+    outputs[0]->setType(inputs[0]->getType());
+    return dim;
+}
+
+int ReduceMeanOp::launch(pet_hip_stream_t stream) {
+    const Dim &d = inputs[0]->getDims();
+    size_t outer = 1, inner = 1;
+    for (int i = 0; i < axis; ++i)
+        outer *= (size_t)d[i];
+    for (size_t i = axis + 1; i < d.size(); ++i)
+        inner *= (size_t)d[i];
+    return pet_hip_reduce_mean(inputs[0]->devicePtr(), outputs[0]->devicePtr(), outer,
+                               (size_t)d[axis], inner, stream);
+}
+
+double ReduceMeanOp::perf(PerfEngine *, int rounds, int warmupRounds) {
+    return timeLaunches(std::min(rounds, 50), std::min(warmupRounds, 10));
+}
+
+std::string ReduceMeanOp::toString() const {
+    return "ReduceMean(axis=" + std::to_string(axis) + ")";
+}
+
 // ---- Activation / Pool / Softmax / LayerNorm / Reshape -----------------------------
 
 ActivationOp::ActivationOp(Tensor *input, Tensor *output, ActType act)

@@ -336,6 +336,45 @@ def batchnorm(x, scale, bias, mean, var, eps=1e-5, out=None):
     return out
 
 
+def gather(x, indices, axis, out=None):
+    """GatherOp (shape rule operator.cc:3420-3428): the index dims lead the output.
+    indices: int32 or float32 (holding integers) tensor on the device."""
+    if indices.dtype not in (torch.int32, torch.float32):
+        raise abi.PetHipError(1, "indices must be int32 or float32")
+    _chk(x, out)
+    if not (indices.is_cuda and indices.is_contiguous()):
+        raise abi.PetHipError(1, "indices must be a contiguous device tensor")
+    pre = 1
+    for d in x.shape[:axis]:
+        pre *= d
+    post = 1
+    for d in x.shape[axis + 1:]:
+        post *= d
+    shp = list(indices.shape) + list(x.shape[:axis]) + list(x.shape[axis + 1:])
+    if out is None:
+        out = torch.empty(shp, device=x.device, dtype=torch.float32)
+    abi.call("pet_hip_gather", _ptr(x), indices.data_ptr(), int(indices.dtype == torch.float32),
+             _ptr(out), pre, x.shape[axis], post, indices.numel(), _stream())
+    return out
+
+
+def reduce_mean(x, axis, out=None):
+    """ReduceMeanOp (shape rule operator.cc:3454-3458): mean over one axis, kept as 1."""
+    _chk(x, out)
+    outer = 1
+    for d in x.shape[:axis]:
+        outer *= d
+    inner = 1
+    for d in x.shape[axis + 1:]:
+        inner *= d
+    shp = list(x.shape)
+    shp[axis] = 1
+    if out is None:
+        out = torch.empty(shp, device=x.device, dtype=torch.float32)
+    abi.call("pet_hip_reduce_mean", _ptr(x), _ptr(out), outer, x.shape[axis], inner, _stream())
+    return out
+
+
 def bias_act(x, bias, act="none", ch_axis=1, out=None):
     _chk(x, bias, out)
     outer = 1

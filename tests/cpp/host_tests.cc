@@ -562,6 +562,54 @@ static bool test_batchnorm_pow_div() {
     return true;
 }
 
+// GatherOp / ReduceMeanOp: the reference holds shape rules only
+// (src/Graph/operator.cc:3409-3458); an embedding look-up followed by a mean.
+static bool test_gather_reduce_mean() {
+    Graph g;
+    auto table = g.tensor({20, 8}), idx = g.tensor({2, 3}, Tensor::Int32);
+    auto ga = g.gather(table, idx, 0);
+    EXPECT(ga->getOutputs()[0]->getDims() == (Dim{2, 3, 8}));
+    auto rm = g.reduceMean(ga->getOutputs()[0], 2);
+    EXPECT(rm->getOutputs()[0]->getDims() == (Dim{2, 3, 1}));
+    g.updateConnection();
+    auto s1 = std::make_shared<SubGraph>(g.getOperators());
+    auto s2 = std::make_shared<SubGraph>(g.getOperators());
+    const float rows[6] = {3.f, 19.f, 0.f, -1.f, 7.f, 3.f}; // -1 counts from the end
+    for (size_t i = 0; i < s1->getInputs().size(); ++i) {
+        Tensor *t = s1->getInputs()[i];
+        if (t->size() == 6)
+            t->setData(rows);
+        else
+            t->dataRand(41);
+        s2->getInputs()[i]->setData(t->getDataPtr());
+    }
+    EXPECT(s1->compute());
+    Tensor *tab = nullptr;
+    for (auto t : s1->getInputs())
+        if (t->size() == 160)
+            tab = t;
+    EXPECT(tab != nullptr);
+    Tensor *out = s1->getOutputs()[0];
+    for (int j = 0; j < 6; ++j) {
+        int r = rows[j] < 0 ? 20 + (int)rows[j] : (int)rows[j];
+        double want = 0;
+        for (int q = 0; q < 8; ++q)
+            want += tab->getData({r, q});
+        want /= 8.0;
+        EXPECT(std::fabs((double)out->getData(j) - want) <= 1e-5 * std::max(1.0, std::fabs(want)));
+    }
+    CodeEngine ce;
+    auto exec = ce.instantiate(s2);
+    EXPECT(exec != nullptr);
+    EXPECT(exec->launch() && exec->sync());
+    s2->getOutputs()[0]->deviceWritten();
+    EXPECT(equalArrays(out->getDataPtr(), s2->getOutputs()[0]->getDataPtr(), out->size()));
+    std::string code = ce.genCode(s2);
+    EXPECT(code.find("pet_hip_gather(") != std::string::npos);
+    EXPECT(code.find("pet_hip_reduce_mean(") != std::string::npos);
+    return true;
+}
+
 // src/Mutant/generator.cc:1327-1381: two convolutions of one input become one
 // (weights concatenated on dim 0, result split on dim 1); :1159-1234: two
 // convolutions of different inputs and filter counts 8 and 12 become one
@@ -652,6 +700,7 @@ int main(int argc, char **argv) {
         {"perf_engine_memo", test_perf_engine_memo},
         {"split_ratio_and_eltwise", test_split_ratio_and_eltwise},
         {"batchnorm_pow_div", test_batchnorm_pow_div},
+        {"gather_reduce_mean", test_gather_reduce_mean},
         {"conv_merge_programs", test_conv_merge_programs},
     };
     std::string only = argc > 1 ? argv[1] : "";

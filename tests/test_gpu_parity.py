@@ -691,6 +691,33 @@ def test_pow_div_batchnorm(ops):
         ops.batchnorm(dev(x), dev(sc[:-1]), dev(bi), dev(me), dev(va))
 
 
+def test_gather_reduce_mean(ops):
+    """Gather: bit-exact, int32 and fp32-held indices, negative and out-of-range ones.
+    ReduceMean: 1e-5 relative (fp32 running sum against the oracle's double)."""
+    rng = np.random.default_rng(14)
+    x = rng.standard_normal((3, 50, 4, 6)).astype(np.float32)
+    for axis in range(4):
+        for shape in [(7,), (2, 3), (1,)]:
+            idx = rng.integers(-x.shape[axis], x.shape[axis], shape).astype(np.int32)
+            ref = oracle.gather(x, idx, axis)
+            for dt in (torch.int32, torch.float32):
+                got = host(ops.gather(dev(x), torch.from_numpy(idx).to(dt).cuda(), axis))
+                assert got.shape == ref.shape and got.tobytes() == ref.tobytes(), (axis, shape)
+    idx = np.array([49, 50, -50, -51], dtype=np.int32)
+    got = host(ops.gather(dev(x), torch.from_numpy(idx).cuda(), 1))
+    assert got.tobytes() == oracle.gather(x, idx, 1).tobytes() and not got[1].any()
+    table = rng.standard_normal((30522 // 8, 768)).astype(np.float32)   # an embedding look-up
+    tok = rng.integers(0, table.shape[0], (128,)).astype(np.int32)
+    assert host(ops.gather(dev(table), torch.from_numpy(tok).cuda(), 0)).tobytes() == \
+        table[tok].tobytes()
+
+    for shape in [(3, 50, 4, 6), (2, 7, 300), (5, 1000), (4, 512, 7, 7), (1, 3)]:
+        x = rng.standard_normal(shape).astype(np.float32)
+        for axis in range(len(shape)):
+            np.testing.assert_allclose(host(ops.reduce_mean(dev(x), axis)),
+                                       oracle.reduce_mean(x, axis), rtol=1e-5, atol=1e-6)
+
+
 def test_activation_pool_softmax_layernorm(ops):
     rng = np.random.default_rng(10)
     x = rng.standard_normal((2, 3, 9, 9)).astype(np.float32)

@@ -18,7 +18,8 @@ CASES = ["conv_vs_oracle", "conv_invalid_groups", "transpose_n2h_h2n", "batch_ge
          "pad_conv_slice_verification", "corrected_h2n_program",
          "dilated_space_to_batch_program", "code_engine_graph_runtime", "perf_engine_memo",
          "split_ratio_and_eltwise", "conv_merge_programs", "conv3d_prepacked_graph",
-         "random_graphs_replay_equals_eager", "batchnorm_pow_div"]
+         "random_graphs_replay_equals_eager", "batchnorm_pow_div",
+         "gather_reduce_mean"]
 
 
 def test_host_library_is_built_and_exports_the_operator_classes():
