@@ -54,6 +54,28 @@ typedef enum pet_hip_eltwise_op {
                         reference's CPU body at :3259 subtracts) */
 } pet_hip_eltwise_op;
 
+/* Flags of the *_ex contraction entry points: what a graph runtime fuses across
+ * launches. No counterpart upstream, where cuDNN / cuBLAS calls stand alone. */
+typedef enum pet_hip_call_flags {
+    /* y already holds bias (or zeros): a launch that accumulates into y (see the
+     * *_accumulates queries) skips its initialising launch; bias must still be passed.
+     * Not together with a residual. Other launches overwrite y as usual. */
+    PET_HIP_CALL_Y_INITIALISED = 1,
+    /* act is ReLU and every reader of y applies it on load (the two flags below): a
+     * launch that accumulates into y leaves the ReLU out; others apply it as usual,
+     * which the readers' second ReLU does not change. */
+    PET_HIP_CALL_DEFER_RELU = 2,
+    PET_HIP_CALL_X_RELU = 4,   /* use max(x, 0) for x */
+    PET_HIP_CALL_RES_RELU = 8  /* use max(residual, 0) for the residual */
+} pet_hip_call_flags;
+
+/* One output of pet_hip_bias_fill_batch: y[o][c][i] = bias[c] (zeros when bias is NULL). */
+typedef struct pet_hip_fill {
+    float *y;
+    const float *bias;
+    size_t outer, ch, inner;
+} pet_hip_fill;
+
 /* Opaque handles (a hipStream_t / hipEvent_t / hipGraphExec_t underneath). */
 typedef void *pet_hip_stream_t;
 typedef void *pet_hip_event_t;
@@ -160,6 +182,12 @@ PET_HIP_API int pet_hip_bmm_res_f32(int transA, int transB, int b, int m, int n,
                         const float *B, float *C, const float *bias, const float *residual,
                         int act, pet_hip_stream_t stream);
 
+/* Matmul with every optional operand; flags: PET_HIP_CALL_Y_INITIALISED only. */
+PET_HIP_API int pet_hip_bmm_ex_f32(int transA, int transB, int b, int m, int n, int k, const float *A,
+                       const float *B, float *C, const float *bias, const float *residual, int act,
+                       unsigned flags, pet_hip_stream_t stream);
+PET_HIP_API int pet_hip_bmm_accumulates(int transA, int transB, int b, int m, int n, int k, int *yes);
+
 /* Constant 3-D filters, reordered once: [f][c/groups][kt][r][s] -> kt-major
  * [kt][f][c/groups][r][s] (same element count), so that each kt slice is a 2-D
  * filter bank the convolution kernel reads with 16-byte loads. This is a
@@ -179,6 +207,32 @@ PET_HIP_API int pet_hip_conv3d_packed_f32(const float *x, const float *packed, c
                               float *y, int n, int c, int t, int h, int wd, int f, int kt, int r,
                               int s, int pt, int ph, int pw, int st, int sh, int sw, int dt,
                               int dh, int dw, int groups, int act, pet_hip_stream_t stream);
+
+/* The same contractions with every optional operand and the flags above, for graph
+ * runtimes (the host layer's CodeEngine plans them): a split or stream-K launch
+ * normally runs as "initialise y, accumulate, activate"; with the initialisations of a
+ * whole graph batched into one pet_hip_bias_fill_batch launch at its start, and ReLU
+ * left to the convolutions that read y, it is one launch. */
+PET_HIP_API int pet_hip_conv2d_ex_f32(const float *x, const float *w, const float *bias,
+                          const float *residual, float *y, int n, int c, int h, int wd, int f,
+                          int r, int s, int ph, int pw, int sh, int sw, int dh, int dw, int groups,
+                          int act, unsigned flags, pet_hip_stream_t stream);
+PET_HIP_API int pet_hip_conv3d_ex_f32(const float *x, const float *w, int w_is_packed, const float *bias,
+                          const float *residual, float *y, int n, int c, int t, int h, int wd,
+                          int f, int kt, int r, int s, int pt, int ph, int pw, int st, int sh,
+                          int sw, int dt, int dh, int dw, int groups, int act, unsigned flags,
+                          pet_hip_stream_t stream);
+/* *yes = 1 when a launch of this shape accumulates into y with atomics (and so starts
+ * by writing bias into all of y, unless told that y is initialised). Depends on the
+ * shape and on PET_HIP_DETERMINISTIC only. */
+PET_HIP_API int pet_hip_conv2d_accumulates(int n, int c, int h, int wd, int f, int r, int s, int ph,
+                               int pw, int sh, int sw, int dh, int dw, int groups, int *yes);
+PET_HIP_API int pet_hip_conv3d_accumulates(int n, int c, int t, int h, int wd, int f, int kt, int r,
+                               int s, int pt, int ph, int pw, int st, int sh, int sw, int dt,
+                               int dh, int dw, int groups, int w_is_packed, int *yes);
+/* y[o][c][i] = bias[c] for `count` outputs in one launch (a convolution's output is
+ * [n][f][pixels], a matmul's [b*m][n][1]). */
+PET_HIP_API int pet_hip_bias_fill_batch(const pet_hip_fill *fills, int count, pet_hip_stream_t stream);
 
 /* Batched row-major matmul C[b,m,n] = A'[b,m,k] * B'[b,k,n]; transA: A stored
  * [b,k,m]; transB: B stored [b,n,k]. bias (may be NULL) is [n], added per

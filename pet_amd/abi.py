@@ -12,6 +12,14 @@ LIB_PATH = os.path.join(_HERE, "lib", "libpet_hip.so")
 
 ACT = {"none": 0, "relu": 1, "sigmoid": 2, "tanh": 3, "gelu": 4, None: 0}
 ELT = {"add": 0, "sub": 1, "mul": 2, "div": 3}
+# pet_hip_call_flags
+Y_INITIALISED, DEFER_RELU, X_RELU, RES_RELU = 1, 2, 4, 8
+
+
+class Fill(ctypes.Structure):
+    """pet_hip_fill"""
+    _fields_ = [("y", ctypes.c_void_p), ("bias", ctypes.c_void_p), ("outer", ctypes.c_size_t),
+                ("ch", ctypes.c_size_t), ("inner", ctypes.c_size_t)]
 
 _c_int_p = ctypes.POINTER(ctypes.c_int)
 _vp = ctypes.c_void_p
@@ -49,6 +57,13 @@ SIGNATURES = {
     "pet_hip_conv2d_res_f32": [_vp] * 5 + [_i] * 15 + [_vp],
     "pet_hip_conv3d_res_f32": [_vp, _vp, _i, _vp, _vp, _vp] + [_i] * 20 + [_vp],
     "pet_hip_bmm_res_f32": [_i] * 6 + [_vp] * 5 + [_i, _vp],
+    "pet_hip_conv2d_ex_f32": [_vp] * 5 + [_i] * 15 + [ctypes.c_uint, _vp],
+    "pet_hip_conv3d_ex_f32": [_vp, _vp, _i, _vp, _vp, _vp] + [_i] * 20 + [ctypes.c_uint, _vp],
+    "pet_hip_bmm_ex_f32": [_i] * 6 + [_vp] * 5 + [_i, ctypes.c_uint, _vp],
+    "pet_hip_conv2d_accumulates": [_i] * 14 + [_c_int_p],
+    "pet_hip_conv3d_accumulates": [_i] * 20 + [_c_int_p],
+    "pet_hip_bmm_accumulates": [_i] * 6 + [_c_int_p],
+    "pet_hip_bias_fill_batch": [_vp, _i, _vp],
     "pet_hip_conv3d_pack_filters": [_vp, _vp] + [_i] * 5 + [_vp],
     "pet_hip_conv3d_packed_f32": [_vp] * 4 + [_i] * 20 + [_vp],
     "pet_hip_bmm_f32": [_i] * 6 + [_vp] * 4 + [_i, _vp],

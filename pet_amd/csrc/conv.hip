@@ -47,6 +47,12 @@ struct ConvParams {
     int sk_mode;   // split-K: 0 partial tiles + ordered sum in one launch, 1 atomics into y
     float *ws;     // split-K: partial tiles, [tile][split][register][thread]
     int *cnt;      // split-K: arrival counter per tile, zero between launches
+    // caller-side fusion across launches (the *_ex entry points)
+    int x_relu;     // the input is used as max(x, 0): its producer left ReLU to the readers
+    int res_relu;   // the same for the residual operand
+    int y_init;     // y already holds bias (or 0): a split launch does not initialise it
+    int defer_relu; // a split launch leaves its ReLU to the readers of y
+    int *dry_atomic; // not null: report whether the launch would accumulate into y, launch nothing
     FastDiv fd_krs, fd_rs, fd_s;     // k -> (c, kt, r, s)
     FastDiv fd_opix, fd_ohw, fd_ow;  // pixel -> (n, ot, oh, ow)
 };
@@ -175,7 +181,8 @@ __global__ __launch_bounds__(Cfg::NT) void conv_pipe_kernel(ConvParams p) {
             const int row = i - A_VPT;
 #pragma unroll
             for (int pp = 0; pp < PPL; ++pp)
-                st[Cfg::A_ELEMS + b_lds + NW * row * B_LD + pp * 64] = preB[set][row][pp];
+                st[Cfg::A_ELEMS + b_lds + NW * row * B_LD + pp * 64] =
+                    p.x_relu ? fmaxf(preB[set][row][pp], 0.f) : preB[set][row][pp];
         }
     };
     auto r_piece = [&](int set, int i, const float *st) __attribute__((always_inline)) {
@@ -269,8 +276,10 @@ __global__ __launch_bounds__(Cfg::NT) void conv_pipe_kernel(ConvParams p) {
                     float v = acc[tm][tn][r];
                     if (bias)
                         v += bias[f];
-                    if (rb)
-                        v += rb[(unsigned)f * (unsigned)p.OPIX];
+                    if (rb) {
+                        const float rv = rb[(unsigned)f * (unsigned)p.OPIX];
+                        v += p.res_relu ? fmaxf(rv, 0.f) : rv;
+                    }
                     yb[(unsigned)f * (unsigned)p.OPIX] = apply_act(v, p.act);
                 }
             }
@@ -559,7 +568,8 @@ __global__ __launch_bounds__(Cfg::NT) void conv_plane_kernel(ConvParams p) {
             const int row = i - NA;
 #pragma unroll
             for (int pp = 0; pp < PPL; ++pp)
-                st[b_lds + NW * row * B_LD + pp * 64] = preB[row][pp];
+                st[b_lds + NW * row * B_LD + pp * 64] =
+                    p.x_relu ? fmaxf(preB[row][pp], 0.f) : preB[row][pp];
         }
     };
     auto r_piece = [&](int set, int i, const float *st) __attribute__((always_inline)) {
@@ -743,8 +753,11 @@ __global__ __launch_bounds__(Cfg::NT) void conv_plane_kernel(ConvParams p) {
                     float4 v = *reinterpret_cast<const float4 *>(lds + fl * C_LD + 4 * q);
                     const float bf = bias ? bias[f] : 0.f;
                     if (rb) {
-                        const float4 rv =
+                        float4 rv =
                             *reinterpret_cast<const float4 *>(rb + (unsigned)f * (unsigned)p.OPIX);
+                        if (p.res_relu)
+                            rv = make_float4(fmaxf(rv.x, 0.f), fmaxf(rv.y, 0.f), fmaxf(rv.z, 0.f),
+                                             fmaxf(rv.w, 0.f));
                         v.x += rv.x;
                         v.y += rv.y;
                         v.z += rv.z;
@@ -796,8 +809,10 @@ __global__ __launch_bounds__(Cfg::NT) void conv_plane_kernel(ConvParams p) {
                         float v = acc[tm][tn][r];
                         if (bias)
                             v += bias[f];
-                        if (rb)
-                            v += rb[(unsigned)f * (unsigned)p.OPIX];
+                        if (rb) {
+                            const float rv = rb[(unsigned)f * (unsigned)p.OPIX];
+                            v += p.res_relu ? fmaxf(rv, 0.f) : rv;
+                        }
                         yb[(unsigned)f * (unsigned)p.OPIX] = apply_act(v + colbias, p.act);
                     }
                 }
@@ -857,8 +872,9 @@ int pick_tile(int M, int N, int batch) {
 // column) or 0, plus the residual if there is one (which may be y itself); the
 // partial sums are then added atomically.
 __global__ __launch_bounds__(256) void splitk_init_kernel(float *y, const float *__restrict__ bias,
-                                                          const float *res, int bias_mode,
-                                                          unsigned F, unsigned OPIX, size_t total) {
+                                                          const float *res, int res_relu,
+                                                          int bias_mode, unsigned F, unsigned OPIX,
+                                                          size_t total) {
     size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
     const size_t step = (size_t)gridDim.x * 256;
     for (; i < total; i += step) {
@@ -869,7 +885,7 @@ __global__ __launch_bounds__(256) void splitk_init_kernel(float *y, const float 
             v = bias_mode == 2 ? bias[pix] : bias[f];
         }
         if (res)
-            v += res[i];
+            v += res_relu ? fmaxf(res[i], 0.f) : res[i];
         y[i] = v;
     }
 }
@@ -994,11 +1010,19 @@ int launch_plane_cfg(ConvParams p, hipStream_t stream) {
         }
         p.xcd_chunk = (int)chunk;
     }
-    if (p.atomic_out) {
+    if (p.dry_atomic) {
+        *p.dry_atomic = p.atomic_out;
+        return PET_HIP_OK;
+    }
+    if (p.atomic_out && p.y_init && p.res)
+        return set_error(PET_HIP_ERR_INVALID,
+                         "an initialised output cannot take a residual: fold it into the "
+                         "initialisation or leave the flag out");
+    if (p.atomic_out && !p.y_init) {
         const size_t total = (size_t)p.NPIX * p.F;
         unsigned igrid = (unsigned)std::min<size_t>((total + 255) / 256, 4096);
         hipLaunchKernelGGL(splitk_init_kernel, dim3(igrid), dim3(256), 0, stream, p.y, p.bias,
-                           p.res, p.bias_mode, (unsigned)p.F, (unsigned)p.OPIX, total);
+                           p.res, p.res_relu, p.bias_mode, (unsigned)p.F, (unsigned)p.OPIX, total);
         int rc = check_launch("splitk_init_kernel");
         if (rc)
             return rc;
@@ -1018,7 +1042,8 @@ int launch_plane_cfg(ConvParams p, hipStream_t stream) {
         hipLaunchKernelGGL((conv_plane_kernel<Cfg, DIM, false>), grid, dim3(Cfg::NT), lds_bytes,
                            stream, p);
     int rc = check_launch("conv_plane_kernel");
-    if (rc == PET_HIP_OK && p.atomic_out && p.act != PET_HIP_ACT_NONE)
+    if (rc == PET_HIP_OK && p.atomic_out && p.act != PET_HIP_ACT_NONE &&
+        !(p.defer_relu && p.act == PET_HIP_ACT_RELU))
         rc = pet_hip_activation(p.y, p.y, (size_t)p.NPIX * p.F, p.act, (pet_hip_stream_t)stream);
     return rc;
 }
@@ -1103,6 +1128,8 @@ int launch_conv(ConvParams &p, hipStream_t stream) {
         return set_error(PET_HIP_ERR_UNSUPPORTED,
                          "kt-major filters are only read by the plane kernel; this shape does "
                          "not use it (pet_hip_conv3d_pack_filters would have said so)");
+    if (p.dry_atomic) // the general kernel never accumulates into y
+        return PET_HIP_OK;
     const bool veca = (p.K % 4 == 0) && (((uintptr_t)p.w & 15) == 0);
     switch (pick_tile(p.M, p.NPIX, p.G)) {
     case 0:
@@ -1119,7 +1146,13 @@ int launch_conv(ConvParams &p, hipStream_t stream) {
 int conv_common(const float *x, const float *w, const float *bias, float *y, int n, int c, int t,
                 int h, int wd, int f, int kt, int r, int s, int pt, int ph, int pw, int st, int sh,
                 int sw, int dt, int dh, int dw, int groups, int act, hipStream_t stream,
-                bool wpacked = false, const float *res = nullptr) {
+                bool wpacked = false, const float *res = nullptr, unsigned flags = 0,
+                int *dry = nullptr) {
+    if (flags & ~(unsigned)(PET_HIP_CALL_Y_INITIALISED | PET_HIP_CALL_DEFER_RELU |
+                            PET_HIP_CALL_X_RELU | PET_HIP_CALL_RES_RELU))
+        return set_error(PET_HIP_ERR_INVALID, "unknown call flags 0x%x", flags);
+    if ((flags & PET_HIP_CALL_DEFER_RELU) && act != PET_HIP_ACT_RELU)
+        return set_error(PET_HIP_ERR_INVALID, "only a ReLU can be left to the readers");
     if (n < 0 || c <= 0 || t <= 0 || h <= 0 || wd <= 0 || f <= 0 || kt <= 0 || r <= 0 || s <= 0 ||
         groups <= 0 || st <= 0 || sh <= 0 || sw <= 0 || dt <= 0 || dh <= 0 || dw <= 0 || pt < 0 ||
         ph < 0 || pw < 0)
@@ -1148,6 +1181,12 @@ int conv_common(const float *x, const float *w, const float *bias, float *y, int
     if (in_elems >= (1ll << 31) || out_elems >= (1ll << 31) || kk >= (1ll << 30) ||
         (long long)f * kk >= (1ll << 31))
         return set_error(PET_HIP_ERR_UNSUPPORTED, "convolution operands above 2^31 elements");
+    if (dry) {
+        // shape query: the operands only have to look aligned
+        x = w = reinterpret_cast<const float *>(uintptr_t(256));
+        y = reinterpret_cast<float *>(uintptr_t(512));
+        *dry = 0;
+    }
     if (!x || !w || !y)
         return set_error(PET_HIP_ERR_INVALID, "null tensor pointer");
     if (res == y)
@@ -1184,6 +1223,11 @@ int conv_common(const float *x, const float *w, const float *bias, float *y, int
     p.act = act;
     p.bias_mode = 1;
     p.splitk = 1;
+    p.x_relu = (flags & PET_HIP_CALL_X_RELU) != 0;
+    p.res_relu = (flags & PET_HIP_CALL_RES_RELU) != 0;
+    p.y_init = (flags & PET_HIP_CALL_Y_INITIALISED) != 0;
+    p.defer_relu = (flags & PET_HIP_CALL_DEFER_RELU) != 0;
+    p.dry_atomic = dry;
     p.wpacked = wpacked;
     if (wpacked && !packed_filters_apply(f, c / groups, kt, r, s))
         return set_error(PET_HIP_ERR_UNSUPPORTED, "no kt-major form for this filter shape");
@@ -1208,11 +1252,14 @@ namespace mfma {
 // pixels, A[b] ([m][k]) its filters. Returns -1 when the plane kernel does not
 // apply (k not a multiple of 32, operands above 2 GiB, misaligned A).
 int bmm_as_grouped_1x1(const float *A, const float *B, float *C, const float *bias,
-                       const float *res, int b, int m, int n, int k, int act, hipStream_t stream) {
+                       const float *res, int b, int m, int n, int k, int act, hipStream_t stream,
+                       unsigned flags, int *dry) {
     if (k % 32 != 0 || b > 65535)
         return -1;
     ConvParams p;
     memset(&p, 0, sizeof(p));
+    p.y_init = (flags & PET_HIP_CALL_Y_INITIALISED) != 0;
+    p.dry_atomic = dry;
     p.x = B;
     p.w = A;
     p.bias = bias;
@@ -1285,6 +1332,45 @@ int pet_hip_conv3d_res_f32(const float *x, const float *w, int w_is_packed, cons
     PET_REQUIRE_INIT();
     return conv_common(x, w, bias, y, n, c, t, h, wd, f, kt, r, s, pt, ph, pw, st, sh, sw, dt, dh,
                        dw, groups, act, as_stream(stream), w_is_packed != 0, residual);
+}
+
+int pet_hip_conv2d_ex_f32(const float *x, const float *w, const float *bias,
+                          const float *residual, float *y, int n, int c, int h, int wd, int f,
+                          int r, int s, int ph, int pw, int sh, int sw, int dh, int dw, int groups,
+                          int act, unsigned flags, pet_hip_stream_t stream) {
+    PET_REQUIRE_INIT();
+    return conv_common(x, w, bias, y, n, c, 1, h, wd, f, 1, r, s, 0, ph, pw, 1, sh, sw, 1, dh, dw,
+                       groups, act, as_stream(stream), false, residual, flags);
+}
+
+int pet_hip_conv3d_ex_f32(const float *x, const float *w, int w_is_packed, const float *bias,
+                          const float *residual, float *y, int n, int c, int t, int h, int wd,
+                          int f, int kt, int r, int s, int pt, int ph, int pw, int st, int sh,
+                          int sw, int dt, int dh, int dw, int groups, int act, unsigned flags,
+                          pet_hip_stream_t stream) {
+    PET_REQUIRE_INIT();
+    return conv_common(x, w, bias, y, n, c, t, h, wd, f, kt, r, s, pt, ph, pw, st, sh, sw, dt, dh,
+                       dw, groups, act, as_stream(stream), w_is_packed != 0, residual, flags);
+}
+
+int pet_hip_conv2d_accumulates(int n, int c, int h, int wd, int f, int r, int s, int ph, int pw,
+                               int sh, int sw, int dh, int dw, int groups, int *yes) {
+    PET_REQUIRE_INIT();
+    if (!yes)
+        return set_error(PET_HIP_ERR_INVALID, "null result pointer");
+    return conv_common(nullptr, nullptr, nullptr, nullptr, n, c, 1, h, wd, f, 1, r, s, 0, ph, pw, 1,
+                       sh, sw, 1, dh, dw, groups, PET_HIP_ACT_NONE, nullptr, false, nullptr, 0, yes);
+}
+
+int pet_hip_conv3d_accumulates(int n, int c, int t, int h, int wd, int f, int kt, int r, int s,
+                               int pt, int ph, int pw, int st, int sh, int sw, int dt, int dh,
+                               int dw, int groups, int w_is_packed, int *yes) {
+    PET_REQUIRE_INIT();
+    if (!yes)
+        return set_error(PET_HIP_ERR_INVALID, "null result pointer");
+    return conv_common(nullptr, nullptr, nullptr, nullptr, n, c, t, h, wd, f, kt, r, s, pt, ph, pw,
+                       st, sh, sw, dt, dh, dw, groups, PET_HIP_ACT_NONE, nullptr, w_is_packed != 0,
+                       nullptr, 0, yes);
 }
 
 int pet_hip_conv3d_pack_filters(const float *w, float *packed, int f, int cpg, int kt, int r,

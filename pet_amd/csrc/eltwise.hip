@@ -3,6 +3,7 @@
 #include "common.h"
 
 #include <algorithm>
+#include <cstring>
 
 using namespace pet;
 
@@ -214,6 +215,35 @@ __global__ __launch_bounds__(256) void reduce_mean_kernel(const float *__restric
         for (size_t d = 0; d < dim; ++d)
             s += src[d * inner];
         y[o] = s / (float)dim;
+    }
+}
+
+// Several outputs set to their bias (or zero) in one launch: blockIdx.y picks the
+// output, y[o][c][i] = bias[c].
+constexpr int kMaxFills = 24;
+struct FillBatch {
+    float *y[kMaxFills];
+    const float *bias[kMaxFills];
+    unsigned ch[kMaxFills], inner[kMaxFills];
+    unsigned long long total[kMaxFills];
+};
+
+__global__ __launch_bounds__(256) void bias_fill_batch_kernel(FillBatch fb) {
+    const int j = blockIdx.y;
+    float *__restrict__ y = fb.y[j];
+    const float *__restrict__ bias = fb.bias[j];
+    const unsigned ch = fb.ch[j], inner = fb.inner[j];
+    const size_t total = fb.total[j];
+    const bool vec = inner % 4 == 0 && ((uintptr_t)y & 15) == 0;
+    const size_t step = (size_t)gridDim.x * 256;
+    if (vec) {
+        for (size_t q = (size_t)blockIdx.x * 256 + threadIdx.x; q * 4 < total; q += step) {
+            const float v = bias ? bias[(unsigned)((q * 4 / inner) % ch)] : 0.f;
+            *reinterpret_cast<float4 *>(y + q * 4) = make_float4(v, v, v, v);
+        }
+    } else {
+        for (size_t i = (size_t)blockIdx.x * 256 + threadIdx.x; i < total; i += step)
+            y[i] = bias ? bias[(unsigned)((i / inner) % ch)] : 0.f;
     }
 }
 
@@ -573,6 +603,44 @@ int pet_hip_reduce_mean(const float *x, float *y, size_t outer, size_t dim, size
     hipLaunchKernelGGL(reduce_mean_kernel, dim3(grid_for(threads)), dim3(256), 0, as_stream(stream),
                        x, y, outer, dim, inner);
     return check_launch("reduce_mean_kernel");
+}
+
+int pet_hip_bias_fill_batch(const pet_hip_fill *fills, int count, pet_hip_stream_t stream) {
+    PET_REQUIRE_INIT();
+    if (count < 0 || (count > 0 && !fills))
+        return set_error(PET_HIP_ERR_INVALID, "bad fill list");
+    for (int base = 0; base < count; base += kMaxFills) {
+        FillBatch fb;
+        memset(&fb, 0, sizeof(fb));
+        int nb = 0;
+        size_t most = 0;
+        for (int i = base; i < count && i < base + kMaxFills; ++i) {
+            const pet_hip_fill &f = fills[i];
+            const size_t total = f.outer * f.ch * f.inner;
+            if (total == 0)
+                continue;
+            if (!f.y)
+                return set_error(PET_HIP_ERR_INVALID, "fill %d has no output", i);
+            if (f.ch >= (1ull << 32) || f.inner >= (1ull << 32))
+                return set_error(PET_HIP_ERR_UNSUPPORTED, "fill %d is too large", i);
+            fb.y[nb] = f.y;
+            fb.bias[nb] = f.bias;
+            fb.ch[nb] = (unsigned)f.ch;
+            fb.inner[nb] = (unsigned)f.inner;
+            fb.total[nb] = total;
+            most = std::max(most, total);
+            ++nb;
+        }
+        if (nb == 0)
+            continue;
+        const unsigned gx = (unsigned)std::min<size_t>((most / 4 + 255) / 256 + 1, 1024);
+        hipLaunchKernelGGL(bias_fill_batch_kernel, dim3(gx, nb), dim3(256), 0, as_stream(stream),
+                           fb);
+        int rc = check_launch("bias_fill_batch_kernel");
+        if (rc)
+            return rc;
+    }
+    return PET_HIP_OK;
 }
 
 int pet_hip_bias_act(const float *x, const float *bias, float *y, size_t outer, size_t ch,

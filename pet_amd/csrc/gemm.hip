@@ -153,7 +153,15 @@ int launch_bmm_t(const GemmParams &p, int batch, bool vec, hipStream_t stream) {
 namespace {
 
 int bmm_common(int transA, int transB, int b, int m, int n, int k, const float *A, const float *B,
-               float *C, const float *bias, const float *res, int act, pet_hip_stream_t stream) {
+               float *C, const float *bias, const float *res, int act, pet_hip_stream_t stream,
+               unsigned flags = 0, int *dry = nullptr) {
+    if (flags & ~(unsigned)PET_HIP_CALL_Y_INITIALISED)
+        return set_error(PET_HIP_ERR_INVALID, "matmul takes PET_HIP_CALL_Y_INITIALISED only");
+    if (dry) {
+        *dry = 0;
+        A = B = reinterpret_cast<const float *>(uintptr_t(256));
+        C = reinterpret_cast<float *>(uintptr_t(512));
+    }
     if (b < 0 || m < 0 || n < 0 || k < 0)
         return set_error(PET_HIP_ERR_INVALID, "negative matmul dims");
     if (act < PET_HIP_ACT_NONE || act > PET_HIP_ACT_GELU)
@@ -165,6 +173,8 @@ int bmm_common(int transA, int transB, int b, int m, int n, int k, const float *
     if (res == C)
         return set_error(PET_HIP_ERR_INVALID, "the residual must not be the output buffer");
     const size_t cn = (size_t)b * m * n;
+    if (k == 0 && dry)
+        return PET_HIP_OK;
     if (k == 0) {
         // empty contraction: C = act(bias + residual)
         int rc = res ? pet_hip_memcpy_d2d(C, res, cn * sizeof(float), stream)
@@ -191,10 +201,13 @@ int bmm_common(int transA, int transB, int b, int m, int n, int k, const float *
     p.sC = (long long)m * n;
     p.act = res ? PET_HIP_ACT_NONE : act;
     if (!transA && !transB) {
-        int rc = bmm_as_grouped_1x1(A, B, C, bias, res, b, m, n, k, act, as_stream(stream));
+        int rc = bmm_as_grouped_1x1(A, B, C, bias, res, b, m, n, k, act, as_stream(stream), flags,
+                                    dry);
         if (rc >= 0)
             return rc;
     }
+    if (dry) // the general kernel never accumulates into C
+        return PET_HIP_OK;
     // the general kernel has no residual operand: add it, and apply the activation,
     // in two small launches afterwards
     auto finish = [&](int rc) {
@@ -236,6 +249,21 @@ int pet_hip_bmm_res_f32(int transA, int transB, int b, int m, int n, int k, cons
                         int act, pet_hip_stream_t stream) {
     PET_REQUIRE_INIT();
     return bmm_common(transA, transB, b, m, n, k, A, B, C, bias, residual, act, stream);
+}
+
+int pet_hip_bmm_ex_f32(int transA, int transB, int b, int m, int n, int k, const float *A,
+                       const float *B, float *C, const float *bias, const float *residual, int act,
+                       unsigned flags, pet_hip_stream_t stream) {
+    PET_REQUIRE_INIT();
+    return bmm_common(transA, transB, b, m, n, k, A, B, C, bias, residual, act, stream, flags);
+}
+
+int pet_hip_bmm_accumulates(int transA, int transB, int b, int m, int n, int k, int *yes) {
+    PET_REQUIRE_INIT();
+    if (!yes)
+        return set_error(PET_HIP_ERR_INVALID, "null result pointer");
+    return bmm_common(transA, transB, b, m, n, k, nullptr, nullptr, nullptr, nullptr, nullptr,
+                      PET_HIP_ACT_NONE, nullptr, 0, yes);
 }
 
 } // extern "C"

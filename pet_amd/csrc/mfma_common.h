@@ -245,8 +245,8 @@ inline int forced_tile() {
 
 // conv.hip: non-transposed batched matmul through the plane convolution kernel.
 int bmm_as_grouped_1x1(const float *A, const float *B, float *C, const float *bias,
-                       const float *res, int b, int m,
-                       int n, int k, int act, hipStream_t stream);
+                       const float *res, int b, int m, int n, int k, int act, hipStream_t stream,
+                       unsigned flags = 0, int *dry = nullptr);
 
 } // namespace mfma
 } // namespace pet

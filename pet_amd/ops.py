@@ -34,8 +34,9 @@ def conv_out_dim(i, k, p, s, d):
 
 
 def conv2d(x, w, ph, pw, sh=1, sw=1, dh=1, dw=1, bias=None, act="none", out=None,
-           residual=None):
-    """act(conv(x, w) + bias + residual); residual has the output's shape."""
+           residual=None, flags=0):
+    """act(conv(x, w) + bias + residual); residual has the output's shape. flags:
+    pet_hip_call_flags (abi.Y_INITIALISED, DEFER_RELU, X_RELU, RES_RELU)."""
     _chk(x, w, bias, out, residual)
     n, c, h, wd = x.shape
     f, cpg, r, s = w.shape
@@ -45,15 +46,47 @@ def conv2d(x, w, ph, pw, sh=1, sw=1, dh=1, dw=1, bias=None, act="none", out=None
     oh, ow = conv_out_dim(h, r, ph, sh, dh), conv_out_dim(wd, s, pw, sw, dw)
     if out is None:
         out = torch.empty((n, f, max(oh, 0), max(ow, 0)), device=x.device, dtype=torch.float32)
+    if residual is not None and tuple(residual.shape) != tuple(out.shape):
+        raise abi.PetHipError(1, "residual shape differs from the output's")
+    if flags:
+        abi.call("pet_hip_conv2d_ex_f32", _ptr(x), _ptr(w), _ptr(bias), _ptr(residual), _ptr(out),
+                 n, c, h, wd, f, r, s, ph, pw, sh, sw, dh, dw, groups, abi.ACT[act], flags,
+                 _stream())
+        return out
     if residual is not None:
-        if tuple(residual.shape) != tuple(out.shape):
-            raise abi.PetHipError(1, "residual shape differs from the output's")
         abi.call("pet_hip_conv2d_res_f32", _ptr(x), _ptr(w), _ptr(bias), _ptr(residual), _ptr(out),
                  n, c, h, wd, f, r, s, ph, pw, sh, sw, dh, dw, groups, abi.ACT[act], _stream())
         return out
     abi.call("pet_hip_conv2d_f32", _ptr(x), _ptr(w), _ptr(bias), _ptr(out), n, c, h, wd, f, r, s,
              ph, pw, sh, sw, dh, dw, groups, abi.ACT[act], _stream())
     return out
+
+
+def conv2d_accumulates(x_shape, w_shape, ph, pw, sh=1, sw=1, dh=1, dw=1):
+    """Whether conv2d on these shapes adds partial sums into its output with atomics."""
+    abi.init(torch.cuda.current_device())
+    n, c, h, wd = x_shape
+    f, cpg, r, s = w_shape
+    yes = ctypes.c_int(0)
+    abi.call("pet_hip_conv2d_accumulates", n, c, h, wd, f, r, s, ph, pw, sh, sw, dh, dw, c // cpg,
+             ctypes.byref(yes))
+    return bool(yes.value)
+
+
+def bmm_accumulates(b, m, n, k, transA=False, transB=False):
+    abi.init(torch.cuda.current_device())
+    yes = ctypes.c_int(0)
+    abi.call("pet_hip_bmm_accumulates", int(transA), int(transB), b, m, n, k, ctypes.byref(yes))
+    return bool(yes.value)
+
+
+def bias_fill_batch(items):
+    """items: (y, bias or None, outer, ch, inner) tuples; y[o][c][i] = bias[c], one launch."""
+    arr = (abi.Fill * max(1, len(items)))()
+    for i, (y, bias, outer, ch, inner) in enumerate(items):
+        _chk(y, bias)
+        arr[i] = abi.Fill(y.data_ptr(), 0 if bias is None else bias.data_ptr(), outer, ch, inner)
+    abi.call("pet_hip_bias_fill_batch", arr, len(items), _stream())
 
 
 class PackedFilters:
@@ -110,7 +143,8 @@ def conv3d(x, w, pad, stride=(1, 1, 1), dil=(1, 1, 1), bias=None, act="none", ou
     return out
 
 
-def matmul(A, B, transA=False, transB=False, bias=None, act="none", out=None, residual=None):
+def matmul(A, B, transA=False, transB=False, bias=None, act="none", out=None, residual=None,
+           flags=0):
     """MatmulOp on [b, ., .] tensors (MatmulOp::computeShape, operator.cc:717-726);
     with residual: act(A @ B + bias + residual)."""
     _chk(A, B, bias, out, residual)
@@ -123,9 +157,13 @@ def matmul(A, B, transA=False, transB=False, bias=None, act="none", out=None, re
         raise abi.PetHipError(1, "matmul shapes do not agree")
     if out is None:
         out = torch.empty((b, m, n), device=A.device, dtype=torch.float32)
+    if residual is not None and residual.numel() != out.numel():
+        raise abi.PetHipError(1, "residual size differs from the output's")
+    if flags:
+        abi.call("pet_hip_bmm_ex_f32", int(transA), int(transB), b, m, n, k, _ptr(A), _ptr(B),
+                 _ptr(out), _ptr(bias), _ptr(residual), abi.ACT[act], flags, _stream())
+        return out
     if residual is not None:
-        if residual.numel() != out.numel():
-            raise abi.PetHipError(1, "residual size differs from the output's")
         abi.call("pet_hip_bmm_res_f32", int(transA), int(transB), b, m, n, k, _ptr(A), _ptr(B),
                  _ptr(out), _ptr(bias), _ptr(residual), abi.ACT[act], _stream())
         return out

@@ -653,6 +653,71 @@ def test_eltwise_bit_exact(ops):
     assert got.tobytes() == oracle.eltwise("add", [r0, r1], r0.shape).tobytes()
 
 
+def test_cross_launch_fusion_flags(ops):
+    """The *_ex entry points a graph runtime uses: ReLU applied by the reader (x and
+    residual), outputs initialised by one batched fill, ReLU left out by a launch that
+    accumulates with atomics. Small integers: every sum is exact, so all forms agree
+    bit for bit whatever the order of the atomic adds."""
+    from pet_amd import abi
+    rng = np.random.default_rng(21)
+
+    def ints(shape, lo=-3, hi=4):
+        return rng.integers(lo, hi, shape).astype(np.float32)
+
+    # (x shape, w shape, pad, stride): split-K / stream-K shapes and plain ones, 3x3, 1x1, 7x7
+    cases = [((1, 64, 56, 56), (64, 64, 3, 3), 1, 1), ((1, 256, 14, 14), (256, 256, 3, 3), 1, 1),
+             ((4, 512, 32, 32), (64, 512, 3, 3), 1, 1), ((1, 64, 56, 56), (128, 64, 1, 1), 0, 2),
+             ((2, 3, 30, 30), (16, 3, 7, 7), 3, 2), ((1, 24, 9, 11), (8, 24, 3, 3), 1, 1)]
+    saw = set()
+    for xs, ws, pad, st in cases:
+        x, w, b = ints(xs), ints(ws), ints((ws[0],))
+        dx, dw_, db = dev(x), dev(w), dev(b)
+        acc = ops.conv2d_accumulates(xs, ws, pad, pad, st, st)
+        saw.add(acc)
+        plain = ops.conv2d(dx, dw_, pad, pad, st, st, bias=db, act="relu")
+        want = host(plain)
+        assert want.tobytes() == np.maximum(oracle.conv2d(x, w, pad, pad, st, st)
+                                            + b[None, :, None, None], 0).tobytes()
+        res = ints(want.shape)
+        dres = dev(res)
+        # reader-side ReLU on x and on the residual
+        got = ops.conv2d(dx, dw_, pad, pad, st, st, bias=db, act="relu", residual=dres,
+                         flags=abi.X_RELU | abi.RES_RELU)
+        ref = ops.conv2d(dev(np.maximum(x, 0)), dw_, pad, pad, st, st, bias=db, act="relu",
+                         residual=dev(np.maximum(res, 0)))
+        assert host(got).tobytes() == host(ref).tobytes(), (xs, ws)
+        # output initialised by the batched fill (two outputs in one launch)
+        y1, y2 = torch.empty_like(plain), torch.empty_like(plain)
+        ops.bias_fill_batch([(y1, db, want.shape[0], want.shape[1], want.shape[2] * want.shape[3]),
+                             (y2, None, want.shape[0], want.shape[1], want.shape[2] * want.shape[3])])
+        assert host(y1).tobytes() == np.broadcast_to(b[None, :, None, None], want.shape).tobytes()
+        assert not host(y2).any()
+        ops.conv2d(dx, dw_, pad, pad, st, st, bias=db, act="relu", out=y1, flags=abi.Y_INITIALISED)
+        assert host(y1).tobytes() == want.tobytes(), (xs, ws, acc)
+        # ReLU left to the readers: unapplied by an accumulating launch only
+        pre = host(ops.conv2d(dx, dw_, pad, pad, st, st, bias=db, act="relu", flags=abi.DEFER_RELU))
+        assert np.maximum(pre, 0).tobytes() == want.tobytes()
+        assert (pre.min() < 0) == acc, (xs, ws, acc)
+        # an initialised output cannot also take a residual when the launch accumulates
+        if acc:
+            with pytest.raises(Exception):
+                ops.conv2d(dx, dw_, pad, pad, st, st, bias=db, residual=dres, out=y1,
+                           flags=abi.Y_INITIALISED)
+    assert saw == {True, False}
+    with pytest.raises(Exception):
+        ops.conv2d(dx, dw_, pad, pad, st, st, act="tanh", flags=abi.DEFER_RELU)
+    with pytest.raises(Exception):
+        ops.conv2d(dx, dw_, pad, pad, st, st, flags=64)
+
+    for (bb, m, n, k) in [(1, 128, 768, 768), (3, 128, 768, 768), (12, 128, 64, 128), (1, 64, 48, 20)]:
+        A, B, bias = ints((bb, m, k)), ints((bb, k, n)), ints((n,))
+        want = host(ops.matmul(dev(A), dev(B), bias=dev(bias)))
+        y = torch.empty((bb, m, n), device="cuda")
+        ops.bias_fill_batch([(y, dev(bias), bb * m, n, 1)])
+        ops.matmul(dev(A), dev(B), bias=dev(bias), out=y, flags=abi.Y_INITIALISED)
+        assert host(y).tobytes() == want.tobytes(), (bb, m, n, k, ops.bmm_accumulates(bb, m, n, k))
+
+
 def test_pow_div_batchnorm(ops):
     """PowOp: bit-exact (the same chain of fp32 products as the CPU loop). Div:
     division proper, correctly rounded like numpy's. BatchNorm: 1e-5 relative
