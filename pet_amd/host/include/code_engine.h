@@ -27,11 +27,13 @@ class GraphExec {
     size_t numAliasedOps() const { return nAliasOps; }
     // Transposes that run as part of the transpose that follows them.
     size_t numFoldedOps() const { return nFoldedOps; }
+    // output initialisations of accumulating contractions, batched into the first launch
+    size_t numHoistedFills() const { return nHoistedFills; }
 
   private:
     friend class CodeEngine;
     pet_hip_graph_t graph = nullptr;
-    size_t nLaunchOps = 0, nAliasOps = 0, nFoldedOps = 0;
+    size_t nLaunchOps = 0, nAliasOps = 0, nFoldedOps = 0, nHoistedFills = 0;
 };
 
 class CodeEngine {

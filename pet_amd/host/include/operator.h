@@ -126,9 +126,13 @@ class Operator {
     // out = finalAct(op(inputs) + bias + residual), residual and out laid out like
     // the operator's output. The graph runtime uses it to run "contraction, Add,
     // activation" as one operator. PET_HIP_ERR_UNSUPPORTED elsewhere.
+    // flags: pet_hip_call_flags, what the graph runtime fuses across launches.
     virtual int launchFused(pet_hip_stream_t stream, const float *residual, ActType finalAct,
-                            float *out);
+                            float *out, unsigned flags = 0);
     virtual bool canTakeResidual() const { return false; }
+    // Contractions only: whether a launch adds partial sums into the output with
+    // atomics, i.e. starts by writing the bias into all of it.
+    virtual bool accumulates() const { return false; }
 
     virtual int numInputs() = 0;
     virtual int numOutputs() = 0;
@@ -190,7 +194,8 @@ class ConvOp : public Operator {
     double perf(PerfEngine *pe, int rounds = 200, int warmupRounds = 200) override;
     int launch(pet_hip_stream_t stream) override;
     int launchFused(pet_hip_stream_t stream, const float *residual, ActType finalAct,
-                    float *out) override;
+                    float *out, unsigned flags = 0) override;
+    bool accumulates() const override;
     bool canTakeResidual() const override { return act == None; }
     std::string toString() const override;
     int numInputs() override { return 2; }
@@ -242,7 +247,8 @@ class Conv3dOp : public Operator {
     double perf(PerfEngine *pe, int rounds = 200, int warmupRounds = 200) override;
     int launch(pet_hip_stream_t stream) override;
     int launchFused(pet_hip_stream_t stream, const float *residual, ActType finalAct,
-                    float *out) override;
+                    float *out, unsigned flags = 0) override;
+    bool accumulates() const override;
     bool canTakeResidual() const override { return act == None; }
     std::string toString() const override;
     int numInputs() override { return 2; }
@@ -285,7 +291,8 @@ class MatmulOp : public Operator {
     double perf(PerfEngine *pe, int rounds = 200, int warmupRounds = 200) override;
     int launch(pet_hip_stream_t stream) override;
     int launchFused(pet_hip_stream_t stream, const float *residual, ActType finalAct,
-                    float *out) override;
+                    float *out, unsigned flags = 0) override;
+    bool accumulates() const override;
     bool canTakeResidual() const override { return act == None; }
     std::string toString() const override;
     int numInputs() override { return 2; }

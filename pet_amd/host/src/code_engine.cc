@@ -173,6 +173,124 @@ FusedTails planFusedTails(const OpVec &order, const TensorVec &graphOutputs,
     return plan;
 }
 
+// What is fused across launches (pet_hip_call_flags):
+//  * a contraction whose launch adds partial sums into its output starts by writing the
+//    bias there; for the ones without a residual these initialisations are batched into
+//    one launch at the start of the graph (nothing else writes those buffers);
+//  * a convolution with ReLU whose result is only read by convolutions (as their input
+//    or as the residual of their fused tail) may leave the ReLU to those readers, which
+//    apply it on load: the activation launch that follows an accumulating launch
+//    goes away. ReLU applied twice changes nothing, so the readers need not know
+//    whether the producer accumulated.
+struct FillSpec {
+    Tensor *out, *bias;
+    size_t outer, ch, inner;
+};
+
+struct LaunchPlan {
+    std::map<const Operator *, unsigned> flags; // by contraction
+    std::vector<FillSpec> fills;
+    std::set<const Tensor *> preAct; // tensors that may hold values before their ReLU
+};
+
+bool isConvOp(const Operator *op) {
+    return op->getType() == Operator::Conv || op->getType() == Operator::Conv3d;
+}
+
+bool isContraction(const Operator *op) { return isConvOp(op) || op->getType() == Operator::Matmul; }
+
+Operator::ActType ownAct(Operator *op) {
+    if (auto c = dynamic_cast<ConvOp *>(op))
+        return c->getAct();
+    if (auto c = dynamic_cast<Conv3dOp *>(op))
+        return c->getAct();
+    if (auto m = dynamic_cast<MatmulOp *>(op))
+        return m->getAct();
+    return Operator::None;
+}
+
+Tensor *ownBias(Operator *op) {
+    if (auto c = dynamic_cast<ConvOp *>(op))
+        return c->getBias();
+    if (auto c = dynamic_cast<Conv3dOp *>(op))
+        return c->getBias();
+    if (auto m = dynamic_cast<MatmulOp *>(op))
+        return m->getBias();
+    return nullptr;
+}
+
+LaunchPlan planLaunchFlags(const OpVec &order, const TensorVec &graphOutputs,
+                           const std::set<const Operator *> &skipped,
+                           const std::set<const Operator *> &folded, const FusedTails &tails,
+                           const std::function<bool(const Tensor *)> &ownStorage) {
+    LaunchPlan plan;
+    static const bool off = getenv("PET_HOST_NO_LAUNCH_FUSION") != nullptr;
+    if (off)
+        return plan;
+    std::set<const Tensor *> outs(graphOutputs.begin(), graphOutputs.end());
+    struct Eff {
+        Operator *c;
+        Tensor *out;
+        Operator::ActType act;
+        bool hasRes;
+    };
+    std::vector<Eff> effs;
+    for (auto op : order) {
+        if (skipped.count(op) || folded.count(op) || weightOnly(op))
+            continue;
+        auto tail = tails.atAdd.find(op);
+        if (tail != tails.atAdd.end())
+            effs.push_back({tail->second.contraction, tail->second.out, tail->second.act, true});
+        else if (isContraction(op) && !tails.absorbed.count(op))
+            effs.push_back({op, op->getOutputs()[0], ownAct(op), false});
+    }
+    for (auto &e : effs) {
+        if (e.hasRes || !ownStorage(e.out) || !e.c->accumulates())
+            continue;
+        const Dim &d = e.out->getDims();
+        FillSpec f{e.out, ownBias(e.c), 0, 0, 0};
+        if (isConvOp(e.c)) {
+            f.outer = (size_t)d[0];
+            f.ch = (size_t)d[1];
+            f.inner = e.out->size() / (f.outer * f.ch);
+        } else { // matmul: the bias runs along the last dim
+            f.ch = (size_t)d.back();
+            f.outer = e.out->size() / f.ch;
+            f.inner = 1;
+        }
+        plan.fills.push_back(f);
+        plan.flags[e.c] |= PET_HIP_CALL_Y_INITIALISED;
+    }
+    for (auto &e : effs) {
+        if (!isConvOp(e.c) || e.act != Operator::Relu || outs.count(e.out) || !ownStorage(e.out))
+            continue;
+        const OpVec &users = e.out->getInputOf();
+        std::map<const Operator *, unsigned> want;
+        bool ok = !users.empty();
+        for (auto u : users) {
+            auto tail = tails.atAdd.find(u);
+            if (skipped.count(u) || folded.count(u) || weightOnly(u)) {
+                ok = false;
+            } else if (isConvOp(u) && u->getInputs()[0] == e.out && u->getInputs()[1] != e.out) {
+                want[u] |= PET_HIP_CALL_X_RELU;
+            } else if (tail != tails.atAdd.end() && tail->second.residual == e.out &&
+                       isConvOp(tail->second.contraction) &&
+                       tail->second.contraction->getInputs()[1] != e.out) {
+                want[tail->second.contraction] |= PET_HIP_CALL_RES_RELU;
+            } else {
+                ok = false;
+            }
+        }
+        if (!ok)
+            continue;
+        for (auto &w : want)
+            plan.flags[w.first] |= w.second;
+        plan.flags[e.c] |= PET_HIP_CALL_DEFER_RELU;
+        plan.preAct.insert(e.out);
+    }
+    return plan;
+}
+
 // Micro-ops of a row of transposes, lowered on the first one's input.
 bool lowerChain(const std::vector<TransposeOp *> &row, TransProgram &prog) {
     std::vector<std::shared_ptr<TransBasic>> all;
@@ -288,13 +406,22 @@ std::unique_ptr<GraphExec> CodeEngine::instantiate(std::shared_ptr<SubGraph> &gr
                                       [](const FusedTail &f) {
                                           return f.residual->devicePtr() != f.out->devicePtr();
                                       });
+    LaunchPlan lp = planLaunchFlags(order, graph->getOutputs(), plan.skipped, rows.folded, tails,
+                                    [](const Tensor *) { return true; });
+    auto flagsOf = [&](const Operator *op) {
+        auto it = lp.flags.find(op);
+        return it == lp.flags.end() ? 0u : it->second;
+    };
     auto launchOp = [&](Operator *op, pet_hip_stream_t st) -> int {
         auto tail = tails.atAdd.find(op);
         if (tail != tails.atAdd.end()) {
             const FusedTail &f = tail->second;
             return f.contraction->launchFused(st, f.residual->devicePtr(), f.act,
-                                              f.out->devicePtr());
+                                              f.out->devicePtr(), flagsOf(f.contraction));
         }
+        if (flagsOf(op))
+            return op->launchFused(st, nullptr, ownAct(op), op->getOutputs()[0]->devicePtr(),
+                                   flagsOf(op));
         auto it = rows.chains.find(op);
         return it == rows.chains.end() ? op->launch(st) : launchChain(it->second, st);
     };
@@ -321,7 +448,18 @@ std::unique_ptr<GraphExec> CodeEngine::instantiate(std::shared_ptr<SubGraph> &gr
     if (!petOk(pet_hip_graph_begin_capture(s), "pet_hip_graph_begin_capture"))
         return nullptr;
     bool ok = true;
+    if (!lp.fills.empty()) {
+        std::vector<pet_hip_fill> fills;
+        for (auto &f : lp.fills)
+            fills.push_back({f.out->devicePtr(), f.bias ? f.bias->devicePtr() : nullptr, f.outer,
+                             f.ch, f.inner});
+        ok = petOk(pet_hip_bias_fill_batch(fills.data(), (int)fills.size(), s),
+                   "pet_hip_bias_fill_batch");
+        exec->nHoistedFills = fills.size();
+    }
     for (auto op : order) {
+        if (!ok)
+            break;
         if (plan.skipped.count(op)) {
             exec->nAliasOps++;
             continue;
@@ -355,7 +493,7 @@ std::unique_ptr<GraphExec> CodeEngine::instantiate(std::shared_ptr<SubGraph> &gr
             auto tail = tails.atAdd.find(prod);
             if (tail != tails.atAdd.end() && tail->second.out != t)
                 inside = true;
-            if (inside)
+            if (inside || lp.preAct.count(t)) // not there, or there without its ReLU
                 continue;
             t->deviceWritten();
             t->setComputed();
@@ -493,6 +631,12 @@ std::string CodeEngine::genCode(std::shared_ptr<SubGraph> &graph) {
     FusedTails tails = planFusedTails(order, graph->getOutputs(), skipped, [&](const FusedTail &f) {
         return !viewOf.count(f.residual) && !viewOf.count(f.out);
     });
+    LaunchPlan lp = planLaunchFlags(order, graph->getOutputs(), skipped, rows.folded, tails,
+                                    [](const Tensor *) { return true; });
+    auto flagsOf = [&](const Operator *op) {
+        auto it = lp.flags.find(op);
+        return it == lp.flags.end() ? 0u : it->second;
+    };
     // set while a contraction is emitted in place of the Add that follows it
     const FusedTail *tail = nullptr;
     std::function<bool(Operator *)> emitOp = [&](Operator *op) -> bool {
@@ -511,34 +655,41 @@ std::string CodeEngine::genCode(std::shared_ptr<SubGraph> &graph) {
         }
         if (auto conv = dynamic_cast<ConvOp *>(op)) {
             auto d = op->getInputs()[0]->getDims(), w = op->getInputs()[1]->getDims();
-            c << (tail ? "pet_hip_conv2d_res_f32(" : "pet_hip_conv2d_f32(") << in(0) << ", " << in(1)
-              << ", " << nullable(e, conv->getBias()) << ", " << res << out(0) << ", " << d[0]
-              << ", " << d[1]
-              << ", " << d[2] << ", " << d[3] << ", " << w[0] << ", " << w[2] << ", " << w[3]
+            const unsigned fl = flagsOf(op);
+            c << (fl     ? "pet_hip_conv2d_ex_f32("
+                  : tail ? "pet_hip_conv2d_res_f32("
+                         : "pet_hip_conv2d_f32(")
+              << in(0) << ", " << in(1) << ", " << nullable(e, conv->getBias()) << ", "
+              << (fl && !tail ? std::string("nullptr, ") : res) << out(0) << ", " << d[0] << ", "
+              << d[1] << ", " << d[2] << ", " << d[3] << ", " << w[0] << ", " << w[2] << ", " << w[3]
               << ", " << conv->getPh() << ", " << conv->getPw() << ", " << conv->getSh() << ", "
               << conv->getSw() << ", " << conv->getDh() << ", " << conv->getDw() << ", "
-              << d[1] / w[1] << ", " << actOf(conv->getAct()) << ", s)";
+              << d[1] / w[1] << ", " << actOf(conv->getAct()) << ", "
+              << (fl ? std::to_string(fl) + "u, " : std::string()) << "s)";
         } else if (auto c3 = dynamic_cast<Conv3dOp *>(op)) {
             auto d = op->getInputs()[0]->getDims(), w = op->getInputs()[1]->getDims();
             // filters with a kt-major copy (made before capture, below) use it
             const bool pk = packedName.count(op) != 0;
             const std::string filt =
                 pk ? packedName[op] + "_ok ? " + packedName[op] + " : " + in(1) : in(1);
-            if (tail)
-                c << "pet_hip_conv3d_res_f32(" << in(0) << ", " << filt << ", "
-                  << (pk ? packedName[op] + "_ok" : std::string("0")) << ", ";
+            const unsigned fl = flagsOf(op);
+            if (tail || fl)
+                c << (fl ? "pet_hip_conv3d_ex_f32(" : "pet_hip_conv3d_res_f32(") << in(0) << ", "
+                  << filt << ", " << (pk ? packedName[op] + "_ok" : std::string("0")) << ", ";
             else if (pk)
                 c << "(" << packedName[op] << "_ok ? pet_hip_conv3d_packed_f32 : "
                   << "pet_hip_conv3d_f32)(" << in(0) << ", " << filt << ", ";
             else
                 c << "pet_hip_conv3d_f32(" << in(0) << ", " << in(1) << ", ";
-            c << nullable(e, c3->getBias()) << ", " << res << out(0);
+            c << nullable(e, c3->getBias()) << ", " << (fl && !tail ? std::string("nullptr, ") : res)
+              << out(0);
             for (int v : {d[0], d[1], d[2], d[3], d[4], w[0], w[2], w[3], w[4]})
                 c << ", " << v;
             for (const Dim *v : {&c3->getPad(), &c3->getStride(), &c3->getDilation()})
                 for (int x : *v)
                     c << ", " << x;
-            c << ", " << d[1] / w[1] << ", " << actOf(c3->getAct()) << ", s)";
+            c << ", " << d[1] / w[1] << ", " << actOf(c3->getAct()) << ", "
+              << (fl ? std::to_string(fl) + "u, " : std::string()) << "s)";
         } else if (auto ln = dynamic_cast<LayerNormOp *>(op)) {
             size_t cols = (size_t)op->getInputs()[0]->getDims().back();
             c << "pet_hip_layernorm(" << in(0) << ", " << nullable(e, ln->getGamma()) << ", "
@@ -549,11 +700,16 @@ std::string CodeEngine::genCode(std::shared_ptr<SubGraph> &graph) {
             bool ta, tb;
             int b, m, n, k;
             std::tie(ta, tb, b, m, n, k) = mm->getArgs();
-            c << (tail ? "pet_hip_bmm_res_f32(" : "pet_hip_bmm_f32(") << ta << ", " << tb << ", " << b
-              << ", " << m << ", " << n << ", " << k << ", " << in(0) << ", " << in(1) << ", "
-              << out(0) << ", " << nullable(e, mm->getBias()) << ", "
-              << (tail ? e.name(tail->residual) + ", " : std::string()) << actOf(mm->getAct())
-              << ", s)";
+            const unsigned fl = flagsOf(op);
+            c << (fl     ? "pet_hip_bmm_ex_f32("
+                  : tail ? "pet_hip_bmm_res_f32("
+                         : "pet_hip_bmm_f32(")
+              << ta << ", " << tb << ", " << b << ", " << m << ", " << n << ", " << k << ", "
+              << in(0) << ", " << in(1) << ", " << out(0) << ", " << nullable(e, mm->getBias())
+              << ", "
+              << (tail ? e.name(tail->residual) + ", " : fl ? std::string("nullptr, ") : std::string())
+              << actOf(mm->getAct()) << ", " << (fl ? std::to_string(fl) + "u, " : std::string())
+              << "s)";
         } else if (auto tr = dynamic_cast<TransposeOp *>(op)) {
             TransProgram prog;
             std::vector<TransposeOp *> row = {tr};
@@ -717,6 +873,19 @@ std::string CodeEngine::genCode(std::shared_ptr<SubGraph> &graph) {
     e.line("    CHECK(pet_hip_stream_sync(s));");
     e.line("    // the rest is captured once and replayed as a HIP graph");
     e.line("    CHECK(pet_hip_graph_begin_capture(s));");
+    if (!lp.fills.empty()) {
+        e.line("    // outputs that accumulating contractions add into: their bias, in one launch");
+        std::string l = "    const pet_hip_fill fills[] = {";
+        for (size_t i = 0; i < lp.fills.size(); ++i) {
+            const FillSpec &f = lp.fills[i];
+            l += std::string(i ? ", " : "") + "{" + e.name(f.out) + ", " + nullable(e, f.bias) + ", " +
+                 std::to_string(f.outer) + ", " + std::to_string(f.ch) + ", " +
+                 std::to_string(f.inner) + "}";
+        }
+        e.line(l + "};");
+        e.line("    CHECK(pet_hip_bias_fill_batch(fills, " + std::to_string(lp.fills.size()) +
+               ", s));");
+    }
     for (auto op : order)
         if (!weightOnly(op) && !skipped.count(op) && !rows.folded.count(op) &&
             !tails.absorbed.count(op) && !emitOp(op))

@@ -64,7 +64,7 @@ Tensor *Operator::compute() {
     return outputs[0];
 }
 
-int Operator::launchFused(pet_hip_stream_t, const float *, ActType, float *) {
+int Operator::launchFused(pet_hip_stream_t, const float *, ActType, float *, unsigned) {
     return PET_HIP_ERR_UNSUPPORTED;
 }
 
@@ -308,15 +308,25 @@ int ConvOp::launch(pet_hip_stream_t stream) {
 }
 
 int ConvOp::launchFused(pet_hip_stream_t stream, const float *residual, ActType finalAct,
-                        float *out) {
+                        float *out, unsigned flags) {
     auto in = inputs[0]->getDims(), wt = inputs[1]->getDims();
     int groups = in[1] / wt[1];
-    if (groups <= 0 || wt[0] % groups != 0 || act != None)
+    if (groups <= 0 || wt[0] % groups != 0 || (residual != nullptr && act != None))
         return PET_HIP_ERR_INVALID;
-    return pet_hip_conv2d_res_f32(inputs[0]->devicePtr(), inputs[1]->devicePtr(),
-                                  bias ? bias->devicePtr() : nullptr, residual, out, in[0], in[1],
-                                  in[2], in[3], wt[0], wt[2], wt[3], ph, pw, sh, sw, dh, dw, groups,
-                                  (int)finalAct, stream);
+    return pet_hip_conv2d_ex_f32(inputs[0]->devicePtr(), inputs[1]->devicePtr(),
+                                 bias ? bias->devicePtr() : nullptr, residual, out, in[0], in[1],
+                                 in[2], in[3], wt[0], wt[2], wt[3], ph, pw, sh, sw, dh, dw, groups,
+                                 (int)finalAct, flags, stream);
+}
+
+bool ConvOp::accumulates() const {
+    auto in = inputs[0]->getDims(), wt = inputs[1]->getDims();
+    int groups = wt[1] > 0 ? in[1] / wt[1] : 0, yes = 0;
+    if (groups <= 0)
+        return false;
+    return pet_hip_conv2d_accumulates(in[0], in[1], in[2], in[3], wt[0], wt[2], wt[3], ph, pw, sh,
+                                      sw, dh, dw, groups, &yes) == PET_HIP_OK &&
+           yes != 0;
 }
 
 double ConvOp::perf(PerfEngine *pe, int rounds, int warmupRounds) {
@@ -462,18 +472,30 @@ int Conv3dOp::launch(pet_hip_stream_t stream) {
 }
 
 int Conv3dOp::launchFused(pet_hip_stream_t stream, const float *residual, ActType finalAct,
-                          float *out) {
+                          float *out, unsigned flags) {
     auto in = inputs[0]->getDims(), wt = inputs[1]->getDims();
     int groups = in[1] / wt[1];
-    if (groups <= 0 || wt[0] % groups != 0 || act != None)
+    if (groups <= 0 || wt[0] % groups != 0 || (residual != nullptr && act != None))
         return PET_HIP_ERR_INVALID;
     const bool usePacked = usesPackedFilters();
-    return pet_hip_conv3d_res_f32(inputs[0]->devicePtr(), usePacked ? packed : inputs[1]->devicePtr(),
-                                  usePacked, bias ? bias->devicePtr() : nullptr, residual, out,
-                                  in[0], in[1], in[2], in[3], in[4], wt[0], wt[2], wt[3], wt[4],
-                                  pad[0], pad[1], pad[2], stride[0], stride[1], stride[2],
-                                  dilation[0], dilation[1], dilation[2], groups, (int)finalAct,
-                                  stream);
+    return pet_hip_conv3d_ex_f32(inputs[0]->devicePtr(), usePacked ? packed : inputs[1]->devicePtr(),
+                                 usePacked, bias ? bias->devicePtr() : nullptr, residual, out,
+                                 in[0], in[1], in[2], in[3], in[4], wt[0], wt[2], wt[3], wt[4],
+                                 pad[0], pad[1], pad[2], stride[0], stride[1], stride[2],
+                                 dilation[0], dilation[1], dilation[2], groups, (int)finalAct,
+                                 flags, stream);
+}
+
+bool Conv3dOp::accumulates() const {
+    auto in = inputs[0]->getDims(), wt = inputs[1]->getDims();
+    int groups = wt[1] > 0 ? in[1] / wt[1] : 0, yes = 0;
+    if (groups <= 0)
+        return false;
+    return pet_hip_conv3d_accumulates(in[0], in[1], in[2], in[3], in[4], wt[0], wt[2], wt[3],
+                                      wt[4], pad[0], pad[1], pad[2], stride[0], stride[1],
+                                      stride[2], dilation[0], dilation[1], dilation[2], groups,
+                                      usesPackedFilters(), &yes) == PET_HIP_OK &&
+           yes != 0;
 }
 
 double Conv3dOp::perf(PerfEngine *, int rounds, int warmupRounds) {
@@ -571,15 +593,22 @@ int MatmulOp::launch(pet_hip_stream_t stream) {
 }
 
 int MatmulOp::launchFused(pet_hip_stream_t stream, const float *residual, ActType finalAct,
-                          float *out) {
-    if (act != None)
+                          float *out, unsigned flags) {
+    if (residual != nullptr && act != None)
         return PET_HIP_ERR_INVALID;
     bool ta, tb;
     int b, m, n, k;
     std::tie(ta, tb, b, m, n, k) = getArgs();
-    return pet_hip_bmm_res_f32(ta, tb, b, m, n, k, inputs[0]->devicePtr(), inputs[1]->devicePtr(),
-                               out, bias ? bias->devicePtr() : nullptr, residual, (int)finalAct,
-                               stream);
+    return pet_hip_bmm_ex_f32(ta, tb, b, m, n, k, inputs[0]->devicePtr(), inputs[1]->devicePtr(),
+                              out, bias ? bias->devicePtr() : nullptr, residual, (int)finalAct,
+                              flags, stream);
+}
+
+bool MatmulOp::accumulates() const {
+    bool ta, tb;
+    int b, m, n, k, yes = 0;
+    std::tie(ta, tb, b, m, n, k) = getArgs();
+    return pet_hip_bmm_accumulates(ta, tb, b, m, n, k, &yes) == PET_HIP_OK && yes != 0;
 }
 
 double MatmulOp::perf(PerfEngine *pe, int rounds, int warmupRounds) {

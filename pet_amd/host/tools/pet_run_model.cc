@@ -122,9 +122,11 @@ int main(int argc, char **argv) {
     if (!emit.empty() && ce.genCode(sg, emit) != 0)
         return 1;
     std::printf("{\"model\": \"%s\", \"ms\": %.5f, \"gflop\": %.3f, \"tflops\": %.2f, "
-                "\"operators\": %zu, \"kernels\": %zu, \"aliased\": %zu, \"folded\": %zu",
+                "\"operators\": %zu, \"kernels\": %zu, \"aliased\": %zu, \"folded\": %zu, "
+                "\"hoisted_fills\": %zu",
                 m.name.c_str(), ms, m.gflop, m.gflop / ms, sg->getOperators().size(),
-                exec->numKernelOps(), exec->numAliasedOps(), exec->numFoldedOps());
+                exec->numKernelOps(), exec->numAliasedOps(), exec->numFoldedOps(),
+                exec->numHoistedFills());
     if (check)
         std::printf(", \"max_abs_diff_vs_eager\": %.3g, \"max_abs_eager\": %.3g", maxDiff, maxRef);
     std::printf("}\n");

@@ -496,6 +496,71 @@ static bool test_split_ratio_and_eltwise() {
     return true;
 }
 
+// What the graph runtime fuses across launches, on two residual blocks whose
+// convolutions split K (64 channels on 28x28): ReLU left to the convolutions that
+// read a tensor (as input and as residual), output initialisations batched into one
+// launch. Signed data, so a ReLU applied in the wrong place, or not at all, shows.
+static bool test_launch_fusion_block() {
+    Graph g;
+    auto x = g.tensor({1, 64, 28, 28});
+    Tensor *w[4];
+    for (auto &t : w)
+        t = g.tensor({64, 64, 3, 3});
+    auto c1 = static_cast<ConvOp *>(g.conv(x, w[0], 1, 1));
+    c1->setAct(Operator::Relu);
+    auto c2 = g.conv(c1->getOutputs()[0], w[1], 1, 1);
+    auto r = g.relu(g.add({c2->getOutputs()[0], x})->getOutputs()[0])->getOutputs()[0];
+    auto c3 = static_cast<ConvOp *>(g.conv(r, w[2], 1, 1));
+    c3->setAct(Operator::Relu);
+    auto c4 = g.conv(c3->getOutputs()[0], w[3], 1, 1);
+    g.relu(g.add({c4->getOutputs()[0], r})->getOutputs()[0]);
+    g.updateConnection();
+    auto s1 = std::make_shared<SubGraph>(g.getOperators());
+    auto s2 = std::make_shared<SubGraph>(g.getOperators());
+    unsigned state = 777;
+    for (size_t i = 0; i < s1->getInputs().size(); ++i) {
+        Tensor *t = s1->getInputs()[i];
+        std::vector<float> v(t->size());
+        const float scale = t->getDims()[0] == 1 ? 0.5f : 0.03125f; // image : filters
+        for (auto &e : v) {
+            state = state * 1664525u + 1013904223u;
+            e = scale * (float)((int)((state >> 16) % 9u) - 4);
+        }
+        t->setData(v.data());
+        s2->getInputs()[i]->setData(v.data());
+    }
+    EXPECT(s1->compute());
+    CodeEngine ce;
+    auto exec = ce.instantiate(s2);
+    EXPECT(exec != nullptr);
+    // c1 and c3 have no residual: their initialisations are batched; the four launches
+    // left are the four convolutions (both Adds and all ReLUs ride in them)
+    EXPECT(exec->numHoistedFills() == 2);
+    EXPECT(exec->numKernelOps() == 4);
+    Tensor *o1 = s1->getOutputs()[0], *o2 = s2->getOutputs()[0];
+    EXPECT(s1->getOutputs().size() == 1 && s2->getOutputs().size() == 1);
+    for (int rep = 0; rep < 3; ++rep) {
+        EXPECT(exec->launch() && exec->sync());
+        o2->deviceWritten();
+        const float *a = o1->getDataPtr(), *b = o2->getDataPtr();
+        double worst = 0, big = 0;
+        bool negative = false;
+        for (size_t i = 0; i < o1->size(); ++i) {
+            worst = std::max(worst, (double)std::fabs(a[i] - b[i]));
+            big = std::max(big, (double)std::fabs(a[i]));
+            negative = negative || b[i] < 0;
+        }
+        EXPECT(!negative && big > 1.0 && worst <= 1e-5 * big);
+    }
+    std::string code = ce.genCode(s2);
+    EXPECT(code.find("pet_hip_bias_fill_batch(fills, 2, s)") != std::string::npos);
+    // c1: initialised + ReLU deferred (3); c2's tail: reads with ReLU, defers its own (6);
+    // c3: initialised, reads with ReLU, defers (7); c4's tail: input and residual with ReLU (12)
+    for (const char *f : {", 3u, s)", ", 6u, s)", ", 7u, s)", ", 12u, s)"})
+        EXPECT(code.find(f) != std::string::npos);
+    return true;
+}
+
 // BatchNormOp / PowOp / DivOp (src/Graph/operator.cc:2660-2681, 3330-3343, 3246-3262;
 // Div divides here, see the class): operator by operator against the formulas on
 // the host, then the same graph through the graph runtime and the emitter.
@@ -699,6 +764,7 @@ int main(int argc, char **argv) {
         {"emit_program", test_emit_program},
         {"perf_engine_memo", test_perf_engine_memo},
         {"split_ratio_and_eltwise", test_split_ratio_and_eltwise},
+        {"launch_fusion_block", test_launch_fusion_block},
         {"batchnorm_pow_div", test_batchnorm_pow_div},
         {"gather_reduce_mean", test_gather_reduce_mean},
         {"conv_merge_programs", test_conv_merge_programs},

@@ -19,7 +19,7 @@ CASES = ["conv_vs_oracle", "conv_invalid_groups", "transpose_n2h_h2n", "batch_ge
          "dilated_space_to_batch_program", "code_engine_graph_runtime", "perf_engine_memo",
          "split_ratio_and_eltwise", "conv_merge_programs", "conv3d_prepacked_graph",
          "random_graphs_replay_equals_eager", "batchnorm_pow_div",
-         "gather_reduce_mean"]
+         "gather_reduce_mean", "launch_fusion_block"]
 
 
 def test_host_library_is_built_and_exports_the_operator_classes():
@@ -342,9 +342,11 @@ def test_emitted_model_program_compiles_and_agrees_with_the_runtime(model, tmp_p
     rec = json.loads(res.stdout.strip().splitlines()[-1])
     text = src.read_text()
     if model != "bert":
-        assert "_res_f32(" in text               # a block tail became one call
+        # a block tail became one call, with the ReLU of what it reads applied on load
+        assert re.search(r"pet_hip_conv[23]d_ex_f32\([^;]*, (1[0-5]|[4-9])u, s\)", text)
     else:
         assert "pet_hip_bmm_res_f32(" in text
+    assert "pet_hip_bias_fill_batch(fills, " in text  # initialisations batched up front
     if model == "resnet3d18":
         assert "pet_hip_conv3d_pack_filters(" in text
     exe = tmp_path / "net"
