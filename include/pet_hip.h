@@ -58,8 +58,9 @@ typedef enum pet_hip_eltwise_op {
  * launches. No counterpart upstream, where cuDNN / cuBLAS calls stand alone. */
 typedef enum pet_hip_call_flags {
     /* y already holds bias (or zeros): a launch that accumulates into y (see the
-     * *_accumulates queries) skips its initialising launch; bias must still be passed.
-     * Not together with a residual. Other launches overwrite y as usual. */
+     * *_accumulates queries) skips its initialising launch (a residual, if any, is
+     * added along with the partial sums); bias must still be passed. Other launches
+     * overwrite y as usual. */
     PET_HIP_CALL_Y_INITIALISED = 1,
     /* act is ReLU and every reader of y applies it on load (the two flags below): a
      * launch that accumulates into y leaves the ReLU out; others apply it as usual,

@@ -53,6 +53,8 @@ struct ConvParams {
     int y_init;     // y already holds bias (or 0): a split launch does not initialise it
     int defer_relu; // a split launch leaves its ReLU to the readers of y
     int *dry_atomic; // not null: report whether the launch would accumulate into y, launch nothing
+    int res_first;   // accumulating launch into an initialised y: the workgroup that holds a
+                     // tile's first K step adds the residual along with its partial sums
     FastDiv fd_krs, fd_rs, fd_s;     // k -> (c, kt, r, s)
     FastDiv fd_opix, fd_ohw, fd_ow;  // pixel -> (n, ot, oh, ow)
 };
@@ -791,13 +793,20 @@ __global__ __launch_bounds__(Cfg::NT) void conv_plane_kernel(ConvParams p) {
         if (atomic) {
             // the output was initialised with the bias by a launch before this one;
             // the activation runs in a launch after it
+            const bool add_res = p.res_first && it_begin == 0;
 #pragma unroll
             for (int tm = 0; tm < TM; ++tm)
 #pragma unroll
                 for (int r = 0; r < 16; ++r) {
                     int f = m0 + wm0 + tm * 32 + (r / 4) * 8 + hk * 4 + (r % 4);
-                    if (f < p.M)
-                        unsafeAtomicAdd(yb + (unsigned)f * (unsigned)p.OPIX, acc[tm][tn][r]);
+                    if (f < p.M) {
+                        float v = acc[tm][tn][r];
+                        if (add_res) {
+                            const float rv = rb[(unsigned)f * (unsigned)p.OPIX];
+                            v += p.res_relu ? fmaxf(rv, 0.f) : rv;
+                        }
+                        unsafeAtomicAdd(yb + (unsigned)f * (unsigned)p.OPIX, v);
+                    }
                 }
         } else {
 #pragma unroll
@@ -1014,10 +1023,7 @@ int launch_plane_cfg(ConvParams p, hipStream_t stream) {
         *p.dry_atomic = p.atomic_out;
         return PET_HIP_OK;
     }
-    if (p.atomic_out && p.y_init && p.res)
-        return set_error(PET_HIP_ERR_INVALID,
-                         "an initialised output cannot take a residual: fold it into the "
-                         "initialisation or leave the flag out");
+    p.res_first = p.atomic_out && p.y_init && p.res != nullptr;
     if (p.atomic_out && !p.y_init) {
         const size_t total = (size_t)p.NPIX * p.F;
         unsigned igrid = (unsigned)std::min<size_t>((total + 255) / 256, 4096);

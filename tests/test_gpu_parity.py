@@ -698,11 +698,13 @@ def test_cross_launch_fusion_flags(ops):
         pre = host(ops.conv2d(dx, dw_, pad, pad, st, st, bias=db, act="relu", flags=abi.DEFER_RELU))
         assert np.maximum(pre, 0).tobytes() == want.tobytes()
         assert (pre.min() < 0) == acc, (xs, ws, acc)
-        # an initialised output cannot also take a residual when the launch accumulates
-        if acc:
-            with pytest.raises(Exception):
-                ops.conv2d(dx, dw_, pad, pad, st, st, bias=db, residual=dres, out=y1,
-                           flags=abi.Y_INITIALISED)
+        # initialised output and a residual: added once, with the partial sums
+        ops.bias_fill_batch([(y1, db, want.shape[0], want.shape[1], want.shape[2] * want.shape[3])])
+        ops.conv2d(dx, dw_, pad, pad, st, st, bias=db, act="relu", residual=dres, out=y1,
+                   flags=abi.Y_INITIALISED | abi.RES_RELU)
+        ref = ops.conv2d(dx, dw_, pad, pad, st, st, bias=db, act="relu",
+                         residual=dev(np.maximum(res, 0)))
+        assert host(y1).tobytes() == host(ref).tobytes(), (xs, ws, acc)
     assert saw == {True, False}
     with pytest.raises(Exception):
         ops.conv2d(dx, dw_, pad, pad, st, st, act="tanh", flags=abi.DEFER_RELU)
@@ -716,6 +718,12 @@ def test_cross_launch_fusion_flags(ops):
         ops.bias_fill_batch([(y, dev(bias), bb * m, n, 1)])
         ops.matmul(dev(A), dev(B), bias=dev(bias), out=y, flags=abi.Y_INITIALISED)
         assert host(y).tobytes() == want.tobytes(), (bb, m, n, k, ops.bmm_accumulates(bb, m, n, k))
+        res = ints((bb, m, n))
+        want_r = host(ops.matmul(dev(A), dev(B), bias=dev(bias), residual=dev(res)))
+        ops.bias_fill_batch([(y, dev(bias), bb * m, n, 1)])
+        ops.matmul(dev(A), dev(B), bias=dev(bias), residual=dev(res), out=y,
+                   flags=abi.Y_INITIALISED)
+        assert host(y).tobytes() == want_r.tobytes(), (bb, m, n, k)
 
 
 def test_pow_div_batchnorm(ops):
