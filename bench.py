@@ -307,6 +307,85 @@ def main():
                 entry["pet_TFLOP/s"] = gflop / entry["pet_ms"]
             other[name] = entry
 
+    # ---- every distinct contraction of the other configurations by itself: 20 launches
+    # captured into one graph (so that Python's call overhead stays out), replayed, with
+    # the roofline it sits under: min(fp32 MFMA peak, arithmetic intensity x HBM peak)
+    cfg_layers = []
+    if not args.no_configs:
+        def time_in_graph(fn, reps=20):
+            with torch.cuda.stream(stream):
+                for _ in range(3):
+                    fn()
+                stream.synchronize()
+                abi.call("pet_hip_graph_begin_capture", sp)
+                try:
+                    for _ in range(reps):
+                        fn()
+                finally:
+                    gh = ctypes.c_void_p(0)
+                    abi.call("pet_hip_graph_end_capture", sp, ctypes.byref(gh))
+            ms = time_graph(gh, 5, 2) / reps
+            abi.call("pet_hip_graph_destroy", gh)
+            return ms
+
+        def layer_line(name, ms, flop, nbytes):
+            tf = flop / ms / 1e9
+            roof = min(MFMA_FP32_PEAK_TFLOPS, flop / nbytes * HBM_PEAK_GBS / 1e3)
+            cfg_layers.append({"layer": name, "ms": ms, "TFLOP/s": tf, "GFLOP": flop / 1e9,
+                           "roof_TFLOP/s": roof, "frac_roof": tf / roof})
+
+        def conv2_layer(name, c, h, f, r, st, pad):
+            lx = torch.randn((1, c, h, h), device=dev)
+            lw = torch.randn((f, c, r, r), device=dev) * 0.05
+            ly = ops.conv2d(lx, lw, pad, pad, st, st, act="relu")
+            ms = time_in_graph(lambda: ops.conv2d(lx, lw, pad, pad, st, st, act="relu", out=ly))
+            layer_line(name, ms, 2.0 * ly.numel() * c * r * r,
+                       4.0 * (lx.numel() + lw.numel() + ly.numel()))
+
+        def conv3_layer(name, c, t, h, f, k, st, pad):
+            lx = torch.randn((1, c, t, h, h), device=dev)
+            lw = torch.randn((f, c) + k, device=dev) * 0.05
+            pk = ops.conv3d_pack_filters(lw) or lw
+            ly = ops.conv3d(lx, pk, pad, st, act="relu")
+            ms = time_in_graph(lambda: ops.conv3d(lx, pk, pad, st, act="relu", out=ly))
+            layer_line(name, ms, 2.0 * ly.numel() * c * k[0] * k[1] * k[2],
+                       4.0 * (lx.numel() + lw.numel() + ly.numel()))
+
+        def mm_layer(name, b, m, n, k, tb=False):
+            la = torch.randn((b, m, k), device=dev)
+            lb = torch.randn((b, n, k) if tb else (b, k, n), device=dev)
+            lc = ops.matmul(la, lb, False, tb)
+            ms = time_in_graph(lambda: ops.matmul(la, lb, False, tb, out=lc))
+            layer_line(name, ms, 2.0 * b * m * n * k, 4.0 * b * (m * k + k * n + m * n))
+
+        try:
+            conv2_layer("c1/c3 conv3x3 64->64 @56", 64, 56, 64, 3, 1, 1)
+            conv2_layer("c3 stem 7x7/2 3->64 @224", 3, 224, 64, 7, 2, 3)
+            for c, h, f, st in [(64, 56, 128, 2), (128, 28, 128, 1), (128, 28, 256, 2),
+                                (256, 14, 256, 1), (256, 14, 512, 2), (512, 7, 512, 1)]:
+                conv2_layer("c3 conv3x3/%d %d->%d @%d" % (st, c, f, h), c, h, f, 3, st, 1)
+            for c, h, f in [(64, 56, 128), (128, 28, 256), (256, 14, 512)]:
+                conv2_layer("c3 conv1x1/2 %d->%d @%d" % (c, f, h), c, h, f, 1, 2, 0)
+            mm_layer("c3 fc 1x512x1000", 1, 1, 1000, 512)
+            mm_layer("c4 qkv b3 128x768x768", 3, 128, 768, 768)
+            mm_layer("c4 scores b12 128x128x64 (B transposed)", 12, 128, 128, 64, True)
+            mm_layer("c4 probs x V b12 128x64x128", 12, 128, 64, 128)
+            mm_layer("c4 out-proj 128x768x768", 1, 128, 768, 768)
+            mm_layer("c4 ffn1 128x3072x768", 1, 128, 3072, 768)
+            mm_layer("c4 ffn2 128x768x3072", 1, 128, 768, 3072)
+            conv3_layer("c5 stem 3x7x7/(1,2,2) 3->64 @16x112", 3, 16, 112, 64, (3, 7, 7),
+                        (1, 2, 2), (1, 3, 3))
+            for c, t, h, f, st in [(64, 16, 56, 64, 1), (64, 16, 56, 128, 2), (128, 8, 28, 128, 1),
+                                   (128, 8, 28, 256, 2), (256, 4, 14, 256, 1),
+                                   (256, 4, 14, 512, 2), (512, 2, 7, 512, 1)]:
+                conv3_layer("c5 conv3x3x3/%d %d->%d @%dx%d" % (st, c, f, t, h), c, t, h, f,
+                            (3, 3, 3), (st, st, st), (1, 1, 1))
+            for c, t, h, f in [(64, 16, 56, 128), (128, 8, 28, 256), (256, 4, 14, 512)]:
+                conv3_layer("c5 conv1x1x1/2 %d->%d @%dx%d" % (c, f, t, h), c, t, h, f, (1, 1, 1),
+                            (2, 2, 2), (0, 0, 0))
+        except Exception as exc:  # report, do not lose the main measurement
+            cfg_layers.append({"error": str(exc)[:200]})
+
     # ---- the same networks through the C++ host layer (tpm::Graph -> SubGraph ->
     # CodeEngine::instantiate -> HIP graph replay), the path a PET user takes
     host_path = {}
@@ -383,6 +462,7 @@ def main():
         "cpu_baseline": cpu,
         "per_op": per_op,
         "configs": other,
+        "config_layers": cfg_layers,
         "host_layer_graphs": host_path,
     }
     print(json.dumps(out))
