@@ -3,7 +3,7 @@
 Inputs are small integers (every contraction below stays exact in fp32), expected
 outputs come from routines that share no code with the oracle or the HIP library:
 torch's CPU convolutions and numpy's matmul / reshape / transpose / pad / split /
-concatenate / tile. The transposes are the reference's own closed form
+concatenate / tile / take / mean and integer powers. The transposes are the reference's own closed form
 (reshape -> transpose -> reshape, src/Test/dat/transpose_test/transpose_ops.op:1-3
 and src/Test/transpose_test_2.py:4-31) on an iota input (src/Test/transpose_test_2.cc:24);
 the matmul triple is the reference's batch-GEMM merge case
@@ -91,6 +91,17 @@ def main():
     out["lay_pad"] = np.pad(z, [(0, 0), (1, 0), (2, 1), (0, 3)])
     out["lay_slice"] = np.ascontiguousarray(z[:, 1:5, 2:4, :3])  # begin (0,1,2,0), end (0,1,1,1)
     out["lay_extend"] = np.concatenate([z, z, z], axis=1)        # extend dim 1 by 2 copies
+    # ---- element-wise powers and division, gather, mean over an axis (all exact)
+    e = ints((3, 4, 5))
+    d = np.array([2, -4, 0.5, 8, -1], np.float32)
+    out["elt_x"], out["elt_pow3"], out["elt_d"], out["elt_div"] = e, e ** 3, d, e / d
+    tab, idx = ints((7, 6)), np.array([[5, 0, 3], [2, 2, -1]], np.int32)
+    out["ga_x"], out["ga_idx"] = tab, idx
+    out["ga_axis0"] = tab[idx % 7]                                        # [2, 3, 6]
+    out["ga_axis1"] = np.ascontiguousarray(np.moveaxis(tab[:, idx % 6], 0, 2))  # [2, 3, 7]
+    r = ints((2, 8, 4))
+    out["rm_x"] = r
+    out["rm_axis1"], out["rm_axis2"] = r.mean(axis=1, keepdims=True), r.mean(axis=2, keepdims=True)
     np.savez_compressed(os.path.join(HERE, "golden.npz"), **out)
     print("wrote", os.path.join(HERE, "golden.npz"), len(out), "arrays")
 

@@ -22,6 +22,12 @@ class OracleBackend:
     def get(self, a):
         return np.asarray(a)
 
+    def put_idx(self, a):
+        return np.ascontiguousarray(a)
+
+    def div(self, a, b):
+        return oracle.div(a, b, a.shape)
+
     def __getattr__(self, k):
         return getattr(oracle, k)
 
@@ -40,6 +46,12 @@ class HipBackend:
     def get(self, t):
         self.torch.cuda.synchronize()
         return t.cpu().numpy()
+
+    def put_idx(self, a):
+        return self.torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+    def div(self, a, b):
+        return self.ops.eltwise("div", [a, b], tuple(a.shape))
 
     def __getattr__(self, k):
         return getattr(self.ops, k)
@@ -89,6 +101,16 @@ def check_all(be):
     eq(be.get(be.pad(z, [0, 1, 2, 0], [0, 0, 1, 3])), G["lay_pad"])
     eq(be.get(be.slice_(z, [0, 1, 2, 0], [0, 1, 1, 1])), G["lay_slice"])
     eq(be.get(be.extend(z, 1, 2)), G["lay_extend"])
+    # powers, division, gather (index dims first), mean over an axis
+    e = be.put(G["elt_x"])
+    eq(be.get(be.pow_(e, 3)), G["elt_pow3"])
+    eq(be.get(be.div(e, be.put(G["elt_d"]))), G["elt_div"])
+    tab, idx = be.put(G["ga_x"]), be.put_idx(G["ga_idx"])
+    eq(be.get(be.gather(tab, idx, 0)), G["ga_axis0"])
+    eq(be.get(be.gather(tab, idx, 1)), G["ga_axis1"])
+    r = be.put(G["rm_x"])
+    eq(be.get(be.reduce_mean(r, 1)), G["rm_axis1"])
+    eq(be.get(be.reduce_mean(r, 2)), G["rm_axis2"])
 
 
 def test_oracle_reproduces_golden_vectors():
