@@ -327,6 +327,80 @@ def test_model_graph_replay_equals_operator_by_operator_run(model):
         assert rec["folded"] == 2 and rec["kernels"] == 8
 
 
+def _cpp_module():
+    import glob
+    import importlib
+    import sys
+    assert glob.glob(os.path.join(LIB, "cpp_module*.so")), "run __graft_entry__.build() first"
+    if LIB not in sys.path:
+        sys.path.insert(0, LIB)
+    return importlib.import_module("cpp_module")
+
+
+def test_python_module_builds_graphs_like_the_reference_front_end():
+    """cpp_module (the reference's src/ffi/ffi_pet.cc surface): builder names, argument
+    orders and shape rules, no device needed."""
+    cm = _cpp_module()
+    g = cm.Graph()
+    x, w = g.tensor([1, 8, 12, 12], "FLOAT"), g.tensor([16, 8, 3, 3], "FLOAT")
+    y = g.tensor([1, 16, 12, 12], "FLOAT")
+    conv = g.conv(x, w, y, 1, 1)                      # input, weight, output, ph, pw
+    assert y.getDims() == [1, 16, 12, 12] and "Conv" in conv.toString()
+    t = g.tensor([2, 16, 6, 12], "FLOAT")
+    g.transpose(y, t, 2, [[0, 2], 1, -1, 3], -2)      # H2N as the mutator writes it
+    assert t.getDims() == [2, 16, 6, 12]
+    a, b, c = g.tensor([3, 5, 7], "FLOAT"), g.tensor([3, 7, 4], "FLOAT"), g.tensor([3, 5, 4], "FLOAT")
+    g.matmul(a, b, c)
+    assert c.getDims() == [3, 5, 4]
+    s0, s1 = g.tensor([1, 4, 12, 12], "FLOAT"), g.tensor([1, 12, 12, 12], "FLOAT")
+    g.split(y, [s0, s1], 1, [1, 3])                   # sizes are ratios
+    assert s0.getDims() == [1, 4, 12, 12] and s1.getDims() == [1, 12, 12, 12]
+    p = g.tensor([1, 16, 14, 13], "FLOAT")
+    g.pad(y, p, [0, 0, 1, 0], [0, 0, 1, 1])
+    assert p.getDims() == [1, 16, 14, 13]
+    g.updateConnection()
+    sub = cm.SubGraph(g.getOperators())
+    assert len(sub.getOperators()) == len(g.getOperators()) == 5
+    assert {tuple(i.getDims()) for i in sub.getInputs()} == {(1, 8, 12, 12), (16, 8, 3, 3),
+                                                             (3, 5, 7), (3, 7, 4)}
+
+
+@pytest.mark.gpu
+def test_python_module_runs_a_graph_on_the_device():
+    """Graph built from Python, data from numpy, run operator by operator and as one
+    replayed HIP graph; against the oracle."""
+    import numpy as np
+    import oracle
+    cm = _cpp_module()
+    rng = np.random.default_rng(5)
+    g = cm.Graph()
+    x, w = g.tensor([1, 8, 12, 12], "FLOAT"), g.tensor([16, 8, 3, 3], "FLOAT")
+    y, z = g.tensor([1, 16, 12, 12], "FLOAT"), g.tensor([1, 16, 12, 12], "FLOAT")
+    g.conv(x, w, y, 1, 1)
+    g.relu(y, z)
+    t = g.tensor([2, 16, 6, 12], "FLOAT")
+    g.transpose(z, t, 2, [[0, 2], 1, -1, 3], -2)
+    g.updateConnection()
+    xv = rng.integers(-3, 4, (1, 8, 12, 12)).astype(np.float32)
+    wv = rng.integers(-3, 4, (16, 8, 3, 3)).astype(np.float32)
+    want = oracle.transpose(np.maximum(oracle.conv2d(xv, wv, 1, 1), 0), 2, [[0, 2], 1, -1, 3], -2)
+    for replay in (False, True):
+        sub = cm.SubGraph(g.getOperators())
+        for inp in sub.getInputs():
+            inp.setData(xv if inp.getDims() == [1, 8, 12, 12] else wv)
+        if replay:
+            ce = cm.CodeEngine()
+            ex = ce.instantiate(sub)
+            assert ex.launch() and ex.sync()
+            assert ex.time(2, 5) > 0
+            assert "pet_hip_conv2d" in ce.genCode(sub)
+        else:
+            assert sub.compute()
+            assert sub.perf(cm.PerfEngine()) > 0
+        got = sub.getOutputs()[0].getData()
+        assert got.shape == want.shape and got.tobytes() == want.tobytes(), replay
+
+
 @pytest.mark.gpu
 @pytest.mark.parametrize("model", ["resnet18", "resnet3d18", "bert"])
 def test_emitted_model_program_compiles_and_agrees_with_the_runtime(model, tmp_path):
