@@ -62,6 +62,8 @@ PYBIND11_MODULE(cpp_module, m) {
         .def("size", &Tensor::size)
         .def("getHash", &Tensor::getHash)
         .def("dataRand", [](Tensor &t, int seed) { return t.dataRand(seed); }, "seed"_a = 0)
+        .def("setWeight", [](Tensor &t) { t.setType(Tensor::Weight); })
+        .def("isWeight", [](const Tensor &t) { return t.getType() == Tensor::Weight; })
         .def("setData", &setTensorData)
         .def("getData", &tensorData);
 
@@ -148,6 +150,35 @@ PYBIND11_MODULE(cpp_module, m) {
              py::overload_cast<Tensor *, Tensor *, Tensor *, Tensor *, Tensor *, Tensor *, float,
                                float>(&Graph::batchnorm),
              "input"_a, "scale"_a, "bias"_a, "mean"_a, "var"_a, "output"_a, "epsilon"_a = 1e-5f,
+             "momentum"_a = 0.9f, kRef)
+        // the same builders making their own output tensor (the reference's C++ overloads)
+        .def("conv",
+             py::overload_cast<Tensor *, Tensor *, int, int, int, int, int, int, Tensor *>(
+                 &Graph::conv),
+             "input"_a, "weight"_a, "ph"_a, "pw"_a, "sh"_a = 1, "sw"_a = 1, "dh"_a = 1, "dw"_a = 1,
+             "bias"_a = nullptr, kRef)
+        .def("matmul", py::overload_cast<Tensor *, Tensor *, bool, bool, Tensor *>(&Graph::matmul),
+             "A"_a, "B"_a, "transA"_a = false, "transB"_a = false, "bias"_a = nullptr, kRef)
+        .def("pad", py::overload_cast<Tensor *, const Dim &, const Dim &>(&Graph::pad), kRef)
+        .def("slice", py::overload_cast<Tensor *, const Dim &, const Dim &>(&Graph::slice), kRef)
+        .def("concat", py::overload_cast<const TensorVec &, int>(&Graph::concat), kRef)
+        .def("split", py::overload_cast<Tensor *, int, std::vector<int>>(&Graph::split), kRef)
+        .def("transpose",
+             [](Graph &g, Tensor *in, int split, const py::list &after, int factor) {
+                 return g.transpose(in, split, permFrom(after), factor);
+             },
+             "input"_a, "split"_a, "after"_a, "factor"_a = 2, kRef)
+        .def("add", py::overload_cast<const TensorVec &>(&Graph::add), kRef)
+        .def("mul", py::overload_cast<const TensorVec &>(&Graph::mul), kRef)
+        .def("div", py::overload_cast<Tensor *, Tensor *>(&Graph::div), kRef)
+        .def("pow", py::overload_cast<Tensor *, int>(&Graph::pow), kRef)
+        .def("gather", py::overload_cast<Tensor *, Tensor *, int>(&Graph::gather), kRef)
+        .def("reduceMean", py::overload_cast<Tensor *, int>(&Graph::reduceMean), kRef)
+        .def("relu", py::overload_cast<Tensor *>(&Graph::relu), kRef)
+        .def("batchnorm",
+             py::overload_cast<Tensor *, Tensor *, Tensor *, Tensor *, Tensor *, float, float>(
+                 &Graph::batchnorm),
+             "input"_a, "scale"_a, "bias"_a, "mean"_a, "var"_a, "epsilon"_a = 1e-5f,
              "momentum"_a = 0.9f, kRef)
         .def("setInputs", &Graph::setInputs)
         .def("setOutputs", &Graph::setOutputs)

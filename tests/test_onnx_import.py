@@ -1,0 +1,156 @@
+"""ONNX ingestion without the `onnx` package (pet_amd/onnx_import.py, the role of the
+reference's python/cpp_plugin/import_onnx.py): parser on hand-written files, graph
+building on the CPU, and on the GPU a small residual CNN and an attention-style block
+against torch's CPU operators. No file written by the `onnx` package itself is
+available here, so compatibility with its serialiser rests on the published field
+numbers the writer (tests/onnx_writer.py) and the reader both follow."""
+import glob
+import os
+
+import numpy as np
+import pytest
+
+from tests import onnx_writer as ow
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+pytestmark = pytest.mark.skipif(
+    not glob.glob(os.path.join(ROOT, "pet_amd", "lib", "cpp_module*.so")),
+    reason="cpp_module is not built (pybind11 missing at build time)")
+
+
+def cnn(rng):
+    w = {"w1": rng.standard_normal((8, 3, 3, 3)) * 0.2, "b1": rng.standard_normal(8) * 0.1,
+         "sc": rng.uniform(0.5, 1.5, 8), "bi": rng.standard_normal(8) * 0.1,
+         "me": rng.standard_normal(8) * 0.1, "va": rng.uniform(0.5, 1.5, 8),
+         "w2": rng.standard_normal((8, 8, 3, 3)) * 0.1,
+         "fc": rng.standard_normal((10, 8)) * 0.3, "fb": rng.standard_normal(10) * 0.1}
+    w = {k: v.astype(np.float32) for k, v in w.items()}
+    nodes = [
+        ow.node("Conv", ["x", "w1", "b1"], ["c1"], pads=[1, 1, 1, 1], strides=[1, 1],
+                dilations=[1, 1], kernel_shape=[3, 3], group=1),
+        ow.node("Relu", ["c1"], ["r1"]),
+        ow.node("MaxPool", ["r1"], ["p1"], packed=True, kernel_shape=[2, 2], strides=[2, 2],
+                pads=[0, 0, 0, 0]),
+        ow.node("BatchNormalization", ["p1", "sc", "bi", "me", "va"], ["bn"], epsilon=1e-3),
+        ow.node("Conv", ["bn", "w2"], ["c2"], pads=[1, 1, 1, 1]),
+        ow.node("Add", ["c2", "bn"], ["s"]),
+        ow.node("Relu", ["s"], ["r2"]),
+        ow.node("GlobalAveragePool", ["r2"], ["gap"]),
+        ow.node("Flatten", ["gap"], ["flat"], axis=1),
+        ow.node("Gemm", ["flat", "fc", "fb"], ["logits"], transB=1, alpha=1.0, beta=1.0),
+        ow.node("Softmax", ["logits"], ["prob"], axis=-1),
+    ]
+    data = ow.model(nodes, w, [("x", [1, 3, 16, 16])] + [(k, list(v.shape)) for k, v in w.items()],
+                    [("prob", [1, 10])])
+    return data, w
+
+
+def cnn_reference(x, w):
+    import torch
+    import torch.nn.functional as F
+    t = {k: torch.from_numpy(v) for k, v in w.items()}
+    y = F.relu(F.conv2d(torch.from_numpy(x), t["w1"], t["b1"], padding=1))
+    y = F.max_pool2d(y, 2, 2)
+    bn = F.batch_norm(y, t["me"], t["va"], t["sc"], t["bi"], False, 0.1, 1e-3)
+    y = F.relu(F.conv2d(bn, t["w2"], None, padding=1) + bn)
+    y = F.adaptive_avg_pool2d(y, 1).flatten(1)
+    return F.softmax(F.linear(y, t["fc"], t["fb"]), dim=-1).numpy()
+
+
+def test_parser_reads_packed_and_unpacked_fields():
+    from pet_amd import onnx_import
+    data, w = cnn(np.random.default_rng(0))
+    nodes, inits, inputs, outputs = onnx_import.parse(data)
+    assert [n.op for n in nodes][:4] == ["Conv", "Relu", "MaxPool", "BatchNormalization"]
+    assert nodes[0].attrs["pads"] == [1, 1, 1, 1] and nodes[0].inputs == ["x", "w1", "b1"]
+    assert nodes[2].attrs["kernel_shape"] == [2, 2] and nodes[2].attrs["strides"] == [2, 2]  # packed
+    assert abs(nodes[3].attrs["epsilon"] - 1e-3) < 1e-9 and nodes[9].attrs["transB"] == 1
+    assert nodes[10].attrs["axis"] == -1                                   # negative varint
+    assert set(inits) == set(w) and np.array_equal(inits["w2"], w["w2"])
+    assert inputs[0] == ("x", [1, 3, 16, 16]) and outputs == ["prob"]
+    # int64 initializer through int64_data as well as raw_data
+    t = ow.i(1, 3) + ow.i(2, 7) + ow.s(8, "shape") + ow.ld(7, b"".join(ow.varint(v) for v in (2, -1, 4)))
+    name, arr = onnx_import._tensor(t)
+    assert name == "shape" and arr.tolist() == [2, -1, 4] and arr.dtype == np.int64
+
+
+def test_graph_building_and_shape_rules():
+    from pet_amd import onnx_import
+    data, w = cnn(np.random.default_rng(0))
+    m = onnx_import.load(data)
+    assert m.inputs == ["x"] and set(m.weights) == set(w)
+    shapes = {k: m.tensors[k].getDims() for k in ("c1", "p1", "bn", "c2", "r2", "gap")}
+    assert shapes == {"c1": [1, 8, 16, 16], "p1": [1, 8, 8, 8], "bn": [1, 8, 8, 8],
+                      "c2": [1, 8, 8, 8], "r2": [1, 8, 8, 8], "gap": [1, 8, 1, 1]}
+    # MatmulOp gives 2-D operands a leading 1 (MatmulOp::dimExtend, operator.cc:656-662)
+    assert m.tensors["flat"].getDims() == [1, 1, 8]
+    assert m.tensors["prob"].size() == 10 and m.tensors["w1"].isWeight()
+    assert len(m.graph.getOperators()) == 11
+    with pytest.raises(ValueError):
+        onnx_import.load(ow.model([ow.node("Einsum", ["x"], ["y"])], {}, [("x", [2, 2])], [("y", [2, 2])]))
+    with pytest.raises(ValueError):     # channel-wise broadcast is not a trailing-dim broadcast
+        onnx_import.load(ow.model([ow.node("Mul", ["x", "s"], ["y"])],
+                                  {"s": np.ones((1, 3, 1, 1), np.float32)},
+                                  [("x", [1, 3, 4, 4])], [("y", [1, 3, 4, 4])]))
+
+
+@pytest.mark.gpu
+def test_imported_cnn_matches_torch():
+    from pet_amd import onnx_import
+    rng = np.random.default_rng(1)
+    data, w = cnn(rng)
+    x = rng.standard_normal((1, 3, 16, 16)).astype(np.float32)
+    want = cnn_reference(x, w)
+    m = onnx_import.load(data)
+    for replay in (False, True):
+        sub, feeds = m.subgraph()
+        feeds["x"].setData(x)
+        if replay:
+            ex = m.module.CodeEngine().instantiate(sub)
+            assert ex.launch() and ex.sync()
+        else:
+            assert sub.compute()
+        got = sub.getOutputs()[0].getData().reshape(want.shape)
+        np.testing.assert_allclose(got, want, rtol=1e-4, atol=1e-6)
+
+
+@pytest.mark.gpu
+def test_imported_attention_block_matches_torch():
+    """MatMul / Reshape / Transpose / Softmax / Split / Concat / Gather / ReduceMean / Pow."""
+    import torch
+    from pet_amd import onnx_import
+    rng = np.random.default_rng(2)
+    seq, hid, heads = 8, 16, 2
+    w = {"emb": rng.standard_normal((20, hid)).astype(np.float32),
+         "wqkv": (rng.standard_normal((hid, 3 * hid)) * 0.2).astype(np.float32),
+         "ids": np.array([3, 19, 0, 7, 7, 1, 12, 5], dtype=np.int64),
+         "shp": np.array([seq, heads, hid // heads], dtype=np.int64),
+         "two": np.array([2.0], dtype=np.float32)}
+    nodes = [
+        ow.node("Gather", ["emb", "ids"], ["x"], axis=0),
+        ow.node("MatMul", ["x", "wqkv"], ["qkv"]),
+        ow.node("Split", ["qkv"], ["q", "k", "v"], axis=-1, split=[hid, hid, hid]),
+    ]
+    for n in "qkv":
+        nodes += [ow.node("Reshape", [n, "shp"], [n + "r"]),
+                  ow.node("Transpose", [n + "r"], [n + "h"], perm=[1, 0, 2])]
+    nodes += [ow.node("Transpose", ["kh"], ["kt"], perm=[0, 2, 1]),
+              ow.node("MatMul", ["qh", "kt"], ["sc"]),
+              ow.node("Softmax", ["sc"], ["pr"], axis=-1),
+              ow.node("MatMul", ["pr", "vh"], ["ctx"]),
+              ow.node("Pow", ["ctx", "two"], ["sq"]),
+              ow.node("ReduceMean", ["sq"], ["ms"], axes=[2], keepdims=1),
+              ow.node("Concat", ["ctx", "sq"], ["cat"], axis=2)]
+    data = ow.model(nodes, w, [], [("ms", [heads, seq, 1]), ("cat", [heads, seq, hid])])
+    x = torch.from_numpy(w["emb"])[torch.from_numpy(w["ids"])]
+    q, k, v = (x @ torch.from_numpy(w["wqkv"])).split(hid, dim=-1)
+    qh, kh, vh = (t.reshape(seq, heads, hid // heads).permute(1, 0, 2) for t in (q, k, v))
+    ctx = torch.softmax(qh @ kh.transpose(1, 2), -1) @ vh
+    want = {"ms": (ctx ** 2).mean(2, keepdim=True).numpy(), "cat": torch.cat([ctx, ctx ** 2], 2).numpy()}
+    m = onnx_import.load(data)
+    sub, feeds = m.subgraph()
+    assert feeds == {}
+    assert sub.compute()
+    outs = {tuple(t.getDims()): t.getData() for t in sub.getOutputs()}
+    np.testing.assert_allclose(outs[(heads, seq, 1)], want["ms"], rtol=1e-4, atol=1e-5)
+    np.testing.assert_allclose(outs[(heads, seq, hid)], want["cat"], rtol=1e-4, atol=1e-5)
