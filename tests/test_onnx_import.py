@@ -10,7 +10,10 @@ import os
 import numpy as np
 import pytest
 
-from tests import onnx_writer as ow
+try:
+    from tests import onnx_writer as ow
+except ImportError:          # collected with tests/ itself on sys.path
+    import onnx_writer as ow
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 pytestmark = pytest.mark.skipif(
