@@ -186,7 +186,9 @@ PYBIND11_MODULE(cpp_module, m) {
         .def("getTensors", [](Graph &g) { return g.getTensors(); }, kRef)
         .def("updateConnection", &Graph::updateConnection);
 
-    py::class_<SubGraph, std::shared_ptr<SubGraph>>(m, "SubGraph")
+    // dynamic attributes: Python code parks the Graph a SubGraph was cut from on it (the
+    // SubGraph's operators keep pointing at that Graph's bias-like side tensors)
+    py::class_<SubGraph, std::shared_ptr<SubGraph>>(m, "SubGraph", py::dynamic_attr())
         .def(py::init<>())
         .def(py::init<OpVec>())
         .def("getInputs", [](SubGraph &g) { return g.getInputs(); }, kRef)

@@ -203,6 +203,7 @@ class Model:
         for name, arr in self.weights.items():
             self.tensors[name].setData(arr.astype(np.float32))
         sub = self.module.SubGraph(self.graph.getOperators())
+        sub.model = self    # the side tensors live in self.graph: keep it alive with the SubGraph
         by_hash = {self.tensors[n].getHash(): n for n in list(self.weights) + self.inputs}
         feeds = {}
         for t in sub.getInputs():
@@ -234,11 +235,48 @@ def _sym(pads, n):
     return pads[:n]
 
 
-def load(source, module=None):
-    """source: a path or the bytes of an ONNX file."""
+def fold_batchnorm(nodes, inits, outputs):
+    """Conv -> BatchNormalization with constant parameters, the convolution's result used
+    nowhere else: the normalisation goes into the filters and the bias (what exporters
+    do when they "fold BN"; the benchmark's ResNets are stated that way). Returns the new
+    node list; new initializers are added to `inits`."""
+    users = {}
+    for nd in nodes:
+        for n in nd.inputs:
+            users[n] = users.get(n, 0) + 1
+    by_out = {nd.outputs[0]: nd for nd in nodes if nd.outputs}
+    dropped, out_nodes = set(), []
+    for nd in nodes:
+        if nd.op != "BatchNormalization" or any(n not in inits for n in nd.inputs[1:5]):
+            continue
+        conv = by_out.get(nd.inputs[0])
+        if (conv is None or conv.op != "Conv" or users.get(conv.outputs[0], 0) != 1 or
+                conv.outputs[0] in outputs or any(n not in inits for n in conv.inputs[1:])):
+            continue
+        sc, bi, me, va = (inits[n].astype(np.float64) for n in nd.inputs[1:5])
+        factor = sc / np.sqrt(va + float(nd.attrs.get("epsilon", 1e-5)))
+        w = inits[conv.inputs[1]].astype(np.float64)
+        b = inits[conv.inputs[2]].astype(np.float64) if len(conv.inputs) > 2 else np.zeros(w.shape[0])
+        wn, bn = conv.inputs[1] + "::bn", conv.outputs[0] + "::bn_bias"
+        inits[wn] = (w * factor.reshape((-1,) + (1,) * (w.ndim - 1))).astype(np.float32)
+        inits[bn] = ((b - me) * factor + bi).astype(np.float32)
+        conv.inputs = [conv.inputs[0], wn, bn]
+        conv.outputs = [nd.outputs[0]]
+        dropped.add(id(nd))
+    for nd in nodes:
+        if id(nd) not in dropped:
+            out_nodes.append(nd)
+    return out_nodes
+
+
+def load(source, module=None, fold_bn=True):
+    """source: a path or the bytes of an ONNX file. fold_bn: BatchNormalization after a
+    convolution with constant parameters is folded into that convolution."""
     cm = module or _module()
     data = source if isinstance(source, (bytes, bytearray, memoryview)) else open(source, "rb").read()
     nodes, inits, inputs, outputs = parse(data)
+    if fold_bn:
+        nodes = fold_batchnorm(nodes, inits, outputs)
     g = cm.Graph()
     m = Model(cm, g)
     const = dict(inits)                         # values known at import time

@@ -117,6 +117,48 @@ def test_imported_cnn_matches_torch():
         np.testing.assert_allclose(got, want, rtol=1e-4, atol=1e-6)
 
 
+def _conv_bn_model(rng):
+    w = {"w": (rng.standard_normal((6, 4, 3, 3)) * 0.2), "b": rng.standard_normal(6) * 0.1,
+         "sc": rng.uniform(0.5, 1.5, 6), "bi": rng.standard_normal(6) * 0.1,
+         "me": rng.standard_normal(6) * 0.1, "va": rng.uniform(0.5, 1.5, 6)}
+    w = {k: v.astype(np.float32) for k, v in w.items()}
+    nodes = [ow.node("Conv", ["x", "w", "b"], ["c"], pads=[1, 1, 1, 1], strides=[2, 2]),
+             ow.node("BatchNormalization", ["c", "sc", "bi", "me", "va"], ["n"], epsilon=1e-5),
+             ow.node("Relu", ["n"], ["y"])]
+    return ow.model(nodes, w, [("x", [2, 4, 9, 9])], [("y", [2, 6, 5, 5])]), w
+
+
+def test_batchnorm_after_a_convolution_is_folded():
+    from pet_amd import onnx_import
+    data, w = _conv_bn_model(np.random.default_rng(3))
+    folded = onnx_import.load(data)
+    kept = onnx_import.load(data, fold_bn=False)
+    assert len(folded.graph.getOperators()) == 2 and len(kept.graph.getOperators()) == 3
+    factor = w["sc"] / np.sqrt(w["va"] + np.float32(1e-5))
+    np.testing.assert_allclose(folded.weights["w::bn"], w["w"] * factor[:, None, None, None],
+                               rtol=1e-6)
+    np.testing.assert_allclose(folded.weights["c::bn_bias"], (w["b"] - w["me"]) * factor + w["bi"],
+                               rtol=1e-5, atol=1e-7)
+
+
+@pytest.mark.gpu
+def test_folded_and_unfolded_batchnorm_match_torch():
+    import torch
+    import torch.nn.functional as F
+    from pet_amd import onnx_import
+    rng = np.random.default_rng(3)
+    data, w = _conv_bn_model(rng)
+    x = rng.standard_normal((2, 4, 9, 9)).astype(np.float32)
+    t = {k: torch.from_numpy(v) for k, v in w.items()}
+    want = F.relu(F.batch_norm(F.conv2d(torch.from_numpy(x), t["w"], t["b"], stride=2, padding=1),
+                               t["me"], t["va"], t["sc"], t["bi"], False, 0.1, 1e-5)).numpy()
+    for fold in (True, False):
+        sub, feeds = onnx_import.load(data, fold_bn=fold).subgraph()
+        feeds["x"].setData(x)
+        assert sub.compute()
+        np.testing.assert_allclose(sub.getOutputs()[0].getData(), want, rtol=1e-4, atol=1e-5)
+
+
 @pytest.mark.gpu
 def test_imported_attention_block_matches_torch():
     """MatMul / Reshape / Transpose / Softmax / Split / Concat / Gather / ReduceMean / Pow."""
