@@ -130,6 +130,26 @@ FusedTails planFusedTails(const OpVec &order, const TensorVec &graphOutputs,
     std::map<const Operator *, size_t> pos;
     for (size_t i = 0; i < order.size(); ++i)
         pos[order[i]] = i;
+    // "contraction, activation": the activation rides in the contraction's epilogue (the
+    // reference's fused cuDNN call, src/Graph/operator.cc:478-481). Keyed by the activation.
+    for (auto op : order) {
+        auto actOp = dynamic_cast<ActivationOp *>(op);
+        if (actOp == nullptr || skipped.count(op))
+            continue;
+        Tensor *t = op->getInputs()[0];
+        Operator *prod = t->getOutputOf();
+        if (prod == nullptr || !prod->canTakeResidual() || skipped.count(prod) ||
+            plan.absorbed.count(prod) || weightOnly(prod) || t->getInputOf().size() != 1 ||
+            outs.count(t) || prod->getOutputs().size() != 1)
+            continue;
+        FusedTail tail;
+        tail.contraction = prod;
+        tail.residual = nullptr;
+        tail.act = actOp->getActType();
+        tail.out = actOp->getOutputs()[0];
+        plan.absorbed.insert(prod);
+        plan.atAdd[op] = tail;
+    }
     for (auto op : order) {
         if (op->getType() != Operator::Add || op->getInputs().size() != 2 || skipped.count(op))
             continue;
@@ -240,7 +260,8 @@ LaunchPlan planLaunchFlags(const OpVec &order, const TensorVec &graphOutputs,
             continue;
         auto tail = tails.atAdd.find(op);
         if (tail != tails.atAdd.end())
-            effs.push_back({tail->second.contraction, tail->second.out, tail->second.act, true});
+            effs.push_back({tail->second.contraction, tail->second.out, tail->second.act,
+                            tail->second.residual != nullptr});
         else if (isContraction(op) && !tails.absorbed.count(op))
             effs.push_back({op, op->getOutputs()[0], ownAct(op), false});
     }
@@ -409,7 +430,7 @@ std::unique_ptr<GraphExec> CodeEngine::instantiate(std::shared_ptr<SubGraph> &gr
     FusedTails tails = planFusedTails(order, graph->getOutputs(), plan.skipped,
                                       [](const FusedTail &f) {
                                           return f.residual->devicePtr() != f.out->devicePtr();
-                                      });
+                                      }); // asked for tails with a residual only
     LaunchPlan lp = planLaunchFlags(order, graph->getOutputs(), plan.skipped, rows.folded, tails,
                                     [](const Tensor *) { return true; });
     auto flagsOf = [&](const Operator *op) {
@@ -420,8 +441,8 @@ std::unique_ptr<GraphExec> CodeEngine::instantiate(std::shared_ptr<SubGraph> &gr
         auto tail = tails.atAdd.find(op);
         if (tail != tails.atAdd.end()) {
             const FusedTail &f = tail->second;
-            return f.contraction->launchFused(st, f.residual->devicePtr(), f.act,
-                                              f.out->devicePtr(), flagsOf(f.contraction));
+            return f.contraction->launchFused(st, f.residual ? f.residual->devicePtr() : nullptr,
+                                              f.act, f.out->devicePtr(), flagsOf(f.contraction));
         }
         if (flagsOf(op))
             return op->launchFused(st, nullptr, ownAct(op), op->getOutputs()[0]->devicePtr(),
@@ -649,7 +670,8 @@ std::string CodeEngine::genCode(std::shared_ptr<SubGraph> &graph) {
         auto out = [&](size_t i) {
             return tail ? e.name(tail->out) : e.name(op->getOutputs()[i]);
         };
-        const std::string res = tail ? e.name(tail->residual) + ", " : "";
+        const std::string res =
+            tail ? (tail->residual ? e.name(tail->residual) : std::string("nullptr")) + ", " : "";
         auto actOf = [&](Operator::ActType own) { return (int)(tail ? tail->act : own); };
         if (tails.atAdd.count(op) && tail == nullptr) {
             tail = &tails.atAdd.at(op);
@@ -711,7 +733,7 @@ std::string CodeEngine::genCode(std::shared_ptr<SubGraph> &graph) {
               << ta << ", " << tb << ", " << b << ", " << m << ", " << n << ", " << k << ", "
               << in(0) << ", " << in(1) << ", " << out(0) << ", " << nullable(e, mm->getBias())
               << ", "
-              << (tail ? e.name(tail->residual) + ", " : fl ? std::string("nullptr, ") : std::string())
+              << (tail ? res : fl ? std::string("nullptr, ") : std::string())
               << actOf(mm->getAct()) << ", " << (fl ? std::to_string(fl) + "u, " : std::string())
               << "s)";
         } else if (auto tr = dynamic_cast<TransposeOp *>(op)) {

@@ -199,3 +199,91 @@ def test_imported_attention_block_matches_torch():
     outs = {tuple(t.getDims()): t.getData() for t in sub.getOutputs()}
     np.testing.assert_allclose(outs[(heads, seq, 1)], want["ms"], rtol=1e-4, atol=1e-5)
     np.testing.assert_allclose(outs[(heads, seq, hid)], want["cat"], rtol=1e-4, atol=1e-5)
+
+
+def _resnet18(rng):
+    """ResNet-18 as exporters write it: Conv + BatchNormalization + Relu, residual Add,
+    MaxPool, GlobalAveragePool, Flatten, Gemm. Random parameters."""
+    nodes, w = [], {}
+
+    def conv_bn(name, src, cin, cout, k, stride, pad, relu):
+        fan = cin * k * k
+        w[name + ".w"] = (rng.standard_normal((cout, cin, k, k)) * np.sqrt(2.0 / fan)).astype(np.float32)
+        for p, lo, hi in (("sc", 0.8, 1.2), ("va", 0.8, 1.2)):
+            w[name + "." + p] = rng.uniform(lo, hi, cout).astype(np.float32)
+        for p in ("bi", "me"):
+            w[name + "." + p] = (rng.standard_normal(cout) * 0.05).astype(np.float32)
+        nodes.append(ow.node("Conv", [src, name + ".w"], [name + ".c"], pads=[pad] * 4,
+                             strides=[stride, stride], kernel_shape=[k, k]))
+        nodes.append(ow.node("BatchNormalization",
+                             [name + ".c"] + [name + "." + p for p in ("sc", "bi", "me", "va")],
+                             [name + ".n"], epsilon=1e-5))
+        if relu:
+            nodes.append(ow.node("Relu", [name + ".n"], [name + ".r"]))
+        return name + (".r" if relu else ".n")
+
+    t = conv_bn("stem", "x", 3, 64, 7, 2, 3, True)
+    nodes.append(ow.node("MaxPool", [t], ["pool"], kernel_shape=[3, 3], strides=[2, 2], pads=[1] * 4))
+    t, cin = "pool", 64
+    for stage, cout in enumerate((64, 128, 256, 512)):
+        for blk in range(2):
+            stride = 2 if (stage > 0 and blk == 0) else 1
+            name = "l%d.%d" % (stage + 1, blk)
+            a = conv_bn(name + ".a", t, cin, cout, 3, stride, 1, True)
+            b = conv_bn(name + ".b", a, cout, cout, 3, 1, 1, False)
+            skip = t if (stride == 1 and cin == cout) else conv_bn(name + ".d", t, cin, cout, 1,
+                                                                   stride, 0, False)
+            nodes.append(ow.node("Add", [b, skip], [name + ".s"]))
+            nodes.append(ow.node("Relu", [name + ".s"], [name + ".o"]))
+            t, cin = name + ".o", cout
+    w["fc.w"] = (rng.standard_normal((1000, 512)) * 0.03).astype(np.float32)
+    w["fc.b"] = (rng.standard_normal(1000) * 0.01).astype(np.float32)
+    nodes += [ow.node("GlobalAveragePool", [t], ["gap"]), ow.node("Flatten", ["gap"], ["flat"], axis=1),
+              ow.node("Gemm", ["flat", "fc.w", "fc.b"], ["logits"], transB=1)]
+    return ow.model(nodes, w, [("x", [1, 3, 224, 224])], [("logits", [1, 1000])]), w
+
+
+def _resnet18_torch(x, w):
+    import torch
+    import torch.nn.functional as F
+    t = {k: torch.from_numpy(v) for k, v in w.items()}
+
+    def conv_bn(name, src, stride, pad, relu):
+        y = F.conv2d(src, t[name + ".w"], None, stride=stride, padding=pad)
+        y = F.batch_norm(y, t[name + ".me"], t[name + ".va"], t[name + ".sc"], t[name + ".bi"],
+                         False, 0.1, 1e-5)
+        return F.relu(y) if relu else y
+
+    y = F.max_pool2d(conv_bn("stem", torch.from_numpy(x), 2, 3, True), 3, 2, 1)
+    cin = 64
+    for stage, cout in enumerate((64, 128, 256, 512)):
+        for blk in range(2):
+            stride = 2 if (stage > 0 and blk == 0) else 1
+            name = "l%d.%d" % (stage + 1, blk)
+            b = conv_bn(name + ".b", conv_bn(name + ".a", y, stride, 1, True), 1, 1, False)
+            skip = y if (stride == 1 and cin == cout) else conv_bn(name + ".d", y, stride, 0, False)
+            y, cin = F.relu(b + skip), cout
+    return F.linear(F.adaptive_avg_pool2d(y, 1).flatten(1), t["fc.w"], t["fc.b"]).numpy()
+
+
+@pytest.mark.gpu
+def test_imported_resnet18_matches_torch():
+    """Benchmark configuration 3 end to end through the file front end: 20 convolutions
+    with their BatchNormalization folded at import, replayed as one HIP graph."""
+    from pet_amd import onnx_import
+    rng = np.random.default_rng(18)
+    data, w = _resnet18(rng)
+    x = rng.standard_normal((1, 3, 224, 224)).astype(np.float32)
+    want = _resnet18_torch(x, w)
+    m = onnx_import.load(data)
+    assert sum("Conv" in op.toString() for op in m.graph.getOperators()) == 20
+    assert not any("BatchNorm" in op.toString() for op in m.graph.getOperators())
+    sub, feeds = m.subgraph()
+    feeds["x"].setData(x)
+    ex = m.module.CodeEngine().instantiate(sub)
+    assert ex.launch() and ex.sync()
+    got = sub.getOutputs()[0].getData().reshape(want.shape)
+    scale = np.abs(want).max()
+    assert np.abs(got - want).max() <= 1e-4 * scale, (np.abs(got - want).max(), scale)
+    assert ex.numKernelOps() <= 26 and ex.numHoistedFills() >= 8
+    assert 0.05 < ex.time(5, 20) < 5.0      # ms per inference
