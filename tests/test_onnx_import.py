@@ -98,7 +98,8 @@ def test_graph_building_and_shape_rules():
 
 
 @pytest.mark.gpu
-def test_imported_cnn_matches_torch():
+def test_imported_cnn_matches_torch(tmp_path):
+    import subprocess
     from pet_amd import onnx_import
     rng = np.random.default_rng(1)
     data, w = cnn(rng)
@@ -115,6 +116,17 @@ def test_imported_cnn_matches_torch():
             assert sub.compute()
         got = sub.getOutputs()[0].getData().reshape(want.shape)
         np.testing.assert_allclose(got, want, rtol=1e-4, atol=1e-6)
+    # the program emitted for the imported graph builds against pet_hip.h alone and runs
+    src, exe = tmp_path / "net.cpp", tmp_path / "net"
+    assert m.module.CodeEngine().genCode(sub, str(src)) == 0
+    text = src.read_text()
+    # this BatchNormalization follows the pooling, not a convolution: it stays an operator
+    assert "pet_hip_conv2d" in text and "pet_hip_batchnorm(" in text
+    lib = os.path.join(ROOT, "pet_amd", "lib")
+    subprocess.run(["g++", "-O1", str(src), "-I", os.path.join(ROOT, "include"), "-L", lib,
+                    "-lpet_hip", "-Wl,-rpath," + lib, "-o", str(exe)], check=True)
+    run = subprocess.run([str(exe)], capture_output=True, text=True, timeout=300)
+    assert run.returncode == 0 and "Time(ms)" in run.stdout, run.stdout + run.stderr
 
 
 def _conv_bn_model(rng):
