@@ -338,6 +338,8 @@ def load(source, module=None, fold_bn=True):
             else:
                 raise ValueError("Conv with %d spatial dims" % nsp)
         elif op in ("Relu", "Sigmoid", "Tanh", "Gelu", "Identity", "Cast", "Dropout"):
+            if op == "Gelu" and a.get("approximate", "none") != "none":
+                raise ValueError("Gelu: the exact form only")
             out = same_shape(x)
             {"Relu": g.relu, "Sigmoid": g.sigmoid, "Tanh": g.tanh, "Gelu": g.gelu}.get(
                 op, g.identity)(x, out)
@@ -420,6 +422,12 @@ def load(source, module=None, fold_bn=True):
                 raise ValueError("Softmax over an axis other than the last")
             out = same_shape(x)
             g.softmax(x, out, ax)
+        elif op == "LayerNormalization":
+            if int(a.get("axis", -1)) % len(xd) != len(xd) - 1:
+                raise ValueError("LayerNormalization over more than the last axis")
+            out = same_shape(x)
+            g.layernorm(x, out, tin(ins[1]), tin(ins[2]) if len(ins) > 2 else None,
+                        float(a.get("epsilon", 1e-5)))
         elif op == "Gather":
             idx = tin(ins[1])
             out = g.gather(x, idx, int(a.get("axis", 0)) % len(xd)).getOutput()

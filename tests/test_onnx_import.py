@@ -173,7 +173,8 @@ def test_folded_and_unfolded_batchnorm_match_torch():
 
 @pytest.mark.gpu
 def test_imported_attention_block_matches_torch():
-    """MatMul / Reshape / Transpose / Softmax / Split / Concat / Gather / ReduceMean / Pow."""
+    """MatMul / Reshape / Transpose / Softmax / Split / Concat / Gather / ReduceMean / Pow /
+    LayerNormalization / Gelu."""
     import torch
     from pet_amd import onnx_import
     rng = np.random.default_rng(2)
@@ -197,13 +198,20 @@ def test_imported_attention_block_matches_torch():
               ow.node("MatMul", ["pr", "vh"], ["ctx"]),
               ow.node("Pow", ["ctx", "two"], ["sq"]),
               ow.node("ReduceMean", ["sq"], ["ms"], axes=[2], keepdims=1),
-              ow.node("Concat", ["ctx", "sq"], ["cat"], axis=2)]
-    data = ow.model(nodes, w, [], [("ms", [heads, seq, 1]), ("cat", [heads, seq, hid])])
+              ow.node("Concat", ["ctx", "sq"], ["cat"], axis=2),
+              ow.node("LayerNormalization", ["cat", "ln_g", "ln_b"], ["ln"], axis=-1, epsilon=1e-5),
+              ow.node("Gelu", ["ln"], ["act"])]
+    w["ln_g"] = rng.uniform(0.5, 1.5, hid).astype(np.float32)
+    w["ln_b"] = (rng.standard_normal(hid) * 0.1).astype(np.float32)
+    data = ow.model(nodes, w, [], [("ms", [heads, seq, 1]), ("act", [heads, seq, hid])])
     x = torch.from_numpy(w["emb"])[torch.from_numpy(w["ids"])]
     q, k, v = (x @ torch.from_numpy(w["wqkv"])).split(hid, dim=-1)
     qh, kh, vh = (t.reshape(seq, heads, hid // heads).permute(1, 0, 2) for t in (q, k, v))
     ctx = torch.softmax(qh @ kh.transpose(1, 2), -1) @ vh
-    want = {"ms": (ctx ** 2).mean(2, keepdim=True).numpy(), "cat": torch.cat([ctx, ctx ** 2], 2).numpy()}
+    cat = torch.cat([ctx, ctx ** 2], 2)
+    act = torch.nn.functional.gelu(torch.nn.functional.layer_norm(
+        cat, (hid,), torch.from_numpy(w["ln_g"]), torch.from_numpy(w["ln_b"]), 1e-5))
+    want = {"ms": (ctx ** 2).mean(2, keepdim=True).numpy(), "cat": act.numpy()}
     m = onnx_import.load(data)
     sub, feeds = m.subgraph()
     assert feeds == {}
