@@ -70,6 +70,17 @@ typedef enum pet_hip_call_flags {
     PET_HIP_CALL_RES_RELU = 8  /* use max(residual, 0) for the residual */
 } pet_hip_call_flags;
 
+/* Convolution algorithms, the counterpart of the cuDNN algorithm list ConvOp::perf
+ * times (src/Graph/operator.cc:296-515): how the K loop of a tile is shared out.
+ * PET_HIP_CONV_ALGO(a) goes into the flags of pet_hip_conv2d_ex_f32 / conv3d_ex.
+ * 0: the library's cost model decides (what every other entry point does); 1-5: 1, 2, 4,
+ * 8, 16 workgroups per tile (clamped to what the shape allows); 6: stream-K (when the
+ * shape admits it, else the cost model's split); 7: the cost model's split, never
+ * stream-K. Every algorithm computes the same sums; with more than one workgroup per
+ * tile their order, and so the last bits, can differ. */
+#define PET_HIP_CONV_ALGO_COUNT 8
+#define PET_HIP_CONV_ALGO(a) (((unsigned)(a) & 0xffu) << 8)
+
 /* One output of pet_hip_bias_fill_batch: y[o][c][i] = bias[c] (zeros when bias is NULL). */
 typedef struct pet_hip_fill {
     float *y;

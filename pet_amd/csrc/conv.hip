@@ -53,6 +53,8 @@ struct ConvParams {
     int y_init;     // y already holds bias (or 0): a split launch does not initialise it
     int defer_relu; // a split launch leaves its ReLU to the readers of y
     int *dry_atomic; // not null: report whether the launch would accumulate into y, launch nothing
+    int force_splitk;  // > 0: this many K shares per tile instead of the cost model's choice
+    int force_streamk; // 0 / 1: stream-K off / on instead of the cost model's choice; -1: model
     int res_first;   // accumulating launch into an initialised y: the workgroup that holds a
                      // tile's first K step adds the residual along with its partial sums
     FastDiv fd_krs, fd_rs, fd_s;     // k -> (c, kt, r, s)
@@ -947,7 +949,8 @@ int launch_plane_cfg(ConvParams p, hipStream_t stream) {
             }
         }
     }
-    static const int forced = getenv("PET_HIP_SPLITK") ? atoi(getenv("PET_HIP_SPLITK")) : 0;
+    static const int forced_env = getenv("PET_HIP_SPLITK") ? atoi(getenv("PET_HIP_SPLITK")) : 0;
+    const int forced = p.force_splitk > 0 ? p.force_splitk : forced_env;
     if (forced > 0)
         splitk = std::min(forced, nit);
     if ((long long)p.G * splitk > 65535)
@@ -961,7 +964,8 @@ int launch_plane_cfg(ConvParams p, hipStream_t stream) {
     // no margin the 512->512 layers of the dilated block turn 3 % slower).
     p.streamk = 0;
     {
-        static const int sk_env = getenv("PET_HIP_STREAMK") ? atoi(getenv("PET_HIP_STREAMK")) : -1;
+        static const int sk_env0 = getenv("PET_HIP_STREAMK") ? atoi(getenv("PET_HIP_STREAMK")) : -1;
+        const int sk_env = p.force_streamk >= 0 ? p.force_streamk : sk_env0;
         const long long units = tiles * nit;
         const int wgs = Cfg::BM * Cfg::BN >= 64 * 128 ? 256 : 512;
         const double cost_sk = (double)units / 256 + 2 * c_fixed + c_launches;
@@ -1155,7 +1159,7 @@ int conv_common(const float *x, const float *w, const float *bias, float *y, int
                 bool wpacked = false, const float *res = nullptr, unsigned flags = 0,
                 int *dry = nullptr) {
     if (flags & ~(unsigned)(PET_HIP_CALL_Y_INITIALISED | PET_HIP_CALL_DEFER_RELU |
-                            PET_HIP_CALL_X_RELU | PET_HIP_CALL_RES_RELU))
+                            PET_HIP_CALL_X_RELU | PET_HIP_CALL_RES_RELU | 0xff00u))
         return set_error(PET_HIP_ERR_INVALID, "unknown call flags 0x%x", flags);
     if ((flags & PET_HIP_CALL_DEFER_RELU) && act != PET_HIP_ACT_RELU)
         return set_error(PET_HIP_ERR_INVALID, "only a ReLU can be left to the readers");
@@ -1234,6 +1238,21 @@ int conv_common(const float *x, const float *w, const float *bias, float *y, int
     p.y_init = (flags & PET_HIP_CALL_Y_INITIALISED) != 0;
     p.defer_relu = (flags & PET_HIP_CALL_DEFER_RELU) != 0;
     p.dry_atomic = dry;
+    p.force_streamk = -1;
+    {
+        // algorithm override, bits 8-15 of the flags (0: the cost model decides)
+        static const int kSplit[] = {0, 1, 2, 4, 8, 16, 0, 0};
+        const unsigned algo = (flags >> 8) & 0xffu;
+        if (algo >= PET_HIP_CONV_ALGO_COUNT)
+            return set_error(PET_HIP_ERR_INVALID, "unknown convolution algorithm %u", algo);
+        p.force_splitk = kSplit[algo];
+        if (algo >= 1 && algo <= 5)
+            p.force_streamk = 0;
+        else if (algo == 6)
+            p.force_streamk = 1;
+        else if (algo == 7)
+            p.force_streamk = 0;
+    }
     p.wpacked = wpacked;
     if (wpacked && !packed_filters_apply(f, c / groups, kt, r, s))
         return set_error(PET_HIP_ERR_UNSUPPORTED, "no kt-major form for this filter shape");
@@ -1266,6 +1285,7 @@ int bmm_as_grouped_1x1(const float *A, const float *B, float *C, const float *bi
     memset(&p, 0, sizeof(p));
     p.y_init = (flags & PET_HIP_CALL_Y_INITIALISED) != 0;
     p.dry_atomic = dry;
+    p.force_streamk = -1;
     p.x = B;
     p.w = A;
     p.bias = bias;

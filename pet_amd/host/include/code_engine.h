@@ -51,6 +51,7 @@ class CodeEngine {
     int genCode(std::shared_ptr<SubGraph> &graph, const std::string &filename);
 
   private:
+    void importAlgos(const OpVec &order);
     std::shared_ptr<PerfEngine> perfEngine;
 };
 

@@ -204,6 +204,12 @@ class ConvOp : public Operator {
     Tensor *getBias() const { return bias; }
     void setAct(ActType a) { act = a; }
     ActType getAct() const { return act; }
+    // Which of the backend's PET_HIP_CONV_ALGO_COUNT ways of sharing out the K loop the
+    // launches use; perf() leaves the fastest one here (0: the library's cost model),
+    // CodeEngine takes it from an imported PerfEngine (the role of ConvResult::algo and
+    // PerfEngine::getConvAlgo in the reference, src/Graph/code_engine.cc:874-878).
+    void setAlgo(int a) { algo = a; }
+    int getAlgo() const { return algo; }
     bool same(const ConvOp &rhs);
     PaddingMode getPaddingMode() { return padding; }
     int getDh() const { return dh; }
@@ -226,6 +232,7 @@ class ConvOp : public Operator {
     Tensor *bias; // side pointer, not a graph edge
     ActType act;
     PaddingMode padding;
+    int algo = 0;
 };
 
 // ---- Conv3d (extension: the reference has no 3-D convolution) -----------------

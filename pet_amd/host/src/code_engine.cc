@@ -395,6 +395,19 @@ static AliasPlan planAliases(const OpVec &order) {
     return plan;
 }
 
+// Convolutions take the algorithm an imported PerfEngine found fastest for their
+// arguments (src/Graph/code_engine.cc:874-878 reads the cuDNN algorithm the same way).
+void CodeEngine::importAlgos(const OpVec &order) {
+    if (!perfEngine)
+        return;
+    for (auto op : order)
+        if (auto conv = dynamic_cast<ConvOp *>(op)) {
+            ConvArgs args = conv->getArgs(perfEngine->withPenalty());
+            if (perfEngine->checkOpPerf(Operator::Conv, args))
+                conv->setAlgo(perfEngine->getConvAlgo(args));
+        }
+}
+
 std::unique_ptr<GraphExec> CodeEngine::instantiate(std::shared_ptr<SubGraph> &graph) {
     if (!petInit())
         return nullptr;
@@ -425,6 +438,7 @@ std::unique_ptr<GraphExec> CodeEngine::instantiate(std::shared_ptr<SubGraph> &gr
             for (Tensor *t : {bn->getScale(), bn->getBias(), bn->getMean(), bn->getVar()})
                 t->devicePtr();
     }
+    importAlgos(order);
     AliasPlan plan = planAliases(order);
     TransposeChains rows = planTransposeChains(order, graph->getOutputs(), plan.skipped);
     FusedTails tails = planFusedTails(order, graph->getOutputs(), plan.skipped,
@@ -560,6 +574,7 @@ std::string CodeEngine::genCode(std::shared_ptr<SubGraph> &graph) {
     OpVec order;
     if (!graph->topoOrder(order))
         return "";
+    importAlgos(order);
     Emitter e;
     e.line("// Generated by tpm::CodeEngine for the MI355X backend.");
     e.line("// Build: hipcc -O2 prog.cpp -I<repo>/include -L<repo>/pet_amd/lib -lpet_hip "
@@ -681,7 +696,7 @@ std::string CodeEngine::genCode(std::shared_ptr<SubGraph> &graph) {
         }
         if (auto conv = dynamic_cast<ConvOp *>(op)) {
             auto d = op->getInputs()[0]->getDims(), w = op->getInputs()[1]->getDims();
-            const unsigned fl = flagsOf(op);
+            const unsigned fl = flagsOf(op) | PET_HIP_CONV_ALGO(conv->getAlgo());
             c << (fl     ? "pet_hip_conv2d_ex_f32("
                   : tail ? "pet_hip_conv2d_res_f32("
                          : "pet_hip_conv2d_f32(")

@@ -218,7 +218,7 @@ ConvOp::ConvOp(PaddingMode pm, int sh, int sw, int dh, int dw, Tensor *bias, Act
 
 ConvOp::ConvOp(const ConvOp &rhs)
     : Operator(rhs), ph(rhs.ph), pw(rhs.pw), sh(rhs.sh), sw(rhs.sw), dh(rhs.dh), dw(rhs.dw),
-      bias(rhs.bias), act(rhs.act), padding(rhs.padding) {}
+      bias(rhs.bias), act(rhs.act), padding(rhs.padding), algo(rhs.algo) {}
 
 void ConvOp::initHash() {
     hash = type;
@@ -301,6 +301,12 @@ int ConvOp::launch(pet_hip_stream_t stream) {
     // the reference's compute() returns nullptr when f % g != 0
     if (groups <= 0 || wt[0] % groups != 0)
         return PET_HIP_ERR_INVALID;
+    if (algo != 0)
+        return pet_hip_conv2d_ex_f32(inputs[0]->devicePtr(), inputs[1]->devicePtr(),
+                                     bias ? bias->devicePtr() : nullptr, nullptr,
+                                     outputs[0]->devicePtr(), in[0], in[1], in[2], in[3], wt[0],
+                                     wt[2], wt[3], ph, pw, sh, sw, dh, dw, groups, (int)act,
+                                     PET_HIP_CONV_ALGO(algo), stream);
     return pet_hip_conv2d_f32(inputs[0]->devicePtr(), inputs[1]->devicePtr(),
                               bias ? bias->devicePtr() : nullptr, outputs[0]->devicePtr(), in[0],
                               in[1], in[2], in[3], wt[0], wt[2], wt[3], ph, pw, sh, sw, dh, dw,
@@ -316,7 +322,7 @@ int ConvOp::launchFused(pet_hip_stream_t stream, const float *residual, ActType 
     return pet_hip_conv2d_ex_f32(inputs[0]->devicePtr(), inputs[1]->devicePtr(),
                                  bias ? bias->devicePtr() : nullptr, residual, out, in[0], in[1],
                                  in[2], in[3], wt[0], wt[2], wt[3], ph, pw, sh, sw, dh, dw, groups,
-                                 (int)finalAct, flags, stream);
+                                 (int)finalAct, flags | PET_HIP_CONV_ALGO(algo), stream);
 }
 
 bool ConvOp::accumulates() const {
@@ -331,8 +337,10 @@ bool ConvOp::accumulates() const {
 
 double ConvOp::perf(PerfEngine *pe, int rounds, int warmupRounds) {
     ConvArgs args = getArgs(pe->withPenalty());
-    if (pe->checkOpPerf(Conv, args))
+    if (pe->checkOpPerf(Conv, args)) {
+        algo = pe->getConvAlgo(args);
         return pe->getOpPerf(Conv, args);
+    }
     int n, c, h, w, f, r, s, ph_, pw_, sh_, sw_, dh_, dw_, g, bi, ac;
     std::tie(n, c, h, w, f, r, s, ph_, pw_, sh_, sw_, dh_, dw_, g, bi, ac) = args;
     ConvResult best{INFINITY, 0, 0, true};
@@ -344,17 +352,39 @@ double ConvOp::perf(PerfEngine *pe, int rounds, int warmupRounds) {
             float *wt = pe->getWeightPtr((size_t)f * (c / g) * r * s);
             float *y = pe->getOutputPtr((size_t)n * f * oh * ow);
             float *b = pe->getBiasPtr((size_t)f);
-            if (x && wt && y && b)
-                // bias and activation ride in the kernel's epilogue: one variant to time
-                best.time = timeFn(
-                    [&](pet_hip_stream_t st) {
-                        return pet_hip_conv2d_f32(x, wt, b, y, n, c, h, w, f, r, s, ph_, pw_, sh_,
-                                                  sw_, dh_, dw_, g, ac, st);
-                    },
-                    rounds, warmupRounds);
+            if (x && wt && y && b) {
+                // Bias and activation ride in the kernel's epilogue; what there is to choose
+                // is how the K loop is shared out (the reference loops over cuDNN's
+                // algorithms here, src/Graph/operator.cc:352-470). The cost model's choice
+                // is timed in full; another algorithm has to beat it by 3 % on a shorter
+                // run, then confirm on a full one, to be taken.
+                auto run = [&](int a, int rds, int warm) {
+                    return timeFn(
+                        [&](pet_hip_stream_t st) {
+                            return pet_hip_conv2d_ex_f32(x, wt, b, nullptr, y, n, c, h, w, f, r, s,
+                                                         ph_, pw_, sh_, sw_, dh_, dw_, g, ac,
+                                                         PET_HIP_CONV_ALGO(a), st);
+                        },
+                        rds, warm);
+                };
+                best.time = run(0, rounds, warmupRounds);
+                static const bool tune = getenv("PET_HOST_NO_ALGO_SEARCH") == nullptr;
+                const int quick = std::max(10, rounds / 4);
+                for (int a = 1; tune && a < PET_HIP_CONV_ALGO_COUNT; ++a) {
+                    double t = run(a, quick, std::min(warmupRounds, 10));
+                    if (!(t < 0.97 * best.time))
+                        continue;
+                    t = run(a, rounds, std::min(warmupRounds, 20));
+                    if (t < 0.97 * best.time) {
+                        best.time = t;
+                        best.algo = a;
+                    }
+                }
+            }
         }
     }
     pe->saveOpPerf(Conv, args, best);
+    algo = best.algo;
     return best.time;
 }
 

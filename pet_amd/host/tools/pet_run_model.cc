@@ -2,7 +2,9 @@
 // would: Graph -> SubGraph -> CodeEngine::instantiate (HIP graph) -> replay.
 //
 //   pet_run_model <dilated|dilated:pet|resnet18|bert|resnet3d18> [--rounds N] [--warmup N]
-//                 [--check] [--emit file.cpp]
+//                 [--check] [--tune] [--emit file.cpp]
+// --tune: Operator::perf on every operator first (what the search does); convolutions then
+// run with the algorithm that timed fastest for their arguments.
 //
 // Prints one JSON line: model, ms per replay, GFLOP, TFLOP/s, kernels in the
 // captured graph, operators that cost no kernel (storage sharing, folded
@@ -59,11 +61,11 @@ static bool fillInputs(SubGraph &sg, Graph &owner) {
 
 int main(int argc, char **argv) {
     if (argc < 2) {
-        std::fprintf(stderr, "usage: %s model [--rounds N] [--warmup N] [--check] [--emit f]\n", argv[0]);
+        std::fprintf(stderr, "usage: %s model [--rounds N] [--warmup N] [--check] [--tune] [--emit f]\n", argv[0]);
         return 2;
     }
     int rounds = 200, warmup = 20;
-    bool check = false;
+    bool check = false, tune = false;
     std::string emit;
     for (int i = 2; i < argc; ++i) {
         if (!std::strcmp(argv[i], "--rounds") && i + 1 < argc)
@@ -72,6 +74,8 @@ int main(int argc, char **argv) {
             warmup = std::atoi(argv[++i]);
         else if (!std::strcmp(argv[i], "--check"))
             check = true;
+        else if (!std::strcmp(argv[i], "--tune"))
+            tune = true;
         else if (!std::strcmp(argv[i], "--emit") && i + 1 < argc)
             emit = argv[++i];
     }
@@ -99,6 +103,15 @@ int main(int argc, char **argv) {
         sg->resetComputed();
     }
     CodeEngine ce;
+    int tuned = 0;
+    if (tune) {
+        auto pe = std::make_shared<PerfEngine>();
+        sg->perf(pe.get(), false);
+        ce.importPerfEngine(pe);
+        for (auto op : sg->getOperators())
+            if (auto conv = dynamic_cast<ConvOp *>(op))
+                tuned += conv->getAlgo() != 0;
+    }
     auto exec = ce.instantiate(sg);
     if (!exec) {
         std::fprintf(stderr, "instantiate failed: %s\n", pet_hip_last_error());
@@ -127,6 +140,8 @@ int main(int argc, char **argv) {
                 m.name.c_str(), ms, m.gflop, m.gflop / ms, sg->getOperators().size(),
                 exec->numKernelOps(), exec->numAliasedOps(), exec->numFoldedOps(),
                 exec->numHoistedFills());
+    if (tune)
+        std::printf(", \"convs_off_default_algo\": %d", tuned);
     if (check)
         std::printf(", \"max_abs_diff_vs_eager\": %.3g, \"max_abs_eager\": %.3g", maxDiff, maxRef);
     std::printf("}\n");

@@ -446,6 +446,18 @@ static bool test_perf_engine_memo() {
     EXPECT(pe.checkOpPerf(Operator::Conv, conv.getArgs(pe.withPenalty())));
     double t2 = conv.perf(&pe, 20, 5);
     EXPECT(t1 == t2); // memo hit
+    // the search over the backend's algorithms left its choice on the operator and in
+    // the memo; a copy of the operator picks it up from there
+    EXPECT(conv.getAlgo() >= 0 && conv.getAlgo() < PET_HIP_CONV_ALGO_COUNT);
+    EXPECT(pe.getConvAlgo(conv.getArgs(pe.withPenalty())) == conv.getAlgo());
+    {
+        Tensor oc;
+        ConvOp again(&i0, &w0, &oc, 1, 1);
+        EXPECT(again.perf(&pe, 20, 5) == t1 && again.getAlgo() == conv.getAlgo());
+        again.setAlgo(3); // four workgroups per tile: same result as the default
+        EXPECT(again.compute() != nullptr && conv.compute() != nullptr);
+        EXPECT(equalArrays(oc.getDataPtr(), o0.getDataPtr(), o0.size()));
+    }
     // penalty rows change the key and the measured shape
     i0.addPenalty(2, 1);
     double t3 = conv.perf(&pe, 20, 5);

@@ -726,6 +726,27 @@ def test_cross_launch_fusion_flags(ops):
         assert host(y).tobytes() == want_r.tobytes(), (bb, m, n, k)
 
 
+def test_convolution_algorithms_agree(ops):
+    """PET_HIP_CONV_ALGO(0..7): every way of sharing out the K loop gives the same sums
+    (bit for bit on small integers), on shapes that split, that stream and that do
+    neither; an unknown algorithm is refused."""
+    rng = np.random.default_rng(31)
+    cases = [((1, 64, 56, 56), (64, 64, 3, 3), 1, 1), ((1, 512, 7, 7), (512, 512, 3, 3), 1, 1),
+             ((4, 128, 32, 32), (64, 128, 3, 3), 1, 1), ((1, 128, 28, 28), (256, 128, 1, 1), 0, 2),
+             ((2, 3, 30, 30), (16, 3, 7, 7), 3, 2), ((1, 16, 9, 11), (8, 16, 3, 3), 2, 1)]
+    for xs, ws, pad, st in cases:
+        x = rng.integers(-3, 4, xs).astype(np.float32)
+        w = rng.integers(-3, 4, ws).astype(np.float32)
+        b = rng.integers(-3, 4, (ws[0],)).astype(np.float32)
+        dx, dw_, db = dev(x), dev(w), dev(b)
+        want = host(ops.conv2d(dx, dw_, pad, pad, st, st, bias=db, act="relu"))
+        for algo in range(1, 8):
+            got = host(ops.conv2d(dx, dw_, pad, pad, st, st, bias=db, act="relu", flags=algo << 8))
+            assert got.tobytes() == want.tobytes(), (xs, ws, algo)
+    with pytest.raises(Exception):
+        ops.conv2d(dx, dw_, pad, pad, st, st, flags=8 << 8)
+
+
 def test_pow_div_batchnorm(ops):
     """PowOp: bit-exact (the same chain of fp32 products as the CPU loop). Div:
     division proper, correctly rounded like numpy's. BatchNorm: 1e-5 relative
