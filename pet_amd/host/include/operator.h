@@ -262,6 +262,9 @@ class Conv3dOp : public Operator {
     int numOutputs() override { return 1; }
     void setAct(ActType a) { act = a; }
     ActType getAct() const { return act; }
+    // as ConvOp::setAlgo; perf() leaves the fastest of the backend's algorithms here
+    void setAlgo(int a) { algo = a; }
+    int getAlgo() const { return algo; }
     Tensor *getBias() const { return bias; }
     const Dim &getPad() const { return pad; }
     const Dim &getStride() const { return stride; }
@@ -276,6 +279,7 @@ class Conv3dOp : public Operator {
     float *packed = nullptr;     // kt-major filters, owned
     size_t packedElems = 0;
     uint64_t packedVersion = 0;  // weight tensor's dataVersion() the copy was made from
+    int algo = 0;
 };
 
 // ---- Matmul -------------------------------------------------------------------

@@ -421,7 +421,7 @@ Conv3dOp::Conv3dOp(Tensor *input, Tensor *weight, Tensor *output, const Dim &pad
 
 Conv3dOp::Conv3dOp(const Conv3dOp &rhs)
     : Operator(rhs), pad(rhs.pad), stride(rhs.stride), dilation(rhs.dilation), bias(rhs.bias),
-      act(rhs.act) {}
+      act(rhs.act), algo(rhs.algo) {}
 
 Conv3dOp::~Conv3dOp() {
     if (packed)
@@ -489,6 +489,8 @@ int Conv3dOp::launch(pet_hip_stream_t stream) {
     int groups = in[1] / wt[1];
     if (groups <= 0 || wt[0] % groups != 0)
         return PET_HIP_ERR_INVALID;
+    if (algo != 0)
+        return launchFused(stream, nullptr, act, outputs[0]->devicePtr(), 0);
     const float *w = inputs[1]->devicePtr();
     auto entry = pet_hip_conv3d_f32;
     if (usesPackedFilters()) {
@@ -513,7 +515,7 @@ int Conv3dOp::launchFused(pet_hip_stream_t stream, const float *residual, ActTyp
                                  in[0], in[1], in[2], in[3], in[4], wt[0], wt[2], wt[3], wt[4],
                                  pad[0], pad[1], pad[2], stride[0], stride[1], stride[2],
                                  dilation[0], dilation[1], dilation[2], groups, (int)finalAct,
-                                 flags, stream);
+                                 flags | PET_HIP_CONV_ALGO(algo), stream);
 }
 
 bool Conv3dOp::accumulates() const {
@@ -528,8 +530,30 @@ bool Conv3dOp::accumulates() const {
            yes != 0;
 }
 
+// The same search as ConvOp::perf, on the operator's own tensors (there is no memo for
+// 3-D arguments: the reference has no such operator).
 double Conv3dOp::perf(PerfEngine *, int rounds, int warmupRounds) {
-    return timeLaunches(rounds, warmupRounds);
+    algo = 0;
+    // time what the graph runtime will run: constant filters in their kt-major copy
+    if (petInit() && inputs[1]->getType() == Tensor::Weight && inputs[1]->devicePtr())
+        prepackFilters(petStream());
+    double best = timeLaunches(rounds, warmupRounds);
+    static const bool tune = getenv("PET_HOST_NO_ALGO_SEARCH") == nullptr;
+    int bestAlgo = 0;
+    const int quick = std::max(10, rounds / 4);
+    for (int a = 1; tune && std::isfinite(best) && a < PET_HIP_CONV_ALGO_COUNT; ++a) {
+        algo = a;
+        double t = timeLaunches(quick, std::min(warmupRounds, 10));
+        if (!(t < 0.97 * best))
+            continue;
+        t = timeLaunches(rounds, std::min(warmupRounds, 20));
+        if (t < 0.97 * best) {
+            best = t;
+            bestAlgo = a;
+        }
+    }
+    algo = bestAlgo;
+    return best;
 }
 
 std::string Conv3dOp::toString() const {

@@ -111,6 +111,8 @@ int main(int argc, char **argv) {
         for (auto op : sg->getOperators())
             if (auto conv = dynamic_cast<ConvOp *>(op))
                 tuned += conv->getAlgo() != 0;
+            else if (auto c3 = dynamic_cast<Conv3dOp *>(op))
+                tuned += c3->getAlgo() != 0;
     }
     auto exec = ce.instantiate(sg);
     if (!exec) {
