@@ -194,7 +194,9 @@ PET_HIP_API int pet_hip_bmm_res_f32(int transA, int transB, int b, int m, int n,
                         const float *B, float *C, const float *bias, const float *residual,
                         int act, pet_hip_stream_t stream);
 
-/* Matmul with every optional operand; flags: PET_HIP_CALL_Y_INITIALISED only. */
+/* Matmul with every optional operand; flags: PET_HIP_CALL_Y_INITIALISED and
+ * PET_HIP_CONV_ALGO(a) (the same K-sharing algorithms; transposed operands and k not a
+ * multiple of 32 run on the general kernel, which has one). */
 PET_HIP_API int pet_hip_bmm_ex_f32(int transA, int transB, int b, int m, int n, int k, const float *A,
                        const float *B, float *C, const float *bias, const float *residual, int act,
                        unsigned flags, pet_hip_stream_t stream);

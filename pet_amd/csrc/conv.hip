@@ -1153,6 +1153,14 @@ int launch_conv(ConvParams &p, hipStream_t stream) {
     }
 }
 
+// Algorithm override (PET_HIP_CONV_ALGO, 0: the cost model decides): forced K shares per
+// tile and / or stream-K on or off.
+void apply_algo(ConvParams &p, unsigned algo) {
+    static const int kSplit[PET_HIP_CONV_ALGO_COUNT] = {0, 1, 2, 4, 8, 16, 0, 0};
+    p.force_splitk = algo < PET_HIP_CONV_ALGO_COUNT ? kSplit[algo] : 0;
+    p.force_streamk = algo == 0 ? -1 : (algo == 6 ? 1 : 0);
+}
+
 int conv_common(const float *x, const float *w, const float *bias, float *y, int n, int c, int t,
                 int h, int wd, int f, int kt, int r, int s, int pt, int ph, int pw, int st, int sh,
                 int sw, int dt, int dh, int dw, int groups, int act, hipStream_t stream,
@@ -1238,21 +1246,10 @@ int conv_common(const float *x, const float *w, const float *bias, float *y, int
     p.y_init = (flags & PET_HIP_CALL_Y_INITIALISED) != 0;
     p.defer_relu = (flags & PET_HIP_CALL_DEFER_RELU) != 0;
     p.dry_atomic = dry;
-    p.force_streamk = -1;
-    {
-        // algorithm override, bits 8-15 of the flags (0: the cost model decides)
-        static const int kSplit[] = {0, 1, 2, 4, 8, 16, 0, 0};
-        const unsigned algo = (flags >> 8) & 0xffu;
-        if (algo >= PET_HIP_CONV_ALGO_COUNT)
-            return set_error(PET_HIP_ERR_INVALID, "unknown convolution algorithm %u", algo);
-        p.force_splitk = kSplit[algo];
-        if (algo >= 1 && algo <= 5)
-            p.force_streamk = 0;
-        else if (algo == 6)
-            p.force_streamk = 1;
-        else if (algo == 7)
-            p.force_streamk = 0;
-    }
+    if (((flags >> 8) & 0xffu) >= PET_HIP_CONV_ALGO_COUNT)
+        return set_error(PET_HIP_ERR_INVALID, "unknown convolution algorithm %u",
+                         (flags >> 8) & 0xffu);
+    apply_algo(p, (flags >> 8) & 0xffu);
     p.wpacked = wpacked;
     if (wpacked && !packed_filters_apply(f, c / groups, kt, r, s))
         return set_error(PET_HIP_ERR_UNSUPPORTED, "no kt-major form for this filter shape");
@@ -1285,7 +1282,7 @@ int bmm_as_grouped_1x1(const float *A, const float *B, float *C, const float *bi
     memset(&p, 0, sizeof(p));
     p.y_init = (flags & PET_HIP_CALL_Y_INITIALISED) != 0;
     p.dry_atomic = dry;
-    p.force_streamk = -1;
+    apply_algo(p, (flags >> 8) & 0xffu);
     p.x = B;
     p.w = A;
     p.bias = bias;

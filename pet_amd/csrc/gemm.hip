@@ -155,8 +155,11 @@ namespace {
 int bmm_common(int transA, int transB, int b, int m, int n, int k, const float *A, const float *B,
                float *C, const float *bias, const float *res, int act, pet_hip_stream_t stream,
                unsigned flags = 0, int *dry = nullptr) {
-    if (flags & ~(unsigned)PET_HIP_CALL_Y_INITIALISED)
-        return set_error(PET_HIP_ERR_INVALID, "matmul takes PET_HIP_CALL_Y_INITIALISED only");
+    if (flags & ~(unsigned)(PET_HIP_CALL_Y_INITIALISED | 0xff00u))
+        return set_error(PET_HIP_ERR_INVALID,
+                         "matmul takes PET_HIP_CALL_Y_INITIALISED and an algorithm only");
+    if (((flags >> 8) & 0xffu) >= PET_HIP_CONV_ALGO_COUNT)
+        return set_error(PET_HIP_ERR_INVALID, "unknown algorithm %u", (flags >> 8) & 0xffu);
     if (dry) {
         *dry = 0;
         A = B = reinterpret_cast<const float *>(uintptr_t(256));

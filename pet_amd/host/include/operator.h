@@ -291,7 +291,11 @@ class MatmulOp : public Operator {
              Tensor *bias = nullptr, ActType act = None);
     MatmulOp(bool transA = false, bool transB = false, Tensor *bias = nullptr, ActType act = None);
     MatmulOp(const MatmulOp &rhs)
-        : Operator(rhs), transA(rhs.transA), transB(rhs.transB), bias(rhs.bias), act(rhs.act) {}
+        : Operator(rhs), transA(rhs.transA), transB(rhs.transB), bias(rhs.bias), act(rhs.act),
+          algo(rhs.algo) {}
+    // as ConvOp::setAlgo (MatmulResult::algo, PerfEngine::getMatmulAlgo)
+    void setAlgo(int a) { algo = a; }
+    int getAlgo() const { return algo; }
     MatmulOp *clone() override { return new MatmulOp(*this); }
     // One output point -> the input points it depends on; the closure runs the
     // whole operator on the device.
@@ -323,6 +327,7 @@ class MatmulOp : public Operator {
     bool transA, transB;
     Tensor *bias;
     ActType act;
+    int algo = 0;
 };
 
 // ---- band matrix products (declared, not executed) --------------------------------

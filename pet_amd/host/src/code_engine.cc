@@ -405,6 +405,10 @@ void CodeEngine::importAlgos(const OpVec &order) {
             ConvArgs args = conv->getArgs(perfEngine->withPenalty());
             if (perfEngine->checkOpPerf(Operator::Conv, args))
                 conv->setAlgo(perfEngine->getConvAlgo(args));
+        } else if (auto mm = dynamic_cast<MatmulOp *>(op)) {
+            MatmulArgs args = mm->getArgs();
+            if (perfEngine->checkOpPerf(Operator::Matmul, args))
+                mm->setAlgo(perfEngine->getMatmulAlgo(args));
         }
 }
 
@@ -741,7 +745,7 @@ std::string CodeEngine::genCode(std::shared_ptr<SubGraph> &graph) {
             bool ta, tb;
             int b, m, n, k;
             std::tie(ta, tb, b, m, n, k) = mm->getArgs();
-            const unsigned fl = flagsOf(op);
+            const unsigned fl = flagsOf(op) | PET_HIP_CONV_ALGO(mm->getAlgo());
             c << (fl     ? "pet_hip_bmm_ex_f32("
                   : tail ? "pet_hip_bmm_res_f32("
                          : "pet_hip_bmm_f32(")

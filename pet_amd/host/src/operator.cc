@@ -641,6 +641,8 @@ int MatmulOp::launch(pet_hip_stream_t stream) {
     bool ta, tb;
     int b, m, n, k;
     std::tie(ta, tb, b, m, n, k) = getArgs();
+    if (algo != 0)
+        return launchFused(stream, nullptr, act, outputs[0]->devicePtr(), 0);
     return pet_hip_bmm_f32(ta, tb, b, m, n, k, inputs[0]->devicePtr(), inputs[1]->devicePtr(),
                            outputs[0]->devicePtr(), bias ? bias->devicePtr() : nullptr, (int)act,
                            stream);
@@ -655,7 +657,7 @@ int MatmulOp::launchFused(pet_hip_stream_t stream, const float *residual, ActTyp
     std::tie(ta, tb, b, m, n, k) = getArgs();
     return pet_hip_bmm_ex_f32(ta, tb, b, m, n, k, inputs[0]->devicePtr(), inputs[1]->devicePtr(),
                               out, bias ? bias->devicePtr() : nullptr, residual, (int)finalAct,
-                              flags, stream);
+                              flags | PET_HIP_CONV_ALGO(algo), stream);
 }
 
 bool MatmulOp::accumulates() const {
@@ -667,21 +669,43 @@ bool MatmulOp::accumulates() const {
 
 double MatmulOp::perf(PerfEngine *pe, int rounds, int warmupRounds) {
     MatmulArgs args = getArgs();
-    if (pe->checkOpPerf(Matmul, args))
+    if (pe->checkOpPerf(Matmul, args)) {
+        algo = pe->getMatmulAlgo(args);
         return pe->getOpPerf(Matmul, args);
+    }
     bool ta, tb;
     int b, m, n, k;
     std::tie(ta, tb, b, m, n, k) = args;
     float *A = pe->getMatA((size_t)b * m * k), *B = pe->getMatB((size_t)b * k * n);
     float *C = pe->getMatC((size_t)b * m * n);
     MatmulResult best{INFINITY, true, 0};
-    if (A && B && C)
-        best.time = timeFn(
-            [&](pet_hip_stream_t st) {
-                return pet_hip_bmm_f32(ta, tb, b, m, n, k, A, B, C, nullptr, (int)act, st);
-            },
-            rounds, warmupRounds);
+    if (A && B && C) {
+        // the search of ConvOp::perf (the reference loops over cuBLAS algorithms here,
+        // src/Graph/operator.cc:756-815)
+        auto run = [&](int a, int rds, int warm) {
+            return timeFn(
+                [&](pet_hip_stream_t st) {
+                    return pet_hip_bmm_ex_f32(ta, tb, b, m, n, k, A, B, C, nullptr, nullptr,
+                                              (int)act, PET_HIP_CONV_ALGO(a), st);
+                },
+                rds, warm);
+        };
+        best.time = run(0, rounds, warmupRounds);
+        static const bool tune = getenv("PET_HOST_NO_ALGO_SEARCH") == nullptr;
+        const int quick = std::max(10, rounds / 4);
+        for (int a = 1; tune && !ta && !tb && k % 32 == 0 && a < PET_HIP_CONV_ALGO_COUNT; ++a) {
+            double t = run(a, quick, std::min(warmupRounds, 10));
+            if (!(t < 0.97 * best.time))
+                continue;
+            t = run(a, rounds, std::min(warmupRounds, 20));
+            if (t < 0.97 * best.time) {
+                best.time = t;
+                best.algo = a;
+            }
+        }
+    }
     pe->saveOpPerf(Matmul, args, best);
+    algo = best.algo;
     return best.time;
 }
 

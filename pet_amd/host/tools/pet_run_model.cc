@@ -113,6 +113,8 @@ int main(int argc, char **argv) {
                 tuned += conv->getAlgo() != 0;
             else if (auto c3 = dynamic_cast<Conv3dOp *>(op))
                 tuned += c3->getAlgo() != 0;
+            else if (auto mm = dynamic_cast<MatmulOp *>(op))
+                tuned += mm->getAlgo() != 0;
     }
     auto exec = ce.instantiate(sg);
     if (!exec) {
@@ -143,7 +145,7 @@ int main(int argc, char **argv) {
                 exec->numKernelOps(), exec->numAliasedOps(), exec->numFoldedOps(),
                 exec->numHoistedFills());
     if (tune)
-        std::printf(", \"convs_off_default_algo\": %d", tuned);
+        std::printf(", \"off_default_algo\": %d", tuned);
     if (check)
         std::printf(", \"max_abs_diff_vs_eager\": %.3g, \"max_abs_eager\": %.3g", maxDiff, maxRef);
     std::printf("}\n");
