@@ -393,15 +393,19 @@ def main():
     if not args.no_configs and os.path.exists(run_model):
         import subprocess
         torch.cuda.synchronize()
+        # plain, and with --tune: Operator::perf on every operator first, so that each
+        # contraction runs with the algorithm that timed fastest for it (what PET's search
+        # leaves in its PerfEngine)
         for model in ("dilated:pet", "dilated", "resnet18", "bert", "resnet3d18"):
-            try:
-                res = subprocess.run([run_model, model, "--rounds", str(max(50, args.steps)),
-                                      "--warmup", "10"], capture_output=True, text=True,
-                                     timeout=300)
-                host_path[model] = (json.loads(res.stdout.strip().splitlines()[-1])
-                                    if res.returncode == 0 else {"error": res.stderr[-200:]})
-            except Exception as exc:
-                host_path[model] = {"error": str(exc)[:200]}
+            for key, extra in ((model, []), (model + " tuned", ["--tune"])):
+                try:
+                    res = subprocess.run([run_model, model, "--rounds", str(max(50, args.steps)),
+                                          "--warmup", "10"] + extra, capture_output=True,
+                                         text=True, timeout=300)
+                    host_path[key] = (json.loads(res.stdout.strip().splitlines()[-1])
+                                      if res.returncode == 0 else {"error": res.stderr[-200:]})
+                except Exception as exc:
+                    host_path[key] = {"error": str(exc)[:200]}
 
     dom_flop = conv_flop(DIL * DIL, 512, hs, hs, 512, 3, 3)
     dom_ms = conv_ms[0]

@@ -934,13 +934,28 @@ int launch_plane_cfg(ConvParams p, hipStream_t stream) {
     int splitk = 1;
     const double scale = (double)(Cfg::BM * Cfg::BN) / (64.0 * 64.0);
     const double c_fixed = 3.0 / scale, c_launches = 4.0 / scale, c_contend = 0.1 / scale;
-    double best = ((tiles + 255) / 256) * (nit + c_fixed); // S = 1
-    if (tiles < 256 && nit >= 4) {
+    // A workgroup that has its CU to itself (one wave per SIMD) has nothing to hide its LDS
+    // and barrier waits behind: its steps cost about an eighth more than those of two
+    // co-resident workgroups, whose prologues and epilogues also overlap. (Measured by the
+    // host layer's algorithm search: 256 tiles of 64 steps run faster as 512 workgroups of 32.)
+    static const double solo = getenv("PET_HIP_SOLO_COST") ? atof(getenv("PET_HIP_SOLO_COST")) : 1.12;
+    // ... on long K loops; short ones are bound by their launches either way
+    static const int solo_steps = getenv("PET_HIP_SOLO_STEPS") ? atoi(getenv("PET_HIP_SOLO_STEPS")) : 12;
+    const long long r1 = (tiles + 255) / 256;
+    const bool legacy = solo <= 0.0; // the model before the occupancy terms (for comparison)
+    double best = legacy ? r1 * (nit + c_fixed)
+                         : r1 * nit * (r1 == 1 && nit >= solo_steps ? solo : 1.0) +
+                               ((r1 + 1) / 2) * c_fixed; // S = 1
+    if ((legacy ? tiles < 256 : tiles <= 256) && nit >= 4) {
         static const int max_env =
             getenv("PET_HIP_SPLITK_MAX") ? atoi(getenv("PET_HIP_SPLITK_MAX")) : 64;
         for (int S = 1; S <= std::min(nit / 2, max_env); ++S) {
-            const double rounds = (double)((tiles * S + 255) / 256);
-            double cost = rounds * ((nit + S - 1) / S + c_fixed);
+            const long long rounds = (tiles * S + 255) / 256;
+            double cost = legacy ? rounds * ((nit + S - 1) / S + c_fixed)
+                                 : rounds * ((nit + S - 1) / S) *
+                                           (rounds == 1 && (nit + S - 1) / S >= solo_steps ? solo
+                                                                                           : 1.0) +
+                                       ((rounds + 1) / 2) * c_fixed;
             if (S > 1)
                 cost += c_launches + c_contend * S;
             if (S == 1 || cost < best) {

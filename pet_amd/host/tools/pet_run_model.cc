@@ -109,8 +109,11 @@ int main(int argc, char **argv) {
         sg->perf(pe.get(), false);
         ce.importPerfEngine(pe);
         for (auto op : sg->getOperators())
-            if (auto conv = dynamic_cast<ConvOp *>(op))
+            if (auto conv = dynamic_cast<ConvOp *>(op)) {
                 tuned += conv->getAlgo() != 0;
+                if (conv->getAlgo() != 0 && getenv("PET_HOST_TRACE"))
+                    std::fprintf(stderr, "algo %d: %s\n", conv->getAlgo(), op->toString().c_str());
+            }
             else if (auto c3 = dynamic_cast<Conv3dOp *>(op))
                 tuned += c3->getAlgo() != 0;
             else if (auto mm = dynamic_cast<MatmulOp *>(op))
