@@ -327,6 +327,27 @@ def test_model_graph_replay_equals_operator_by_operator_run(model):
         assert rec["folded"] == 2 and rec["kernels"] == 8
 
 
+@pytest.mark.gpu
+@pytest.mark.parametrize("model", ["resnet18", "bert"])
+def test_model_graph_with_searched_algorithms(model):
+    """pet_run_model --tune --check: Operator::perf searches the backend's algorithms for
+    every contraction first; the graph then runs with what was found and still agrees
+    with the operator-by-operator run. With the search switched off nothing leaves the
+    default."""
+    import json
+    res = subprocess.run([RUN_MODEL, model, "--tune", "--check", "--rounds", "20", "--warmup", "3"],
+                         capture_output=True, text=True, timeout=600)
+    assert res.returncode == 0, res.stderr[-2000:]
+    rec = json.loads(res.stdout.strip().splitlines()[-1])
+    assert rec["max_abs_diff_vs_eager"] <= 1e-4 * rec["max_abs_eager"]
+    assert 0 <= rec["off_default_algo"] <= rec["operators"]
+    env = dict(os.environ, PET_HOST_NO_ALGO_SEARCH="1")
+    res = subprocess.run([RUN_MODEL, model, "--tune", "--rounds", "5", "--warmup", "2"],
+                         capture_output=True, text=True, timeout=600, env=env)
+    assert res.returncode == 0, res.stderr[-2000:]
+    assert json.loads(res.stdout.strip().splitlines()[-1])["off_default_algo"] == 0
+
+
 def _cpp_module():
     import glob
     import importlib
