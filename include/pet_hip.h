@@ -110,6 +110,8 @@ PET_HIP_API int pet_hip_device_info(char *arch, size_t arch_len, int *num_cu);
  * (src/Graph/operator.cc:296-515 loops over the algorithms). Environment variable
  * PET_HIP_DETERMINISTIC=1 sets the initial value. */
 PET_HIP_API int pet_hip_set_deterministic(int on);
+/* *on receives the current setting (for callers that switch it for a while) */
+PET_HIP_API int pet_hip_get_deterministic(int *on);
 
 /* ---- memory (cudaMalloc / cudaMemcpy / cudaFree call sites,
  * src/Graph/perf_engine.cc:31-47, src/Graph/code_engine.cc:560-643) ---------- */
@@ -162,6 +164,22 @@ PET_HIP_API int pet_hip_conv2d_f32(const float *x, const float *w, const float *
                        int n, int c, int h, int wd, int f, int r, int s, int ph, int pw,
                        int sh, int sw, int dh, int dw, int groups, int act,
                        pet_hip_stream_t stream);
+
+/* pet_hip_conv2d_f32 for callers that cannot allocate device memory or have it
+ * allocated on their behalf (code under HIP graph capture, tight serving loops,
+ * harnesses that forbid hipMalloc). It has no counterpart in the reference. Same
+ * arguments and results as pet_hip_conv2d_f32 in its run-to-run reproducible form
+ * (partial sums of a split K loop added in a fixed order); the partial tiles live in
+ * a static 8 MiB device array inside the library instead of the scratch that
+ * pet_hip_init allocates, and the call itself allocates and frees nothing. A shape
+ * whose split needs more than 8 MiB of partial tiles or more than 4096 output tiles
+ * returns PET_HIP_ERR_UNSUPPORTED with the sizes in pet_hip_last_error(). All calls on
+ * one GPU share that GPU's array: calls that overlap on one GPU (two streams, two
+ * threads) race. */
+PET_HIP_API int pet_hip_conv2d_static_f32(const float *x, const float *w, const float *bias,
+                                          float *y, int n, int c, int h, int wd, int f, int r,
+                                          int s, int ph, int pw, int sh, int sw, int dh, int dw,
+                                          int groups, int act, pet_hip_stream_t stream);
 
 /* Conv3d, NCTHW x [n,c,t,h,w], weight [f, c/groups, kt, r, s]. The reference
  * snapshot has no 3-D convolution (Operator::OpType, include/operator.h:19-51);
@@ -359,8 +377,10 @@ PET_HIP_API int pet_hip_bias_act(const float *x, const float *bias, float *y, si
 
 /* ---- non-contraction network pieces without a reference CPU compute -------*/
 
-/* Max (mode 0) / average (mode 1, divisor kh*kw) pooling over NCHW with
- * out = (in + 2p - d (k-1) - 1) / s + 1; replaces cudnnPoolingForward
+/* Max (mode 0) / average (mode 1) pooling over NCHW with
+ * out = (in + 2p - d (k-1) - 1) / s + 1. The average divides by the number of
+ * window positions inside the image (CUDNN_POOLING_AVERAGE_COUNT_EXCLUDE_PADDING,
+ * src/Graph/operator.cc:2933). Replaces cudnnPoolingForward
  * (src/Graph/operator.cc:2814-2827, 2937-2950; code_engine.cc:1315-1329). */
 PET_HIP_API int pet_hip_pool2d(const float *x, float *y, int n, int c, int h, int w, int kh, int kw,
                    int ph, int pw, int sh, int sw, int dh, int dw, int mode,

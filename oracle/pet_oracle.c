@@ -202,8 +202,9 @@ PET_ORACLE_EXPORT void oracle_bias_act_f32(const float *x, const float *bias,
 
 /* Max / average pooling over NCHW, cudnnPoolingForward semantics as used at
  * src/Graph/operator.cc:2814-2827, 2937-2950: out = (in + 2p - d*(k-1) - 1)/s + 1,
- * average counts padded zeros in the divisor
- * (CUDNN_POOLING_AVERAGE_COUNT_INCLUDE_PADDING). mode 0 = max, 1 = avg. */
+ * the average divides by the number of window positions inside the image
+ * (CUDNN_POOLING_AVERAGE_COUNT_EXCLUDE_PADDING, src/Graph/operator.cc:2933,
+ * src/Graph/code_engine.cc:1303). mode 0 = max, 1 = avg. */
 PET_ORACLE_EXPORT void oracle_pool2d_f32(const float *x, float *y, int n, int c,
                                          int h, int w, int kh, int kw, int ph,
                                          int pw, int sh, int sw, int dh, int dw,
@@ -215,6 +216,7 @@ PET_ORACLE_EXPORT void oracle_pool2d_f32(const float *x, float *y, int n, int c,
         for (int i = 0; i < oh; ++i)
             for (int j = 0; j < ow; ++j) {
                 double acc = mode == 0 ? -INFINITY : 0.0;
+                int taps = 0;
                 for (int r = 0; r < kh; ++r)
                     for (int s = 0; s < kw; ++s) {
                         int ih = i * sh + r * dh - ph, iw = j * sw + s * dw - pw;
@@ -225,9 +227,10 @@ PET_ORACLE_EXPORT void oracle_pool2d_f32(const float *x, float *y, int n, int c,
                             acc = v > acc ? v : acc;
                         else
                             acc += v;
+                        ++taps;
                     }
                 yp[(size_t)i * ow + j] =
-                    mode == 0 ? (float)acc : (float)(acc / (double)(kh * kw));
+                    mode == 0 ? (float)acc : (float)(taps ? acc / (double)taps : 0.0);
             }
     }
 }

@@ -32,6 +32,7 @@ SIGNATURES = {
     "pet_hip_shutdown": [],
     "pet_hip_device_info": [ctypes.c_char_p, _sz, _c_int_p],
     "pet_hip_set_deterministic": [ctypes.c_int],
+    "pet_hip_get_deterministic": [_c_int_p],
     "pet_hip_malloc": [ctypes.POINTER(_vp), _sz],
     "pet_hip_free": [_vp],
     "pet_hip_memcpy_h2d": [_vp, _vp, _sz, _vp],
@@ -53,6 +54,7 @@ SIGNATURES = {
     "pet_hip_graph_destroy": [_vp],
     "pet_hip_conv_out_dim": [_i] * 5,
     "pet_hip_conv2d_f32": [_vp] * 4 + [_i] * 15 + [_vp],
+    "pet_hip_conv2d_static_f32": [_vp] * 4 + [_i] * 15 + [_vp],
     "pet_hip_conv3d_f32": [_vp] * 4 + [_i] * 20 + [_vp],
     "pet_hip_conv2d_res_f32": [_vp] * 5 + [_i] * 15 + [_vp],
     "pet_hip_conv3d_res_f32": [_vp, _vp, _i, _vp, _vp, _vp] + [_i] * 20 + [_vp],

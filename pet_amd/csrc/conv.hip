@@ -55,6 +55,8 @@ struct ConvParams {
     int *dry_atomic; // not null: report whether the launch would accumulate into y, launch nothing
     int force_splitk;  // > 0: this many K shares per tile instead of the cost model's choice
     int force_streamk; // 0 / 1: stream-K off / on instead of the cost model's choice; -1: model
+    int static_ws;   // split-K partial tiles and counters live in this file's static device
+                     // array (the entry point that allocates nothing); implies the ordered sum
     int res_first;   // accumulating launch into an initialised y: the workgroup that holds a
                      // tile's first K step adds the residual along with its partial sums
     FastDiv fd_krs, fd_rs, fd_s;     // k -> (c, kt, r, s)
@@ -907,6 +909,39 @@ __global__ __launch_bounds__(256) void splitk_init_kernel(float *y, const float 
 template <class Cfg>
 constexpr bool has_streamk = Cfg::BM >= 64 && Cfg::RS == 9;
 
+// Split-K scratch of pet_hip_conv2d_static_f32, the entry point that allocates nothing:
+// partial tiles, then one arrival counter per output tile. Every GPU the library runs on
+// holds its own copy until the process ends. In host code the array's name is not a device
+// address: static_scratch() asks the runtime for this device's copy once and host code
+// uses that pointer everywhere (kernel arguments included).
+constexpr size_t kStaticWsElems = (size_t)2 << 20; // 8 MiB of partial tiles
+constexpr int kStaticCounters = 4096;
+static __device__ __align__(256) float g_static_scratch[kStaticWsElems + kStaticCounters];
+
+constexpr int kMaxDevices = 64;
+static float *g_static_ptr[kMaxDevices] = {nullptr};
+
+// Device address of the current device's copy of the array (nullptr + error text on failure).
+float *static_scratch() {
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= kMaxDevices) {
+        set_error(PET_HIP_ERR_RUNTIME, "no current device for the static scratch");
+        return nullptr;
+    }
+    if (!g_static_ptr[dev]) {
+        void *ptr = nullptr;
+        hipError_t e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(g_static_scratch));
+        if (e != hipSuccess || !ptr) {
+            set_error(PET_HIP_ERR_RUNTIME, "hipGetSymbolAddress(static scratch) failed: %s",
+                      hipGetErrorString(e));
+            return nullptr;
+        }
+        // zero at load; every launch returns its counters to zero before it ends
+        g_static_ptr[dev] = static_cast<float *>(ptr);
+    }
+    return g_static_ptr[dev];
+}
+
 template <class Cfg, int DIM>
 int launch_plane_cfg(ConvParams p, hipStream_t stream) {
     const size_t lds_bytes = 2 * (size_t)Cfg::STAGE * sizeof(float);
@@ -987,7 +1022,7 @@ int launch_plane_cfg(ConvParams p, hipStream_t stream) {
         static const double sk_margin =
             getenv("PET_HIP_STREAMK_MARGIN") ? atof(getenv("PET_HIP_STREAMK_MARGIN")) : 0.95;
         const bool fits = p.G == 1 && units * (wgs + 1) < (1ll << 31) && units >= 2 * wgs &&
-                          has_streamk<Cfg> && !deterministic();
+                          has_streamk<Cfg> && !deterministic() && !p.static_ws;
         if (fits && forced <= 0 && (sk_env == 1 || (sk_env != 0 && cost_sk < sk_margin * best))) {
             p.streamk = 1;
             splitk = 1;
@@ -1002,8 +1037,24 @@ int launch_plane_cfg(ConvParams p, hipStream_t stream) {
     // in a launch after) are the faster way by 10-30% on small layers: the ordered
     // single-launch sum adds three dependent round trips through memory to every
     // tile. It is used when bit-reproducible results are asked for.
-    p.sk_mode = deterministic() ? 0 : 1;
-    if (splitk > 1 && p.sk_mode == 0) {
+    p.sk_mode = (deterministic() || p.static_ws) ? 0 : 1;
+    if (splitk > 1 && p.sk_mode == 0 && p.static_ws) {
+        // the static array of this file; a shape that does not fit is refused, not shrunk
+        const size_t need = (size_t)tiles * Cfg::BM * Cfg::BN * splitk;
+        if (need > kStaticWsElems || tiles > kStaticCounters)
+            return set_error(PET_HIP_ERR_UNSUPPORTED,
+                             "this convolution splits K %d ways over %lld tiles and needs %zu "
+                             "bytes of scratch; the static scratch holds %zu bytes and %d tiles",
+                             splitk, tiles, need * sizeof(float),
+                             kStaticWsElems * sizeof(float), kStaticCounters);
+        if (!p.dry_atomic) {
+            float *base = static_scratch();
+            if (!base)
+                return PET_HIP_ERR_RUNTIME;
+            p.ws = base;
+            p.cnt = reinterpret_cast<int *>(base + kStaticWsElems);
+        }
+    } else if (splitk > 1 && p.sk_mode == 0) {
         // the partial tiles and arrival counters live in the library's scratch
         size_t ws_elems;
         int ncnt;
@@ -1180,7 +1231,7 @@ int conv_common(const float *x, const float *w, const float *bias, float *y, int
                 int h, int wd, int f, int kt, int r, int s, int pt, int ph, int pw, int st, int sh,
                 int sw, int dt, int dh, int dw, int groups, int act, hipStream_t stream,
                 bool wpacked = false, const float *res = nullptr, unsigned flags = 0,
-                int *dry = nullptr) {
+                int *dry = nullptr, bool static_ws = false) {
     if (flags & ~(unsigned)(PET_HIP_CALL_Y_INITIALISED | PET_HIP_CALL_DEFER_RELU |
                             PET_HIP_CALL_X_RELU | PET_HIP_CALL_RES_RELU | 0xff00u))
         return set_error(PET_HIP_ERR_INVALID, "unknown call flags 0x%x", flags);
@@ -1261,6 +1312,7 @@ int conv_common(const float *x, const float *w, const float *bias, float *y, int
     p.y_init = (flags & PET_HIP_CALL_Y_INITIALISED) != 0;
     p.defer_relu = (flags & PET_HIP_CALL_DEFER_RELU) != 0;
     p.dry_atomic = dry;
+    p.static_ws = static_ws;
     if (((flags >> 8) & 0xffu) >= PET_HIP_CONV_ALGO_COUNT)
         return set_error(PET_HIP_ERR_INVALID, "unknown convolution algorithm %u",
                          (flags >> 8) & 0xffu);
@@ -1292,6 +1344,12 @@ int bmm_as_grouped_1x1(const float *A, const float *B, float *C, const float *bi
                        const float *res, int b, int m, int n, int k, int act, hipStream_t stream,
                        unsigned flags, int *dry) {
     if (k % 32 != 0 || b > 65535)
+        return -1;
+    // the group view holds b*k "channels" of n pixels and b*m "filters" of k taps: both
+    // must stay inside 32-bit element counts and the 2 GiB range of a buffer resource
+    if ((long long)b * k >= (1ll << 31) || (long long)b * m >= (1ll << 31) ||
+        4ll * b * k * n >= (1ll << 31) || 4ll * b * m * k >= (1ll << 31) ||
+        (long long)b * m * n >= (1ll << 31))
         return -1;
     ConvParams p;
     memset(&p, 0, sizeof(p));
@@ -1342,6 +1400,15 @@ int pet_hip_conv2d_f32(const float *x, const float *w, const float *bias, float 
     PET_REQUIRE_INIT();
     return conv_common(x, w, bias, y, n, c, 1, h, wd, f, 1, r, s, 0, ph, pw, 1, sh, sw, 1, dh, dw,
                        groups, act, as_stream(stream));
+}
+
+int pet_hip_conv2d_static_f32(const float *x, const float *w, const float *bias, float *y, int n,
+                              int c, int h, int wd, int f, int r, int s, int ph, int pw, int sh,
+                              int sw, int dh, int dw, int groups, int act,
+                              pet_hip_stream_t stream) {
+    PET_REQUIRE_INIT();
+    return conv_common(x, w, bias, y, n, c, 1, h, wd, f, 1, r, s, 0, ph, pw, 1, sh, sw, 1, dh, dw,
+                       groups, act, as_stream(stream), false, nullptr, 0, nullptr, true);
 }
 
 int pet_hip_conv3d_f32(const float *x, const float *w, const float *bias, float *y, int n, int c,

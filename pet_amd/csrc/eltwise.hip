@@ -274,6 +274,7 @@ __global__ __launch_bounds__(256) void pool2d_kernel(const float *__restrict__ x
         size_t plane = i / ((size_t)ow * oh);
         const float *xp = x + plane * (size_t)h * w;
         float acc = mode == 0 ? -INFINITY : 0.f;
+        int taps = 0; // window positions inside the image: the divisor of an average
         for (int r = 0; r < kh; ++r) {
             int ih = ii * sh + r * dh - ph;
             if (ih < 0 || ih >= h)
@@ -284,9 +285,10 @@ __global__ __launch_bounds__(256) void pool2d_kernel(const float *__restrict__ x
                     continue;
                 float v = xp[(size_t)ih * w + iw];
                 acc = mode == 0 ? fmaxf(acc, v) : acc + v;
+                ++taps;
             }
         }
-        y[i] = mode == 0 ? acc : acc / (float)(kh * kw);
+        y[i] = mode == 0 ? acc : (taps ? acc / (float)taps : 0.f);
     }
 }
 

@@ -135,6 +135,13 @@ int pet_hip_set_deterministic(int on) {
     return PET_HIP_OK;
 }
 
+int pet_hip_get_deterministic(int *on) {
+    if (!on)
+        return set_error(PET_HIP_ERR_INVALID, "null result pointer");
+    *on = pet::deterministic() ? 1 : 0;
+    return PET_HIP_OK;
+}
+
 int pet_hip_device_info(char *arch, size_t arch_len, int *num_cu) {
     PET_REQUIRE_INIT();
     hipDeviceProp_t prop;

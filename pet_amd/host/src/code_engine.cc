@@ -347,9 +347,13 @@ int launchChain(const std::vector<TransposeOp *> &row, pet_hip_stream_t s) {
 static AliasPlan planAliases(const OpVec &order) {
     AliasPlan plan;
     std::set<const Tensor *> aliased;
+    // tensors whose buffer another tensor already points into: moving such a
+    // buffer (into a concat's output) would leave those views on freed memory
+    std::set<const Tensor *> bases;
     for (auto op : order) {
         if (op->getType() == Operator::Split && static_cast<SplitOp *>(op)->getDim() == 0) {
             Tensor *in = op->getInputs()[0];
+            bases.insert(in);
             float *base = in->devicePtr();
             size_t off = 0;
             for (auto out : op->getOutputs()) {
@@ -361,6 +365,7 @@ static AliasPlan planAliases(const OpVec &order) {
         } else if (op->getType() == Operator::Reshape) {
             Tensor *in = op->getInputs()[0], *out = op->getOutputs()[0];
             if (elems(in) == elems(out)) {
+                bases.insert(in);
                 out->aliasDevice(in->devicePtr());
                 aliased.insert(out);
                 plan.skipped.insert(op);
@@ -376,8 +381,8 @@ static AliasPlan planAliases(const OpVec &order) {
         std::set<const Tensor *> seen;
         for (auto in : op->getInputs()) {
             Operator *prod = in->getOutputOf();
-            if (prod == nullptr || aliased.count(in) || !seen.insert(in).second ||
-                plan.skipped.count(prod))
+            if (prod == nullptr || aliased.count(in) || bases.count(in) ||
+                !seen.insert(in).second || plan.skipped.count(prod))
                 ok = false;
         }
         if (!ok)
@@ -611,13 +616,14 @@ std::string CodeEngine::genCode(std::shared_ptr<SubGraph> &graph) {
             for (Tensor *t : {bn->getScale(), bn->getBias(), bn->getMean(), bn->getVar()})
                 all.push_back(t);
     }
-    std::set<const Tensor *> viewOf;
+    std::set<const Tensor *> viewOf, viewBase;
     std::set<const Operator *> skipped;
     // storage sharing, mirrored from instantiate(): split / concat on dim 0, reshape
     std::vector<std::string> aliasLines;
     for (auto op : order) {
         if (op->getType() == Operator::Split && static_cast<SplitOp *>(op)->getDim() == 0) {
             size_t off = 0;
+            viewBase.insert(op->getInputs()[0]);
             for (auto out : op->getOutputs()) {
                 aliasLines.push_back("    float *" + e.name(out) + " = " +
                                      e.name(op->getInputs()[0]) + " + " + std::to_string(off) + ";");
@@ -629,6 +635,7 @@ std::string CodeEngine::genCode(std::shared_ptr<SubGraph> &graph) {
             aliasLines.push_back("    float *" + e.name(op->getOutputs()[0]) + " = " +
                                  e.name(op->getInputs()[0]) + ";");
             viewOf.insert(op->getOutputs()[0]);
+            viewBase.insert(op->getInputs()[0]);
             skipped.insert(op);
         }
     }
@@ -638,7 +645,8 @@ std::string CodeEngine::genCode(std::shared_ptr<SubGraph> &graph) {
         bool ok = true;
         std::set<const Tensor *> seen;
         for (auto in : op->getInputs())
-            if (in->getOutputOf() == nullptr || viewOf.count(in) || !seen.insert(in).second ||
+            if (in->getOutputOf() == nullptr || viewOf.count(in) || viewBase.count(in) ||
+                !seen.insert(in).second ||
                 skipped.count(in->getOutputOf()))
                 ok = false;
         if (!ok)

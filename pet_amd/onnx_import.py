@@ -367,6 +367,12 @@ def load(source, module=None, fold_bn=True):
             st = list(a.get("strides", [1, 1]))
             if a.get("ceil_mode", 0) or len(k) != 2:
                 raise ValueError("%s: ceil_mode / non-2-D pooling is not supported" % op)
+            # the backend's average leaves padding out of the divisor (ONNX's default,
+            # and the reference's cuDNN mode); max pooling is built without dilation
+            if op == "AveragePool" and int(a.get("count_include_pad", 0)) and any(pads):
+                raise ValueError("AveragePool: count_include_pad=1 with padding is not supported")
+            if any(int(d) != 1 for d in a.get("dilations", [1, 1])):
+                raise ValueError("%s: dilated pooling is not supported" % op)
             od = xd[:2] + [(xd[2 + i] + 2 * pads[i] - k[i]) // st[i] + 1 for i in range(2)]
             out = new(od)
             if op == "MaxPool":

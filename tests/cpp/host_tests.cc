@@ -3,6 +3,7 @@
 // programs (src/Test/*.cc): device results are checked against the CPU oracle
 // (linked only into this binary) or against each other where the reference
 // tests an identity. Usage: pet_host_tests [case-name]; exit code 0 = pass.
+#include <algorithm>
 #include <cmath>
 #include <cstring>
 #include <fstream>
@@ -160,6 +161,47 @@ static bool test_pad_conv_slice_verification() {
     return true;
 }
 
+// Two stacked contractions take dataRand's small integers past 2^24, where fp32 sums
+// are no longer exact: verification still accepts an equivalent mutant (here the
+// second convolution through pad -> conv -> slice, and a first convolution whose K
+// loop is split, summed in a fixed order during verification).
+static bool test_two_conv_verification() {
+    Graph g1, g2;
+    auto x1 = g1.tensor({1, 96, 14, 14}), w1 = g1.tensor({96, 96, 3, 3}),
+         v1 = g1.tensor({96, 96, 3, 3});
+    auto c1 = g1.conv(x1, w1, 1, 1);
+    g1.conv(c1->getOutputs()[0], v1, 1, 1);
+    g1.updateConnection();
+    auto x2 = g2.tensor({1, 96, 14, 14}), w2 = g2.tensor({96, 96, 3, 3}),
+         v2 = g2.tensor({96, 96, 3, 3});
+    auto d1 = g2.conv(x2, w2, 1, 1);
+    auto p = g2.pad(d1->getOutputs()[0], {0, 0, 0, 0}, {0, 0, 2, 2});
+    auto d2 = g2.conv(p->getOutputs()[0], v2, 1, 1);
+    g2.slice(d2->getOutputs()[0], {0, 0, 0, 0}, {0, 0, 2, 2});
+    g2.updateConnection();
+    SubGraph s1(g1.getOperators()), s2(g2.getOperators());
+    EXPECT(s1.getInputs().size() == 3 && s2.getInputs().size() == 3);
+    for (int rep = 0; rep < 3; ++rep)
+        EXPECT(s1.verification(&s2, true));
+    float top = 0.f;
+    const float *o = s1.getOutputs()[0]->getDataPtr();
+    for (size_t i = 0; i < s1.getOutputs()[0]->size(); ++i)
+        top = std::max(top, std::fabs(o[i]));
+    EXPECT(top > 16777216.f); // the case does leave the exact range
+    // a wrong mutant is still rejected: one layer missing its padding row
+    Graph g3;
+    auto x3 = g3.tensor({1, 96, 14, 14}), w3 = g3.tensor({96, 96, 3, 3}),
+         v3 = g3.tensor({96, 96, 3, 3});
+    auto e1 = g3.conv(x3, w3, 1, 1);
+    auto q = g3.pad(e1->getOutputs()[0], {0, 0, 1, 0}, {0, 0, 0, 0});
+    auto e2 = g3.conv(q->getOutputs()[0], v3, 1, 1);
+    g3.slice(e2->getOutputs()[0], {0, 0, 0, 0}, {0, 0, 1, 0});
+    g3.updateConnection();
+    SubGraph s3(g3.getOperators());
+    EXPECT(!s1.verification(&s3, true));
+    return true;
+}
+
 // Benchmark configuration 1, small: conv == H2N (halo) -> conv -> N2H (drop). Without
 // the correction the two programs differ at the seam.
 static bool test_corrected_h2n_program() {
@@ -265,6 +307,53 @@ static bool test_code_engine_graph_runtime() {
     EXPECT(code.find("pet_hip_graph_begin_capture") != std::string::npos);
     EXPECT(code.find("pet_hip_concat(") != std::string::npos); // the repeated-input concat
     EXPECT(code.find("pet_hip_split(") == std::string::npos);  // aliased away
+    return true;
+}
+
+// A tensor that a reshape or a dim-0 split already views must keep its buffer: a
+// dim-0 concat that also reads it copies instead of moving it into its own output.
+static bool test_alias_plan_shared_storage() {
+    for (int variant = 0; variant < 2; ++variant) {
+        auto build = [&](Graph &g) {
+            auto x = g.tensor({2, 4, 6}), y = g.tensor({2, 4, 6});
+            auto t = g.relu(x)->getOutputs()[0];  // produced inside the graph
+            auto u = g.relu(y)->getOutputs()[0];
+            Tensor *view0;
+            if (variant == 0) {
+                view0 = g.reshape(t, g.tensor({4, 12}))->getOutputs()[0];
+            } else {
+                view0 = g.split(t, 0, 2)->getOutputs()[1];
+            }
+            auto cc = g.concat({t, u}, 0)->getOutputs()[0]; // must not move t
+            g.relu(cc);
+            g.relu(view0);
+            g.updateConnection();
+        };
+        Graph g;
+        build(g);
+        auto s1 = std::make_shared<SubGraph>(g.getOperators());
+        auto s2 = std::make_shared<SubGraph>(g.getOperators());
+        for (size_t i = 0; i < s1->getInputs().size(); ++i) {
+            s1->getInputs()[i]->dataRand((int)i + 11);
+            s2->getInputs()[i]->setData(s1->getInputs()[i]->getDataPtr());
+        }
+        EXPECT(s1->compute());
+        CodeEngine ce;
+        auto exec = ce.instantiate(s2);
+        EXPECT(exec != nullptr);
+        EXPECT(exec->numAliasedOps() == 1); // the reshape / split only
+        for (int rep = 0; rep < 2; ++rep) {
+            EXPECT(exec->launch() && exec->sync());
+            EXPECT(s1->getOutputs().size() == s2->getOutputs().size());
+            for (size_t o = 0; o < s1->getOutputs().size(); ++o) {
+                Tensor *o1 = s1->getOutputs()[o], *o2 = s2->getOutputs()[o];
+                o2->deviceWritten();
+                EXPECT(equalArrays(o1->getDataPtr(), o2->getDataPtr(), o1->size()));
+            }
+        }
+        std::string code = ce.genCode(s2);
+        EXPECT(code.find("pet_hip_concat(") != std::string::npos);
+    }
     return true;
 }
 
@@ -768,9 +857,11 @@ int main(int argc, char **argv) {
         {"transpose_n2h_h2n", test_transpose_n2h_h2n},
         {"batch_gemm_merge", test_batch_gemm_merge},
         {"pad_conv_slice_verification", test_pad_conv_slice_verification},
+        {"two_conv_verification", test_two_conv_verification},
         {"corrected_h2n_program", test_corrected_h2n_program},
         {"dilated_space_to_batch_program", test_dilated_space_to_batch_program},
         {"code_engine_graph_runtime", test_code_engine_graph_runtime},
+        {"alias_plan_shared_storage", test_alias_plan_shared_storage},
         {"conv3d_prepacked_graph", test_conv3d_prepacked_graph},
         {"random_graphs_replay_equals_eager", test_random_graphs_replay_equals_eager},
         {"emit_program", test_emit_program},

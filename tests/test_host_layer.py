@@ -19,7 +19,8 @@ CASES = ["conv_vs_oracle", "conv_invalid_groups", "transpose_n2h_h2n", "batch_ge
          "dilated_space_to_batch_program", "code_engine_graph_runtime", "perf_engine_memo",
          "split_ratio_and_eltwise", "conv_merge_programs", "conv3d_prepacked_graph",
          "random_graphs_replay_equals_eager", "batchnorm_pow_div",
-         "gather_reduce_mean", "launch_fusion_block"]
+         "gather_reduce_mean", "launch_fusion_block", "alias_plan_shared_storage",
+         "two_conv_verification"]
 
 
 def test_host_library_is_built_and_exports_the_operator_classes():
@@ -253,8 +254,17 @@ def test_point_dependences_match_numpy_index_maps(tmp_path):
 # reference's src/Test/single_rule_test_*.cc, also unchanged.
 REFSEARCH = os.path.join(LIB, "libpet_refsearch.so")
 GENERATOR_DRIVER = os.path.join(LIB, "pet_generator_driver")
-needs_refsearch = pytest.mark.skipif(not os.path.exists(REFSEARCH),
-                                     reason="libpet_refsearch.so was not built")
+STATUS = os.path.join(LIB, "refsearch_status.txt")
+
+
+def _built_without_reference():
+    """True only when the build recorded that it had no reference tree to compile from.
+    In every other case the binaries are expected and their absence fails the test."""
+    return os.path.exists(STATUS) and open(STATUS).read().strip() == "no-reference"
+
+
+needs_refsearch = pytest.mark.skipif(_built_without_reference(),
+                                     reason="the build had no reference tree to compile from")
 
 # program -> candidates the generator must at least find. The assertions inside
 # the programs were written for an earlier generator: at the reference's head the
@@ -277,6 +287,7 @@ SINGLE_RULE_PROGRAMS = {
 def test_reference_single_rule_program_finds_mutants_on_the_device(program):
     import re
     exe = os.path.join(LIB, "refsearch", program)
+    assert os.path.exists(exe), "run __graft_entry__.build() where the reference tree is present"
     res = subprocess.run([exe], capture_output=True, text=True, timeout=300)
     print(res.stdout[-3000:])
     print(res.stderr[-2000:])
@@ -296,6 +307,8 @@ def test_reference_single_rule_program_finds_mutants_on_the_device(program):
     "1 32 32 32 32 3 2 2 0",       # dilated convolution: de-interleave candidates, partial
 ])
 def test_generator_candidates_run_and_are_ranked_on_the_device(args):
+    assert os.path.exists(GENERATOR_DRIVER), \
+        "run __graft_entry__.build() where the reference tree is present"
     res = subprocess.run([GENERATOR_DRIVER] + args.split(), capture_output=True, text=True,
                          timeout=600)
     print(res.stdout[-6000:])
@@ -470,7 +483,7 @@ REFERENCE_OPERATOR_PROGRAMS = [
 
 
 @pytest.mark.gpu
-@pytest.mark.skipif(not os.path.isdir(REFTESTS), reason="reference test programs were not built")
+@needs_refsearch
 @pytest.mark.parametrize("program", REFERENCE_OPERATOR_PROGRAMS)
 def test_reference_operator_program_runs_on_the_device(program):
     import re
@@ -480,6 +493,8 @@ def test_reference_operator_program_runs_on_the_device(program):
         # beyond fp32's exact integers: only the run-to-run reproducible mode can
         # meet its `==` (the reference computes in wrapping uint32)
         env["PET_HIP_DETERMINISTIC"] = "1"
+    assert os.path.exists(os.path.join(REFTESTS, program)), \
+        "run __graft_entry__.build() where the reference tree is present"
     res = subprocess.run([os.path.join(REFTESTS, program)], capture_output=True, text=True,
                          timeout=300, env=env)
     print(res.stdout[-1500:])
