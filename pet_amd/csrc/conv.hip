@@ -9,7 +9,7 @@
 // Both keep A (weights) in LDS as [m][k] and B (the im2col tile) as [k][n] and
 // feed v_mfma_f32_32x32x2_f32; within a K block MFMA step j gives lanes 0-31
 // k = j and lanes 32-63 k = BK/2 + j on both operands.
-#include "mfma_common.h"
+#include "conv_params.h"
 
 using namespace pet;
 using namespace pet::mfma;
@@ -18,50 +18,6 @@ namespace {
 
 // ---- convolution -----------------------------------------------------------------
 
-struct ConvParams {
-    const float *x, *w, *bias;
-    const float *res; // optional residual, laid out like y: y = act(conv + bias + res)
-    float *y;
-    int N, C, T, H, W, F;
-    int KT, R, S;
-    int pt, ph, pw, st, sh, sw, dt, dh, dw;
-    int G, cpg;
-    int OT, OH, OW;
-    int M;    // output channels per group
-    int K;    // cpg * KT * R * S
-    int NPIX; // N * OT * OH * OW
-    int OPIX; // OT * OH * OW
-    int act;
-    int bias_mode; // 1: bias[f] per output channel, 2: bias[pixel] per output column
-    int splitk;    // plane kernel: K steps are dealt to this many workgroups per tile
-    int xcd_chunk; // plane kernel: tiles per XCD when the tile grid is dealt in bands (0: off)
-    int xcd_mg;    // ... and how many M tiles wide a band is
-    FastDiv fd_band, fd_mg, fd_splitk; // divisions by xcd_mg * grid.x, xcd_mg and splitk
-    // stream-K (plane kernel): a 1-D grid of sk_wgs workgroups shares tiles * nit K steps
-    // evenly; a workgroup runs its range as up to three segments of consecutive tiles
-    int streamk, sk_units, sk_tiles_m;
-    FastDiv fd_sk_wgs, fd_sk_nit, fd_sk_tm;
-    int atomic_out; // partial sums are added into y with float atomics
-    int vec_out;   // plane kernel: OPIX % 4 == 0 and y 16-byte aligned: 16-byte output words
-    int wpacked;   // 3-D filters are stored kt-major, [kt][f][c/g][r][s] (plane kernel only)
-    int sk_mode;   // split-K: 0 partial tiles + ordered sum in one launch, 1 atomics into y
-    float *ws;     // split-K: partial tiles, [tile][split][register][thread]
-    int *cnt;      // split-K: arrival counter per tile, zero between launches
-    // caller-side fusion across launches (the *_ex entry points)
-    int x_relu;     // the input is used as max(x, 0): its producer left ReLU to the readers
-    int res_relu;   // the same for the residual operand
-    int y_init;     // y already holds bias (or 0): a split launch does not initialise it
-    int defer_relu; // a split launch leaves its ReLU to the readers of y
-    int *dry_atomic; // not null: report whether the launch would accumulate into y, launch nothing
-    int force_splitk;  // > 0: this many K shares per tile instead of the cost model's choice
-    int force_streamk; // 0 / 1: stream-K off / on instead of the cost model's choice; -1: model
-    int static_ws;   // split-K partial tiles and counters live in this file's static device
-                     // array (the entry point that allocates nothing); implies the ordered sum
-    int res_first;   // accumulating launch into an initialised y: the workgroup that holds a
-                     // tile's first K step adds the residual along with its partial sums
-    FastDiv fd_krs, fd_rs, fd_s;     // k -> (c, kt, r, s)
-    FastDiv fd_opix, fd_ohw, fd_ow;  // pixel -> (n, ot, oh, ow)
-};
 
 
 template <class Cfg, bool VECA, bool IS3D>
@@ -329,14 +285,6 @@ struct PlaneCfg {
                   "bad plane tile");
 };
 
-typedef unsigned uintx4 __attribute__((ext_vector_type(4)));
-
-__device__ __forceinline__ __amdgpu_buffer_rsrc_t make_rsrc(const void *base) {
-    // raw buffer, stride 0, 2 GiB of records, 32-bit float format
-    return __builtin_amdgcn_make_buffer_rsrc(const_cast<void *>(base), 0, 0x80000000, 0x00020000);
-}
-
-constexpr unsigned kOob = 0x80000000u; // voffset that the range check rejects
 
 // DIM 2: 2-D. DIM 3: 3-D with kt > 1 (one kt slice of a filter row is runs of r*s
 // floats, loaded one float at a time). DIM 4: 3-D with kt == 1 (filter rows are
@@ -647,13 +595,45 @@ __global__ __launch_bounds__(Cfg::NT) void conv_plane_kernel(ConvParams p) {
         }
         advance_prefetch();
     };
+    // Two-level sum: every kFlush steps the running tile is added into a second one and
+    // restarted, so no chain of fp32 additions is longer than kFlush * BK + nit / kFlush
+    // terms. On a 4608-term contraction (512 channels x 3x3) one chain's rounding error,
+    // which grows with the square root of its length, was 1.2e-4 of the smallest outputs
+    // against an fp64-accumulated result; 32 vector adds per kFlush steps buy a factor 3.
+    constexpr int kFlush = 8;
+    floatx16 acc2[TM][TN];
+#pragma unroll
+    for (int tm = 0; tm < TM; ++tm)
+#pragma unroll
+        for (int tn = 0; tn < TN; ++tn)
+#pragma unroll
+            for (int r = 0; r < 16; ++r)
+                acc2[tm][tn][r] = 0.f;
     int kt = 0;
     for (; kt + 1 < nit; kt += 2) {
         step(std::integral_constant<int, 0>{});
         step(std::integral_constant<int, 1>{});
+        if (((kt + 2) & (kFlush - 1)) == 0) {
+#pragma unroll
+            for (int tm = 0; tm < TM; ++tm)
+#pragma unroll
+                for (int tn = 0; tn < TN; ++tn)
+#pragma unroll
+                    for (int r = 0; r < 16; ++r) {
+                        acc2[tm][tn][r] += acc[tm][tn][r];
+                        acc[tm][tn][r] = 0.f;
+                    }
+        }
     }
     if (kt < nit)
         step(std::integral_constant<int, 0>{});
+#pragma unroll
+    for (int tm = 0; tm < TM; ++tm)
+#pragma unroll
+        for (int tn = 0; tn < TN; ++tn)
+#pragma unroll
+            for (int r = 0; r < 16; ++r)
+                acc[tm][tn][r] += acc2[tm][tn][r];
 
     // split-K: park the partial tile, and let the workgroup that arrives last add
     // the S partials in a fixed order (the result does not depend on timing).
@@ -1095,11 +1075,7 @@ int launch_plane_cfg(ConvParams p, hipStream_t stream) {
     }
     p.res_first = p.atomic_out && p.y_init && p.res != nullptr;
     if (p.atomic_out && !p.y_init) {
-        const size_t total = (size_t)p.NPIX * p.F;
-        unsigned igrid = (unsigned)std::min<size_t>((total + 255) / 256, 4096);
-        hipLaunchKernelGGL(splitk_init_kernel, dim3(igrid), dim3(256), 0, stream, p.y, p.bias,
-                           p.res, p.res_relu, p.bias_mode, (unsigned)p.F, (unsigned)p.OPIX, total);
-        int rc = check_launch("splitk_init_kernel");
+        int rc = launch_accumulate_init(p, stream);
         if (rc)
             return rc;
     }
@@ -1197,7 +1173,10 @@ __global__ void pack_filters_kernel(const float *__restrict__ w, float *__restri
 }
 
 int launch_conv(ConvParams &p, hipStream_t stream) {
-    int rc = try_launch_plane(p, stream);
+    int rc = try_launch_direct(p, stream);
+    if (rc >= 0)
+        return rc;
+    rc = try_launch_plane(p, stream);
     if (rc >= 0)
         return rc;
     if (p.wpacked)
@@ -1386,7 +1365,17 @@ int bmm_as_grouped_1x1(const float *A, const float *B, float *C, const float *bi
     p.fd_opix = make_fastdiv((unsigned)n);
     p.fd_ohw = make_fastdiv((unsigned)n);
     p.fd_ow = make_fastdiv((unsigned)n);
-    return try_launch_plane(p, stream);
+    p.fd_splitk = make_fastdiv(1);
+    const int rc = try_launch_direct(p, stream);
+    return rc >= 0 ? rc : try_launch_plane(p, stream);
+}
+
+int launch_accumulate_init(const ConvParams &p, hipStream_t stream) {
+    const size_t total = (size_t)p.NPIX * p.F;
+    unsigned igrid = (unsigned)std::min<size_t>((total + 255) / 256, 4096);
+    hipLaunchKernelGGL(splitk_init_kernel, dim3(igrid), dim3(256), 0, stream, p.y, p.bias, p.res,
+                       p.res_relu, p.bias_mode, (unsigned)p.F, (unsigned)p.OPIX, total);
+    return check_launch("splitk_init_kernel");
 }
 
 } // namespace mfma

@@ -598,15 +598,15 @@ static bool test_split_ratio_and_eltwise() {
 }
 
 // What the graph runtime fuses across launches, on two residual blocks whose
-// convolutions split K (64 channels on 28x28): ReLU left to the convolutions that
+// convolutions split K (512 channels on 14x14): ReLU left to the convolutions that
 // read a tensor (as input and as residual), output initialisations batched into one
 // launch. Signed data, so a ReLU applied in the wrong place, or not at all, shows.
 static bool test_launch_fusion_block() {
     Graph g;
-    auto x = g.tensor({1, 64, 28, 28});
+    auto x = g.tensor({1, 512, 14, 14});
     Tensor *w[4];
     for (auto &t : w)
-        t = g.tensor({64, 64, 3, 3});
+        t = g.tensor({512, 512, 3, 3});
     auto c1 = static_cast<ConvOp *>(g.conv(x, w[0], 1, 1));
     c1->setAct(Operator::Relu);
     auto c2 = g.conv(c1->getOutputs()[0], w[1], 1, 1);

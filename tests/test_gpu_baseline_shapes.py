@@ -2,8 +2,7 @@
 configurations, with each configuration's own data distribution.
 
 Every case is checked twice against the CPU oracle: real-valued inputs under the
-per-element bound |got - ref| <= 1e-4 * max(|ref|, 1e-3 * sum|a||b|) (and the
-normwise 1e-4), and small-integer inputs bit for bit (fp32 sums of integers below
+per-element and normwise bounds of tests/tolerance.py (1e-4), and small-integer inputs bit for bit (fp32 sums of integers below
 2^24 are exact, so any indexing mistake shows as a whole-number difference).
 The whole-network tests only bound the final tensor normwise; these pin the
 individual launches the networks are made of: tile grids, K lengths, XCD
@@ -14,10 +13,9 @@ import pytest
 import torch
 
 import oracle
+from tolerance import REL_TOL, max_rel_err
 
 pytestmark = pytest.mark.gpu
-
-REL_TOL = 1e-4
 
 
 def dev(a):
@@ -31,12 +29,6 @@ def host(t):
 
 def ints(rng, shape, lo=-3, hi=4):
     return rng.integers(lo, hi, size=shape).astype(np.float32)
-
-
-def max_rel_err(got, ref, mag):
-    elem = np.max(np.abs(got - ref) / np.maximum(np.abs(ref), 1e-3 * mag))
-    norm = np.max(np.abs(got - ref)) / np.max(np.abs(ref))
-    return float(max(elem, norm))
 
 
 @pytest.fixture(scope="module")
