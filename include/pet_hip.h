@@ -275,6 +275,32 @@ PET_HIP_API int pet_hip_bmm_f32(int transA, int transB, int b, int m, int n, int
                     const float *B, float *C, const float *bias, int act,
                     pet_hip_stream_t stream);
 
+/* Transposed convolution: x NHWF [n,h,w,f], weight RSFC [r,s,f,c], y NHWC [n,oh,ow,c],
+ * oh = pet_hip_conv_trans_out_dim(h, r, ph, sh, dh, oph). Semantics: ConvTransOp::compute,
+ * src/Graph/operator.cc:932-983 (flipped taps, input row (hh + rr*dh - (r-ph-1)) / sh where
+ * exact, taps rr > r - (h + 2ph - r) % sh left out) over the output's own rows and columns,
+ * i.e. the values of src/Test/convtrans_test_1.cc:62-77, 120-135; shape rule
+ * ConvTransOp::computeShape, :1055-1072. bias (may be NULL) is [c]. Replaces
+ * cudnnConvolutionBackwardData (src/Graph/operator.cc:1113-1287, src/Graph/code_engine.cc:
+ * 979-1101). */
+PET_HIP_API int pet_hip_conv_trans_out_dim(int i, int k, int p, int s, int d, int op);
+PET_HIP_API int pet_hip_conv_trans_f32(const float *x, const float *w, const float *bias, float *y,
+                           int n, int h, int wd, int f, int r, int s, int c, int ph, int pw,
+                           int sh, int sw, int dh, int dw, int oph, int opw, int act,
+                           pet_hip_stream_t stream);
+
+/* Band products of sliding-window attention. G2BMM: A, B [bs,m,k] -> C [bs,m,2w+1],
+ * C[b,i,j] = sum_k A[b,i,k] * B[b, i + d*(j-w), k]; GBMML: A [bs,m,2w+1], B [bs,m,n] ->
+ * C [bs,m,n], C[b,i,x] = sum_j A[b,i,j] * B[b, i + d*j - d*w, x]; rows of B outside [0, m)
+ * read as zero. Definitions: Sg2bmmPattern::getExpr / LongformerGBMMPattern::getExpr,
+ * src/nnet/iterator_table.cc:596-630 (G2BMMOp / GBMMLOp have no CPU compute,
+ * src/Graph/operator.cc:1355-1364, 1498-1507). Replace _sg2bmm / _sgbmml, the generated
+ * kernels of include/custom_ops.cuh:3538-3559, 5778-5800 (src/Graph/operator.cc:1442-1463). */
+PET_HIP_API int pet_hip_g2bmm_f32(const float *A, const float *B, float *C, int bs, int m, int k,
+                      int width, int dilation, pet_hip_stream_t stream);
+PET_HIP_API int pet_hip_gbmml_f32(const float *A, const float *B, float *C, int bs, int m, int width,
+                      int n, int dilation, pet_hip_stream_t stream);
+
 /* ---- layout operators (bit-exact copies) ---------------------------------*/
 
 /* TransposeOp::compute after the split has been resolved to flat dims,

@@ -185,6 +185,50 @@ def matmul(A, B, transA=False, transB=False):
     return C
 
 
+def conv_trans_out_dim(i, k, p, s, d, op):
+    """ConvTransOp::computeShape, src/Graph/operator.cc:1066-1067."""
+    return (i - 1) * s - 2 * p + d * (k - 1) + op + 1
+
+
+def conv_trans(x, w, ph, pw, sh=1, sw=1, dh=1, dw=1, oph=0, opw=0):
+    """ConvTransOp::compute: x NHWF [n,h,w,f], w RSFC [r,s,f,c] -> NHWC [n,oh,ow,c]."""
+    x, w = _c(x), _c(w)
+    t = _tier(x, w)
+    n, h, wd, f = x.shape
+    r, s, f2, c = w.shape
+    assert f == f2
+    oh = conv_trans_out_dim(h, r, ph, sh, dh, oph)
+    ow = conv_trans_out_dim(wd, s, pw, sw, dw, opw)
+    y = np.empty((n, oh, ow, c), dtype=x.dtype)
+    rc = getattr(lib(), "oracle_conv_trans_" + t)(_p(x), _p(w), _p(y), n, h, wd, f, r, s, c,
+                                                  ph, pw, sh, sw, dh, dw, oh, ow)
+    return None if rc else y
+
+
+def g2bmm(A, B, width, dilation=1):
+    """C[b,m,j] = sum_k A[b,m,k] B[b, m + d (j - w), k]; A, B [bs,m,k] -> [bs,m,2w+1]."""
+    A, B = _c(A), _c(B)
+    t = _tier(A, B)
+    bs, m, k = A.shape
+    assert B.shape == A.shape
+    C = np.empty((bs, m, 2 * width + 1), dtype=A.dtype)
+    getattr(lib(), "oracle_g2bmm_" + t)(_p(A), _p(B), _p(C), bs, m, k, int(width), int(dilation))
+    return C
+
+
+def gbmml(A, B, dilation=1):
+    """C[b,m,n] = sum_j A[b,m,j] B[b, m + d j - d w, n]; A [bs,m,2w+1], B [bs,m,n]."""
+    A, B = _c(A), _c(B)
+    t = _tier(A, B)
+    bs, m, band = A.shape
+    assert band % 2 == 1 and B.shape[:2] == (bs, m)
+    n = B.shape[2]
+    C = np.empty((bs, m, n), dtype=A.dtype)
+    getattr(lib(), "oracle_gbmml_" + t)(_p(A), _p(B), _p(C), bs, m, (band - 1) // 2, n,
+                                        int(dilation))
+    return C
+
+
 def transpose(x, split, after, factor=2):
     """TransposeOp(input, split, after, factor)::compute."""
     x = _c(x)

@@ -69,6 +69,10 @@ SIGNATURES = {
     "pet_hip_conv3d_pack_filters": [_vp, _vp] + [_i] * 5 + [_vp],
     "pet_hip_conv3d_packed_f32": [_vp] * 4 + [_i] * 20 + [_vp],
     "pet_hip_bmm_f32": [_i] * 6 + [_vp] * 4 + [_i, _vp],
+    "pet_hip_conv_trans_out_dim": [_i] * 6,
+    "pet_hip_conv_trans_f32": [_vp] * 4 + [_i] * 16 + [_vp],
+    "pet_hip_g2bmm_f32": [_vp] * 3 + [_i] * 5 + [_vp],
+    "pet_hip_gbmml_f32": [_vp] * 3 + [_i] * 5 + [_vp],
     "pet_hip_transpose": [_vp, _vp, _c_int_p, _c_int_p, _i, _vp],
     "pet_hip_trans_chain": [_vp, _vp, _c_int_p, _i, _c_int_p, _i, _c_int_p, _c_int_p, _c_int_p, _vp],
     "pet_hip_split": [_vp, ctypes.POINTER(_vp), _i, _c_int_p, _i, _i, _c_int_p, _vp],

@@ -105,6 +105,17 @@ PYBIND11_MODULE(cpp_module, m) {
         .def("matmul",
              py::overload_cast<Tensor *, Tensor *, Tensor *, bool, bool, Tensor *>(&Graph::matmul),
              "A"_a, "B"_a, "C"_a, "transA"_a = false, "transB"_a = false, "bias"_a = nullptr, kRef)
+        .def("convTrans",
+             py::overload_cast<Tensor *, Tensor *, Tensor *, int, int, int, int, int, int, int, int,
+                               Tensor *>(&Graph::convTrans),
+             "input"_a, "weight"_a, "output"_a, "ph"_a, "pw"_a, "sh"_a = 1, "sw"_a = 1,
+             "dh"_a = 1, "dw"_a = 1, "oph"_a = 0, "opw"_a = 0, "bias"_a = nullptr, kRef)
+        .def("g2bmm",
+             py::overload_cast<Tensor *, Tensor *, Tensor *, int, int, Tensor *>(&Graph::g2bmm),
+             "A"_a, "B"_a, "C"_a, "width"_a, "dilation"_a, "bias"_a = nullptr, kRef)
+        .def("gbmml",
+             py::overload_cast<Tensor *, Tensor *, Tensor *, int, Tensor *>(&Graph::gbmml), "A"_a,
+             "B"_a, "C"_a, "dilation"_a, "bias"_a = nullptr, kRef)
         .def("pad",
              py::overload_cast<Tensor *, Tensor *, const Dim &, const Dim &>(&Graph::pad), kRef)
         .def("slice",

@@ -52,6 +52,22 @@ class Graph : public GraphBase {
                    int sh = 1, int sw = 1, int dh = 1, int dw = 1, Tensor *bias = nullptr);
     Operator *conv(Tensor *input, Tensor *weight, ConvOp::PaddingMode pm, int sh = 1, int sw = 1,
                    int dh = 1, int dw = 1, Tensor *bias = nullptr);
+    // Transposed convolution on NCHW input / [f, c, r, s] weight / NCHW output: the layout
+    // transposes around the NHWC operator are part of what is built (include/graph.h:55-74).
+    Tensor *setConvTransInput(Tensor *input);
+    Tensor *setConvTransWeight(Tensor *weight);
+    Tensor *setConvTransOutput(Tensor *outputTrans, Tensor *output = nullptr);
+    Operator *convTrans(Tensor *input, Tensor *weight, Tensor *output, int ph, int pw, int sh = 1,
+                        int sw = 1, int dh = 1, int dw = 1, int oph = 0, int opw = 0,
+                        Tensor *bias = nullptr);
+    Operator *convTrans(Tensor *input, Tensor *weight, Tensor *output,
+                        ConvTransOp::PaddingMode pm, int sh = 1, int sw = 1, int dh = 1,
+                        int dw = 1, int oph = 0, int opw = 0, Tensor *bias = nullptr);
+    Operator *g2bmm(Tensor *A, Tensor *B, Tensor *C, int width, int dilation,
+                    Tensor *bias = nullptr);
+    Operator *g2bmm(Tensor *A, Tensor *B, int width, int dilation, Tensor *bias = nullptr);
+    Operator *gbmml(Tensor *A, Tensor *B, Tensor *C, int dilation, Tensor *bias = nullptr);
+    Operator *gbmml(Tensor *A, Tensor *B, int dilation, Tensor *bias = nullptr);
     Operator *conv3d(Tensor *input, Tensor *weight, Tensor *output, const Dim &pad,
                      const Dim &stride, const Dim &dilation, Tensor *bias = nullptr);
     Operator *matmul(Tensor *A, Tensor *B, Tensor *C, bool transA = false, bool transB = false,

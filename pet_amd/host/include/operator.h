@@ -330,14 +330,72 @@ class MatmulOp : public Operator {
     int algo = 0;
 };
 
-// ---- band matrix products (declared, not executed) --------------------------------
+// ---- ConvTrans -----------------------------------------------------------------------
+// Transposed convolution in the reference's operator-level layout: input NHWF [n,h,w,f],
+// weight RSFC [r,s,f,c], output NHWC [n,oh,ow,c] (include/operator.h:466-612,
+// src/Graph/operator.cc:866-1100). Graph::convTrans takes NCHW tensors and puts the
+// layout transposes around it, as the reference's builder does.
+class ConvTransOp : public Operator {
+  public:
+    enum PaddingMode { Other, Same, Valid };
+
+    ConvTransOp(Tensor *input, Tensor *weight, Tensor *output, int ph, int pw, int sh = 1,
+                int sw = 1, int dh = 1, int dw = 1, int oph = 1, int opw = 1,
+                Tensor *bias = nullptr, ActType act = None);
+    ConvTransOp(Tensor *input, Tensor *weight, int ph, int pw, int sh = 1, int sw = 1, int dh = 1,
+                int dw = 1, int oph = 0, int opw = 0, Tensor *bias = nullptr, ActType act = None);
+    ConvTransOp(int ph, int pw, int sh = 1, int sw = 1, int dh = 1, int dw = 1, int oph = 0,
+                int opw = 0, Tensor *bias = nullptr, ActType act = None);
+    ConvTransOp(Tensor *input, Tensor *weight, Tensor *output, PaddingMode pm = Same, int sh = 1,
+                int sw = 1, int dh = 1, int dw = 1, int oph = 0, int opw = 0,
+                Tensor *bias = nullptr, ActType act = None);
+    ConvTransOp(Tensor *input, Tensor *weight, PaddingMode pm = Same, int sh = 1, int sw = 1,
+                int dh = 1, int dw = 1, int oph = 1, int opw = 1, Tensor *bias = nullptr,
+                ActType act = None);
+    ConvTransOp(PaddingMode pm = Same, int sh = 1, int sw = 1, int dh = 1, int dw = 1,
+                int oph = 0, int opw = 0, Tensor *bias = nullptr, ActType act = None);
+    ConvTransOp(const ConvTransOp &rhs);
+    ConvTransOp *clone() override { return new ConvTransOp(*this); }
+
+    Dim computeShape() override;
+    double perf(PerfEngine *pe, int rounds = 200, int warmupRounds = 200) override;
+    int launch(pet_hip_stream_t stream) override;
+    std::string toString() const override;
+    int numInputs() override { return 2; }
+    int numOutputs() override { return 1; }
+    Tensor *getBias() const { return bias; }
+    void setAct(ActType a) { act = a; }
+    ActType getAct() const { return act; }
+    bool same(const ConvTransOp &rhs);
+    PaddingMode getPaddingMode() { return padding; }
+    int getDh() const { return dh; }
+    int getDw() const { return dw; }
+    int getPh() const { return ph; }
+    int getPw() const { return pw; }
+    int getSh() const { return sh; }
+    int getSw() const { return sw; }
+    int getOph() const { return oph; }
+    int getOpw() const { return opw; }
+    // n, c, h, w, f, r, s, ph, pw, sh, sw, dh, dw, g, bias, act with c the output
+    // channels and f the input features (include/operator.h:584-599)
+    ConvArgs getArgs(int withPenalty) const;
+
+  private:
+    bool checkValid(const TensorVec &inputs) override;
+    void initHash() override;
+    void setPaddingMode();
+    int ph = 0, pw = 0, sh, sw, dh, dw, oph, opw;
+    Tensor *bias; // not part of the graph connections
+    ActType act;
+    PaddingMode padding;
+};
+
+// ---- band matrix products ---------------------------------------------------------------
 // G2BMM (general x general -> band) and GBMML (band x general -> general) are the
-// Longformer attention products the reference runs through generated kernels
-// (include/custom_ops.cuh) and has no host evaluation for
-// (src/Graph/operator.cc:1365-1391). They are declared here, with the
-// reference's shape rules, so that code that names the classes builds; this
-// backend does not run them: launch() reports PET_HIP_ERR_UNSUPPORTED and perf()
-// returns INFINITY, the reference's convention for an operator a backend rejects.
+// sliding-window attention products. The reference has no host evaluation for them
+// (src/Graph/operator.cc:1355-1391, 1498-1527) and runs two generated kernels fixed to
+// one shape (include/custom_ops.cuh:3538-3559); here they run on the device for any
+// shape, by the definitions of src/nnet/iterator_table.cc:596-630.
 typedef std::tuple<int, int, int, int, int> G2BMMGBMMLArgs; // b, m, k, width, dilation
 
 class G2BMMOp : public Operator {

@@ -22,6 +22,12 @@ struct ConvResult {
     bool fuseAct;         // bias + activation are fused in the epilogue
 };
 
+struct ConvTransResult {
+    double time;
+    int algo; // one kernel: always 0
+    size_t workspaceSize;
+};
+
 struct MatmulResult {
     double time;
     bool useStrideBatchAPI;

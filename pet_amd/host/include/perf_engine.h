@@ -34,14 +34,25 @@ class PerfEngine {
     int getMatmulAlgo(const MatmulArgs &args) { return matmulPerf.at(args).algo; }
 
     template <class OpArgs> double getOpPerf(Operator::OpType, const OpArgs &) { return 0.0; }
-    double getOpPerf(Operator::OpType, const ConvArgs &args) { return convPerf.at(args).time; }
+    double getOpPerf(Operator::OpType t, const ConvArgs &args) {
+        return t == Operator::ConvTrans ? convTransPerf.at(args).time : convPerf.at(args).time;
+    }
+    double getOpPerf(Operator::OpType t, const G2BMMGBMMLArgs &args) {
+        return (t == Operator::G2BMM ? g2bmmPerf : gbmmlPerf).at(args);
+    }
+    int getConvTransAlgo(const ConvArgs &args) { return convTransPerf.at(args).algo; }
     double getOpPerf(Operator::OpType, const MatmulArgs &args) { return matmulPerf.at(args).time; }
     double getOpPerf(Operator::OpType t, const PoolArgs &args) {
         return (t == Operator::MaxPool ? maxPoolPerf : avgPoolPerf).at(args);
     }
 
     template <class OpArgs> bool checkOpPerf(Operator::OpType, const OpArgs &) { return true; }
-    bool checkOpPerf(Operator::OpType, const ConvArgs &args) { return convPerf.count(args) != 0; }
+    bool checkOpPerf(Operator::OpType t, const ConvArgs &args) {
+        return (t == Operator::ConvTrans ? convTransPerf.count(args) : convPerf.count(args)) != 0;
+    }
+    bool checkOpPerf(Operator::OpType t, const G2BMMGBMMLArgs &args) {
+        return (t == Operator::G2BMM ? g2bmmPerf : gbmmlPerf).count(args) != 0;
+    }
     bool checkOpPerf(Operator::OpType, const MatmulArgs &args) {
         return matmulPerf.count(args) != 0;
     }
@@ -50,6 +61,12 @@ class PerfEngine {
     }
 
     void saveOpPerf(uint32_t, const ConvArgs &args, const ConvResult &r) { convPerf[args] = r; }
+    void saveOpPerf(uint32_t, const ConvArgs &args, const ConvTransResult &r) {
+        convTransPerf[args] = r;
+    }
+    void saveOpPerf(uint32_t t, const G2BMMGBMMLArgs &args, float ms) {
+        (t == Operator::G2BMM ? g2bmmPerf : gbmmlPerf)[args] = ms;
+    }
     void saveOpPerf(uint32_t, const MatmulArgs &args, const MatmulResult &r) {
         matmulPerf[args] = r;
     }
@@ -69,7 +86,9 @@ class PerfEngine {
 
     int penaltyFlag = 1;
     std::map<ConvArgs, ConvResult> convPerf;
+    std::map<ConvArgs, ConvTransResult> convTransPerf;
     std::map<MatmulArgs, MatmulResult> matmulPerf;
+    std::map<G2BMMGBMMLArgs, float> g2bmmPerf, gbmmlPerf;
     std::map<PoolArgs, float> maxPoolPerf, avgPoolPerf;
     float *buf[4] = {nullptr, nullptr, nullptr, nullptr};
     size_t bufElems[4] = {0, 0, 0, 0};

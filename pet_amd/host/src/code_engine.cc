@@ -743,6 +743,25 @@ std::string CodeEngine::genCode(std::shared_ptr<SubGraph> &graph) {
                     c << ", " << x;
             c << ", " << d[1] / w[1] << ", " << actOf(c3->getAct()) << ", "
               << (fl ? std::to_string(fl) + "u, " : std::string()) << "s)";
+        } else if (auto ct = dynamic_cast<ConvTransOp *>(op)) {
+            auto d = op->getInputs()[0]->getDims(), w = op->getInputs()[1]->getDims();
+            c << "pet_hip_conv_trans_f32(" << in(0) << ", " << in(1) << ", "
+              << nullable(e, ct->getBias()) << ", " << out(0);
+            for (int v : {d[0], d[1], d[2], d[3], w[0], w[1], w[3], ct->getPh(), ct->getPw(),
+                          ct->getSh(), ct->getSw(), ct->getDh(), ct->getDw(), ct->getOph(),
+                          ct->getOpw(), (int)ct->getAct()})
+                c << ", " << v;
+            c << ", s)";
+        } else if (auto g2 = dynamic_cast<G2BMMOp *>(op)) {
+            auto d = op->getInputs()[0]->getDims();
+            c << "pet_hip_g2bmm_f32(" << in(0) << ", " << in(1) << ", " << out(0) << ", " << d[0]
+              << ", " << d[1] << ", " << d[2] << ", " << g2->getWidth() << ", "
+              << g2->getDilation() << ", s)";
+        } else if (auto gb = dynamic_cast<GBMMLOp *>(op)) {
+            auto d = op->getInputs()[0]->getDims();
+            c << "pet_hip_gbmml_f32(" << in(0) << ", " << in(1) << ", " << out(0) << ", " << d[0]
+              << ", " << d[1] << ", " << (d[2] - 1) / 2 << ", " << op->getInputs()[1]->getDims()[2]
+              << ", " << gb->getDilation() << ", s)";
         } else if (auto ln = dynamic_cast<LayerNormOp *>(op)) {
             size_t cols = (size_t)op->getInputs()[0]->getDims().back();
             c << "pet_hip_layernorm(" << in(0) << ", " << nullable(e, ln->getGamma()) << ", "

@@ -115,6 +115,50 @@ Operator *Graph::conv(Tensor *input, Tensor *weight, ConvOp::PaddingMode pm, int
                       int dh, int dw, Tensor *bias) {
     return own(new ConvOp(input, weight, pm, sh, sw, dh, dw, bias));
 }
+// NCHW -> NHWF, [f,c,r,s] -> [r,s,f,c] and NHWC -> NCHW around ConvTransOp
+// (src/Graph/graph.cc:90-131).
+Tensor *Graph::setConvTransInput(Tensor *input) {
+    return own(new TransposeOp(input, -1, {0, 2, 3, 1}))->getOutputs()[0];
+}
+Tensor *Graph::setConvTransWeight(Tensor *weight) {
+    weight->setType(Tensor::Weight);
+    return own(new TransposeOp(weight, -1, {2, 3, 0, 1}))->getOutputs()[0];
+}
+Tensor *Graph::setConvTransOutput(Tensor *outputTrans, Tensor *output) {
+    if (output == nullptr)
+        return own(new TransposeOp(outputTrans, -1, {0, 3, 1, 2}))->getOutputs()[0];
+    own(new TransposeOp(outputTrans, output, -1, {0, 3, 1, 2}));
+    return output;
+}
+Operator *Graph::convTrans(Tensor *input, Tensor *weight, Tensor *output, int ph, int pw, int sh,
+                           int sw, int dh, int dw, int oph, int opw, Tensor *bias) {
+    input = setConvTransInput(input);
+    weight = setConvTransWeight(weight);
+    auto op = own(new ConvTransOp(input, weight, ph, pw, sh, sw, dh, dw, oph, opw, bias));
+    setConvTransOutput(op->getOutputs()[0], output);
+    return op;
+}
+Operator *Graph::convTrans(Tensor *input, Tensor *weight, Tensor *output,
+                           ConvTransOp::PaddingMode pm, int sh, int sw, int dh, int dw, int oph,
+                           int opw, Tensor *bias) {
+    input = setConvTransInput(input);
+    weight = setConvTransWeight(weight);
+    auto op = own(new ConvTransOp(input, weight, pm, sh, sw, dh, dw, oph, opw, bias));
+    setConvTransOutput(op->getOutputs()[0], output);
+    return op;
+}
+Operator *Graph::g2bmm(Tensor *A, Tensor *B, Tensor *C, int width, int dilation, Tensor *bias) {
+    return own(new G2BMMOp(A, B, C, width, dilation, bias));
+}
+Operator *Graph::g2bmm(Tensor *A, Tensor *B, int width, int dilation, Tensor *bias) {
+    return own(new G2BMMOp(A, B, width, dilation, bias));
+}
+Operator *Graph::gbmml(Tensor *A, Tensor *B, Tensor *C, int dilation, Tensor *bias) {
+    return own(new GBMMLOp(A, B, C, dilation, bias));
+}
+Operator *Graph::gbmml(Tensor *A, Tensor *B, int dilation, Tensor *bias) {
+    return own(new GBMMLOp(A, B, dilation, bias));
+}
 Operator *Graph::conv3d(Tensor *input, Tensor *weight, Tensor *output, const Dim &pad,
                         const Dim &stride, const Dim &dilation, Tensor *bias) {
     return own(new Conv3dOp(input, weight, output, pad, stride, dilation, bias));

@@ -407,6 +407,164 @@ std::string ConvOp::toString() const {
     return os.str();
 }
 
+// ---- ConvTransOp ----------------------------------------------------------------
+
+ConvTransOp::ConvTransOp(Tensor *input, Tensor *weight, Tensor *output, int ph, int pw, int sh,
+                         int sw, int dh, int dw, int oph, int opw, Tensor *bias, ActType act)
+    : Operator(ConvTrans, {input, weight}, {output}), ph(ph), pw(pw), sh(sh), sw(sw), dh(dh),
+      dw(dw), oph(oph), opw(opw), bias(bias), act(act), padding(Other) {
+    weight->setType(Tensor::Weight);
+    assert(checkValid({input, weight}));
+    computeShape();
+    setPaddingMode();
+    initHash();
+}
+
+ConvTransOp::ConvTransOp(Tensor *input, Tensor *weight, int ph, int pw, int sh, int sw, int dh,
+                         int dw, int oph, int opw, Tensor *bias, ActType act)
+    : ConvTransOp(input, weight, new Tensor(), ph, pw, sh, sw, dh, dw, oph, opw, bias, act) {}
+
+ConvTransOp::ConvTransOp(int ph, int pw, int sh, int sw, int dh, int dw, int oph, int opw,
+                         Tensor *bias, ActType act)
+    : Operator(ConvTrans), ph(ph), pw(pw), sh(sh), sw(sw), dh(dh), dw(dw), oph(oph), opw(opw),
+      bias(bias), act(act), padding(Other) {
+    initHash();
+}
+
+// The padding-mode constructors keep the mode for hashing and same(); the reference never
+// derives a padding size from it for this operator (its computeShape reads ph and pw as
+// they are, src/Graph/operator.cc:1055-1072), so they stay 0 here as well.
+ConvTransOp::ConvTransOp(Tensor *input, Tensor *weight, Tensor *output, PaddingMode pm, int sh,
+                         int sw, int dh, int dw, int oph, int opw, Tensor *bias, ActType act)
+    : Operator(ConvTrans, {input, weight}, {output}), sh(sh), sw(sw), dh(dh), dw(dw), oph(oph),
+      opw(opw), bias(bias), act(act), padding(pm) {
+    weight->setType(Tensor::Weight);
+    assert(checkValid({input, weight}));
+    computeShape();
+    initHash();
+}
+
+ConvTransOp::ConvTransOp(Tensor *input, Tensor *weight, PaddingMode pm, int sh, int sw, int dh,
+                         int dw, int oph, int opw, Tensor *bias, ActType act)
+    : ConvTransOp(input, weight, new Tensor(), pm, sh, sw, dh, dw, oph, opw, bias, act) {}
+
+ConvTransOp::ConvTransOp(PaddingMode pm, int sh, int sw, int dh, int dw, int oph, int opw,
+                         Tensor *bias, ActType act)
+    : Operator(ConvTrans), sh(sh), sw(sw), dh(dh), dw(dw), oph(oph), opw(opw), bias(bias),
+      act(act), padding(pm) {
+    initHash();
+}
+
+ConvTransOp::ConvTransOp(const ConvTransOp &rhs)
+    : Operator(rhs), ph(rhs.ph), pw(rhs.pw), sh(rhs.sh), sw(rhs.sw), dh(rhs.dh), dw(rhs.dw),
+      oph(rhs.oph), opw(rhs.opw), bias(rhs.bias), act(rhs.act), padding(rhs.padding) {}
+
+void ConvTransOp::initHash() {
+    hash = type;
+    hash = hashAppend(hash, padding);
+    if (padding == Other) {
+        hash = hashAppend(hash, ph);
+        hash = hashAppend(hash, pw);
+    }
+    for (int v : {sh, sw, dh, dw, oph, opw})
+        hash = hashAppend(hash, v);
+    hash = hashPack(hash);
+}
+
+// input [n,h,w,f], weight [r,s,f,c] -> [n, oh, ow, c] (src/Graph/operator.cc:1055-1072)
+Dim ConvTransOp::computeShape() {
+    auto in = inputs[0]->getDims(), wt = inputs[1]->getDims();
+    Dim ret = {in[0], pet_hip_conv_trans_out_dim(in[1], wt[0], ph, sh, dh, oph),
+               pet_hip_conv_trans_out_dim(in[2], wt[1], pw, sw, dw, opw), wt[3]};
+    outputs[0]->setDims(ret);
+    outputs[0]->setType(Tensor::Input);
+    return ret;
+}
+
+void ConvTransOp::setPaddingMode() {
+    auto in = inputs[0]->getDims(), out = outputs[0]->getDims();
+    if (in[1] == out[1] && in[2] == out[2])
+        padding = Same;
+    else if (ph == 0 && pw == 0)
+        padding = Valid;
+}
+
+bool ConvTransOp::checkValid(const TensorVec &ins) {
+    auto input = ins[0], weight = ins[1];
+    if (input->getType() != Tensor::Input || weight->getType() != Tensor::Weight)
+        return false;
+    if (input->getDims().size() != 4 || weight->getDims().size() != 4)
+        return false;
+    // grouped and dilated forms are asserted away upstream (src/Graph/operator.cc:1098-1101)
+    return input->getDims()[3] == weight->getDims()[2];
+}
+
+ConvArgs ConvTransOp::getArgs(int withPenalty) const {
+    auto in = inputs[0]->getDims();
+    auto pen = static_cast<const Tensor *>(inputs[0])->getPenalty();
+    auto wt = inputs[1]->getDims();
+    int n = in[0] + withPenalty * pen[0], h = in[1] + withPenalty * pen[1];
+    int w = in[2] + withPenalty * pen[2], f = in[3] + withPenalty * pen[3];
+    return ConvArgs{n, wt[3], h, w, f, wt[0], wt[1], ph, pw, sh, sw, dh, dw, 1, bias ? 1 : 0,
+                    (int)act};
+}
+
+int ConvTransOp::launch(pet_hip_stream_t stream) {
+    auto in = inputs[0]->getDims(), wt = inputs[1]->getDims();
+    return pet_hip_conv_trans_f32(inputs[0]->devicePtr(), inputs[1]->devicePtr(),
+                                  bias ? bias->devicePtr() : nullptr, outputs[0]->devicePtr(),
+                                  in[0], in[1], in[2], in[3], wt[0], wt[1], wt[3], ph, pw, sh, sw,
+                                  dh, dw, oph, opw, (int)act, stream);
+}
+
+// One kernel: nothing to choose between, where the reference loops over cuDNN's
+// backward-data algorithms (src/Graph/operator.cc:1113-1287). The memo key has no output
+// padding, as upstream (include/operator.h:597), so neither do the timed launches.
+double ConvTransOp::perf(PerfEngine *pe, int rounds, int warmupRounds) {
+    ConvArgs args = getArgs(pe->withPenalty());
+    if (pe->checkOpPerf(ConvTrans, args))
+        return pe->getOpPerf(ConvTrans, args);
+    int n, c, h, w, f, r, s, ph_, pw_, sh_, sw_, dh_, dw_, g, bi, ac;
+    std::tie(n, c, h, w, f, r, s, ph_, pw_, sh_, sw_, dh_, dw_, g, bi, ac) = args;
+    ConvTransResult res{INFINITY, 0, 0};
+    const int oh = pet_hip_conv_trans_out_dim(h, r, ph_, sh_, dh_, 0);
+    const int ow = pet_hip_conv_trans_out_dim(w, s, pw_, sw_, dw_, 0);
+    if (oh > 0 && ow > 0) {
+        float *x = pe->getInputPtr((size_t)n * h * w * f);
+        float *wt = pe->getWeightPtr((size_t)r * s * f * c);
+        float *y = pe->getOutputPtr((size_t)n * oh * ow * c);
+        float *b = pe->getBiasPtr((size_t)c);
+        if (x && wt && y && b)
+            res.time = timeFn(
+                [&](pet_hip_stream_t st) {
+                    return pet_hip_conv_trans_f32(x, wt, bi ? b : nullptr, y, n, h, w, f, r, s, c,
+                                                  ph_, pw_, sh_, sw_, dh_, dw_, 0, 0, ac, st);
+                },
+                rounds, warmupRounds);
+    }
+    pe->saveOpPerf(ConvTrans, args, res);
+    return res.time;
+}
+
+bool ConvTransOp::same(const ConvTransOp &rhs) {
+    bool ret = padding == Other ? (ph == rhs.ph && pw == rhs.pw) : padding == rhs.padding;
+    return ret && sh == rhs.sh && sw == rhs.sw && dh == rhs.dh && dw == rhs.dw;
+}
+
+std::string ConvTransOp::toString() const {
+    std::ostringstream os;
+    os << "ConvTrans[" << hash << "](";
+    if (inputs.size() == 2)
+        os << dimToString(inputs[0]->getDims()) << "," << dimToString(inputs[1]->getDims()) << ",";
+    os << "p=[" << ph << "," << pw << "],s=[" << sh << "," << sw << "],d=[" << dh << "," << dw
+       << "],op=[" << oph << ", " << opw << "],act=" << act;
+    if (inputs.size() == 2)
+        os << "," << tensorTag("input", inputs[0]) << "," << tensorTag("weight", inputs[1]) << ","
+           << tensorTag("output", outputs[0]);
+    os << ")";
+    return os.str();
+}
+
 // ---- Conv3dOp -------------------------------------------------------------------
 
 Conv3dOp::Conv3dOp(Tensor *input, Tensor *weight, Tensor *output, const Dim &pad,
@@ -1748,7 +1906,7 @@ std::string ReshapeOp::toString() const {
            dimToString(outputs[0]->getDims()) + ")";
 }
 
-// ---- band matrix products: shape rules only ------------------------------------
+// ---- band matrix products --------------------------------------------------------
 G2BMMOp::G2BMMOp(Tensor *A, Tensor *B, Tensor *C, int width, int dilation, Tensor *bias,
                  ActType act)
     : Operator(G2BMM, {A, B}, {C}), width(width), dilation(dilation), bias(bias), act(act) {
@@ -1797,16 +1955,49 @@ Dim G2BMMOp::computeShape() {
     return ret;
 }
 
-int G2BMMOp::launch(pet_hip_stream_t) { return PET_HIP_ERR_UNSUPPORTED; }
-double G2BMMOp::perf(PerfEngine *, int, int) { return INFINITY; }
+int G2BMMOp::launch(pet_hip_stream_t stream) {
+    const Dim &a = inputs[0]->getDims();
+    return pet_hip_g2bmm_f32(inputs[0]->devicePtr(), inputs[1]->devicePtr(),
+                             outputs[0]->devicePtr(), a[0], a[1], a[2], width, dilation, stream);
+}
+
+// Timed on the PerfEngine's scratch operands and memoised per (b, m, k, width, dilation),
+// as the reference times _sg2bmm (src/Graph/operator.cc:1424-1468).
+double G2BMMOp::perf(PerfEngine *pe, int rounds, int warmupRounds) {
+    G2BMMGBMMLArgs args = getArgs();
+    if (pe->checkOpPerf(G2BMM, args))
+        return pe->getOpPerf(G2BMM, args);
+    auto [b, m, k, w, d] = args;
+    double ms = INFINITY;
+    if (b > 0 && m > 0 && k > 0) {
+        float *A = pe->getMatA((size_t)b * m * k), *B = pe->getMatB((size_t)b * m * k);
+        float *C = pe->getMatC((size_t)b * m * (2 * w + 1));
+        if (A && B && C)
+            ms = timeFn(
+                [&](pet_hip_stream_t st) { return pet_hip_g2bmm_f32(A, B, C, b, m, k, w, d, st); },
+                rounds, warmupRounds);
+    }
+    pe->saveOpPerf(G2BMM, args, (float)ms);
+    return pe->getOpPerf(G2BMM, args);
+}
+
 std::string G2BMMOp::toString() const {
-    return "G2BMM(width=" + std::to_string(width) + ",dilation=" + std::to_string(dilation) + ")";
+    std::ostringstream os;
+    os << "G2BMM[" << hash << "](";
+    if (inputs.size() == 2)
+        os << dimToString(inputs[0]->getDims()) << "," << dimToString(inputs[1]->getDims()) << ",";
+    os << "width=" << width << ",dilation=" << dilation << ",act=" << act;
+    if (inputs.size() == 2)
+        os << "," << tensorTag("A", inputs[0]) << "," << tensorTag("B", inputs[1]) << ","
+           << tensorTag("C", outputs[0]);
+    os << ")";
+    return os.str();
 }
 
 GBMMLOp::GBMMLOp(Tensor *A, Tensor *B, Tensor *C, int dilation, Tensor *bias, ActType act)
     : Operator(GBMML, {A, B}, {C}), dilation(dilation), bias(bias), act(act) {
-    if (A->getType() == Tensor::Input && B->getType() == Tensor::Input)
-        B->setType(Tensor::Weight);
+    // both operands stay inputs: in attention neither is a constant
+    // (src/Graph/operator.cc:1489-1493)
     assert(checkValid({A, B}));
     computeShape();
     initHash();
@@ -1850,10 +2041,43 @@ Dim GBMMLOp::computeShape() {
     return ret;
 }
 
-int GBMMLOp::launch(pet_hip_stream_t) { return PET_HIP_ERR_UNSUPPORTED; }
-double GBMMLOp::perf(PerfEngine *, int, int) { return INFINITY; }
+int GBMMLOp::launch(pet_hip_stream_t stream) {
+    const Dim &a = inputs[0]->getDims();
+    return pet_hip_gbmml_f32(inputs[0]->devicePtr(), inputs[1]->devicePtr(),
+                             outputs[0]->devicePtr(), a[0], a[1], (a[2] - 1) / 2,
+                             inputs[1]->getDims()[2], dilation, stream);
+}
+
+// As the reference times _sgbmml (src/Graph/operator.cc:1560-1596).
+double GBMMLOp::perf(PerfEngine *pe, int rounds, int warmupRounds) {
+    G2BMMGBMMLArgs args = getArgs();
+    if (pe->checkOpPerf(GBMML, args))
+        return pe->getOpPerf(GBMML, args);
+    auto [b, m, n, w, d] = args;
+    double ms = INFINITY;
+    if (b > 0 && m > 0 && n > 0) {
+        float *A = pe->getMatA((size_t)b * m * (2 * w + 1)), *B = pe->getMatB((size_t)b * m * n);
+        float *C = pe->getMatC((size_t)b * m * n);
+        if (A && B && C)
+            ms = timeFn(
+                [&](pet_hip_stream_t st) { return pet_hip_gbmml_f32(A, B, C, b, m, w, n, d, st); },
+                rounds, warmupRounds);
+    }
+    pe->saveOpPerf(GBMML, args, (float)ms);
+    return pe->getOpPerf(GBMML, args);
+}
+
 std::string GBMMLOp::toString() const {
-    return "GBMML(dilation=" + std::to_string(dilation) + ")";
+    std::ostringstream os;
+    os << "GBMML[" << hash << "](";
+    if (inputs.size() == 2)
+        os << dimToString(inputs[0]->getDims()) << "," << dimToString(inputs[1]->getDims()) << ",";
+    os << "dilation=" << dilation << ",act=" << act;
+    if (inputs.size() == 2)
+        os << "," << tensorTag("A", inputs[0]) << "," << tensorTag("B", inputs[1]) << ","
+           << tensorTag("C", outputs[0]);
+    os << ")";
+    return os.str();
 }
 
 // ---- point dependences ------------------------------------------------------------

@@ -172,6 +172,55 @@ def matmul(A, B, transA=False, transB=False, bias=None, act="none", out=None, re
     return out
 
 
+def conv_trans_out_dim(i, k, p, s, d, op):
+    """ConvTransOp::computeShape, src/Graph/operator.cc:1066-1067."""
+    return (i - 1) * s - 2 * p + d * (k - 1) + op + 1
+
+
+def conv_trans(x, w, ph, pw, sh=1, sw=1, dh=1, dw=1, oph=0, opw=0, bias=None, act="none",
+               out=None):
+    """ConvTransOp: x NHWF [n,h,w,f], w RSFC [r,s,f,c] -> NHWC [n,oh,ow,c]."""
+    _chk(x, w, bias, out)
+    n, h, wd, f = x.shape
+    r, s, f2, c = w.shape
+    if f != f2:
+        raise abi.PetHipError(1, "input features differ from the weight's")
+    oh = conv_trans_out_dim(h, r, ph, sh, dh, oph)
+    ow = conv_trans_out_dim(wd, s, pw, sw, dw, opw)
+    if out is None:
+        out = torch.empty((n, max(oh, 0), max(ow, 0), c), device=x.device, dtype=torch.float32)
+    abi.call("pet_hip_conv_trans_f32", _ptr(x), _ptr(w), _ptr(bias), _ptr(out), n, h, wd, f, r, s,
+             c, ph, pw, sh, sw, dh, dw, oph, opw, abi.ACT[act], _stream())
+    return out
+
+
+def g2bmm(A, B, width, dilation=1, out=None):
+    """G2BMMOp: A, B [bs,m,k] -> [bs,m,2*width+1]."""
+    _chk(A, B, out)
+    bs, m, k = A.shape
+    if tuple(B.shape) != tuple(A.shape):
+        raise abi.PetHipError(1, "g2bmm operands differ in shape")
+    if out is None:
+        out = torch.empty((bs, m, 2 * width + 1), device=A.device, dtype=torch.float32)
+    abi.call("pet_hip_g2bmm_f32", _ptr(A), _ptr(B), _ptr(out), bs, m, k, width, dilation,
+             _stream())
+    return out
+
+
+def gbmml(A, B, dilation=1, out=None):
+    """GBMMLOp: A [bs,m,2w+1], B [bs,m,n] -> [bs,m,n]."""
+    _chk(A, B, out)
+    bs, m, band = A.shape
+    if band % 2 == 0 or tuple(B.shape[:2]) != (bs, m):
+        raise abi.PetHipError(1, "gbmml operands do not agree")
+    n = B.shape[2]
+    if out is None:
+        out = torch.empty((bs, m, n), device=A.device, dtype=torch.float32)
+    abi.call("pet_hip_gbmml_f32", _ptr(A), _ptr(B), _ptr(out), bs, m, (band - 1) // 2, n,
+             dilation, _stream())
+    return out
+
+
 def transpose_params(in_dims, split, after, factor):
     """TransposeOp::setParam (include/operator.h:1124-1144) and the flat-dim
     rule of TransposeOp::computeShape (src/Graph/operator.cc:2340-2381).

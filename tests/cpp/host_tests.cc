@@ -24,6 +24,8 @@ int oracle_matmul_f32(const float *A, const float *B, float *C, int b, int m, in
                       int transA, int transB);
 int oracle_transpose_f32(const float *x, float *y, const int *flatDim, const int *after, int nflat);
 int oracle_conv_out_dim(int i, int k, int p, int s, int d);
+int oracle_g2bmm_f32(const float *A, const float *B, float *C, int bs, int m, int k, int w, int d);
+int oracle_gbmml_f32(const float *A, const float *B, float *C, int bs, int m, int w, int n, int d);
 }
 
 #define EXPECT(cond)                                                                           \
@@ -850,6 +852,119 @@ static bool test_conv_merge_programs() {
     return true;
 }
 
+// src/Test/convtrans_test_1.cc: both cases with the inputs that test builds and the
+// expected values it holds. The operator is NHWC; Graph::convTrans wraps it in the NCHW
+// transposes, and its output is then in the order the reference lists (PyTorch's NCHW).
+static bool convTransCase(int h, int w, int f, int r, int s, int c, int p, int st,
+                          const std::vector<float> &ans) {
+    const int n = 1;
+    // operator level: X[n,h,w,f] = iota, K[r,s,f,c] = ((f*R + r)*S + s)*C + c
+    Tensor input({n, h, w, f}), weight({r, s, f, c});
+    std::vector<float> xv((size_t)n * h * w * f), kv((size_t)r * s * f * c);
+    for (size_t i = 0; i < xv.size(); ++i)
+        xv[i] = (float)i;
+    for (int rr = 0; rr < r; ++rr)
+        for (int ss = 0; ss < s; ++ss)
+            for (int ff = 0; ff < f; ++ff)
+                for (int cc = 0; cc < c; ++cc)
+                    kv[((rr * s + ss) * f + ff) * c + cc] = (float)(((ff * r + rr) * s + ss) * c + cc);
+    input.setData(xv.data());
+    weight.setData(kv.data());
+    ConvTransOp op(&input, &weight, p, p, st, st, 1, 1);
+    Tensor *out = op.getOutputs()[0];
+    const int oh = (h - 1) * st - 2 * p + (r - 1) + 1, ow = (w - 1) * st - 2 * p + (s - 1) + 1;
+    EXPECT(out->getDims() == (Dim{n, oh, ow, c}));
+    EXPECT(op.compute() != nullptr);
+    EXPECT(ans.size() == out->size());
+    const float *o = out->getDataPtr();
+    for (int cc = 0; cc < c; ++cc)
+        for (int hh = 0; hh < oh; ++hh)
+            for (int ww = 0; ww < ow; ++ww)
+                EXPECT(o[(hh * ow + ww) * c + cc] == ans[(cc * oh + hh) * ow + ww]);
+    // graph level: the same numbers as NCHW tensors
+    Graph g;
+    auto gi = g.tensor({n, f, h, w}), gw = g.tensor({f, c, r, s}), go = g.tensor({n, c, oh, ow});
+    g.convTrans(gi, gw, go, p, p, st, st, 1, 1);
+    g.updateConnection();
+    auto sg = std::make_shared<SubGraph>(g.getOperators());
+    std::vector<float> xn(xv.size()), kn(kv.size());
+    for (int hh = 0; hh < h; ++hh)
+        for (int ww = 0; ww < w; ++ww)
+            for (int ff = 0; ff < f; ++ff)
+                xn[(ff * h + hh) * w + ww] = xv[(hh * w + ww) * f + ff];
+    for (int rr = 0; rr < r; ++rr)
+        for (int ss = 0; ss < s; ++ss)
+            for (int ff = 0; ff < f; ++ff)
+                for (int cc = 0; cc < c; ++cc)
+                    kn[((ff * c + cc) * r + rr) * s + ss] = kv[((rr * s + ss) * f + ff) * c + cc];
+    for (auto t : sg->getInputs())
+        t->setData(t->getDims() == (Dim{n, f, h, w}) ? xn.data() : kn.data());
+    EXPECT(sg->compute());
+    EXPECT(sg->getOutputs().size() == 1 && sg->getOutputs()[0]->size() == ans.size());
+    EXPECT(equalArrays(sg->getOutputs()[0]->getDataPtr(), ans.data(), ans.size()));
+    // ... and replayed by the graph runtime, with a timing from the PerfEngine
+    CodeEngine ce;
+    auto sg2 = std::make_shared<SubGraph>(g.getOperators());
+    for (auto t : sg2->getInputs())
+        t->setData(t->getDims() == (Dim{n, f, h, w}) ? xn.data() : kn.data());
+    auto exec = ce.instantiate(sg2);
+    EXPECT(exec != nullptr && exec->launch() && exec->sync());
+    sg2->getOutputs()[0]->deviceWritten();
+    EXPECT(equalArrays(sg2->getOutputs()[0]->getDataPtr(), ans.data(), ans.size()));
+    EXPECT(ce.genCode(sg2).find("pet_hip_conv_trans_f32(") != std::string::npos);
+    PerfEngine pe;
+    double t1 = op.perf(&pe, 5, 2), t2 = op.perf(&pe, 5, 2);
+    EXPECT(std::isfinite(t1) && t1 > 0 && t1 == t2);
+    return true;
+}
+
+static bool test_convtrans_reference_vectors() {
+    EXPECT(convTransCase(2, 2, 3, 4, 4, 2, 1, 2,
+                         {190,  740,  770,  592,  992,  2704, 2836, 1832, 1184, 3232, 3364,
+                          2168, 1114, 2660, 2762, 1624, 193,  755,  785,  604,  1016, 2770,
+                          2902, 1874, 1208, 3298, 3430, 2210, 1135, 2711, 2813, 1654}));
+    EXPECT(convTransCase(1, 1, 3, 2, 2, 2, 0, 1, {40, 46, 52, 58, 43, 49, 55, 61}));
+    return true;
+}
+
+// Sliding-window attention through the band operators: G2BMM, then GBMML on its result,
+// against the oracle; shape rules and the memoised timings.
+static bool test_band_matmuls() {
+    const int bs = 2, m = 70, k = 16, w = 5, d = 2;
+    Graph g;
+    auto q = g.tensor({bs, m, k}), key = g.tensor({bs, m, k}), v = g.tensor({bs, m, k});
+    auto s = g.g2bmm(q, key, w, d);
+    EXPECT(s->getOutputs()[0]->getDims() == (Dim{bs, m, 2 * w + 1}));
+    auto o = g.gbmml(s->getOutputs()[0], v, d);
+    EXPECT(o->getOutputs()[0]->getDims() == (Dim{bs, m, k}));
+    g.updateConnection();
+    auto sg = std::make_shared<SubGraph>(g.getOperators());
+    EXPECT(sg->getInputs().size() == 3);
+    for (size_t i = 0; i < 3; ++i)
+        fillSmall(sg->getInputs()[i], 3 + (int)i);
+    EXPECT(sg->compute());
+    // which graph input is which: q and key feed the first operator, v the second
+    Operator *first = nullptr, *second = nullptr;
+    for (auto op : sg->getOperators())
+        (op->getType() == Operator::G2BMM ? first : second) = op;
+    EXPECT(first && second);
+    std::vector<float> band((size_t)bs * m * (2 * w + 1)), ref((size_t)bs * m * k);
+    oracle_g2bmm_f32(first->getInputs()[0]->getDataPtr(), first->getInputs()[1]->getDataPtr(),
+                     band.data(), bs, m, k, w, d);
+    EXPECT(equalArrays(first->getOutputs()[0]->getDataPtr(), band.data(), band.size()));
+    oracle_gbmml_f32(band.data(), second->getInputs()[1]->getDataPtr(), ref.data(), bs, m, w, k, d);
+    EXPECT(equalArrays(sg->getOutputs()[0]->getDataPtr(), ref.data(), ref.size()));
+    PerfEngine pe;
+    double t1 = first->perf(&pe, 5, 2), t2 = second->perf(&pe, 5, 2);
+    EXPECT(std::isfinite(t1) && t1 > 0 && std::isfinite(t2) && t2 > 0);
+    EXPECT(first->perf(&pe, 5, 2) == t1);
+    CodeEngine ce;
+    std::string code = ce.genCode(sg);
+    EXPECT(code.find("pet_hip_g2bmm_f32(") != std::string::npos &&
+           code.find("pet_hip_gbmml_f32(") != std::string::npos);
+    return true;
+}
+
 int main(int argc, char **argv) {
     std::vector<std::pair<std::string, std::function<bool()>>> cases = {
         {"conv_vs_oracle", test_conv_vs_oracle},
@@ -871,6 +986,8 @@ int main(int argc, char **argv) {
         {"batchnorm_pow_div", test_batchnorm_pow_div},
         {"gather_reduce_mean", test_gather_reduce_mean},
         {"conv_merge_programs", test_conv_merge_programs},
+        {"convtrans_reference_vectors", test_convtrans_reference_vectors},
+        {"band_matmuls", test_band_matmuls},
     };
     std::string only = argc > 1 ? argv[1] : "";
     if (argc > 2)

@@ -20,7 +20,7 @@ CASES = ["conv_vs_oracle", "conv_invalid_groups", "transpose_n2h_h2n", "batch_ge
          "split_ratio_and_eltwise", "conv_merge_programs", "conv3d_prepacked_graph",
          "random_graphs_replay_equals_eager", "batchnorm_pow_div",
          "gather_reduce_mean", "launch_fusion_block", "alias_plan_shared_storage",
-         "two_conv_verification"]
+         "two_conv_verification", "convtrans_reference_vectors", "band_matmuls"]
 
 
 def test_host_library_is_built_and_exports_the_operator_classes():

@@ -480,3 +480,106 @@ def test_unpinned_float_pieces_vs_torch():
         F.layer_norm(torch.from_numpy(s).double(), (17,), torch.from_numpy(g).double(),
                      torch.from_numpy(be).double(), 1e-5).float().numpy(),
         rtol=1e-5, atol=1e-6)
+
+
+# ---- ConvTrans, G2BMM, GBMML ----------------------------------------------------------
+
+def test_conv_trans_reproduces_the_reference_vectors():
+    """The only operator whose expected outputs the reference itself holds
+    (src/Test/convtrans_test_1.cc:62-77, 120-135), in both tiers."""
+    from convtrans_cases import reference_cases
+    for dtype in (np.float32, np.uint32):
+        for x, K, prm, want in reference_cases(dtype):
+            got = oracle.conv_trans(x, K, prm["ph"], prm["pw"], prm["sh"], prm["sw"], prm["dh"],
+                                    prm["dw"])
+            assert got.shape == want.shape
+            np.testing.assert_array_equal(got, want)
+
+
+CONV_TRANS_CASES = [
+    # n, h, w, f, r, s, c, ph, pw, sh, sw, oph, opw
+    (2, 5, 6, 4, 3, 3, 5, 1, 1, 2, 2, 0, 0),
+    (1, 4, 4, 8, 4, 4, 40, 1, 1, 2, 2, 0, 0),
+    (1, 7, 5, 2, 3, 2, 3, 0, 1, 1, 2, 0, 0),
+    (1, 5, 5, 3, 3, 3, 2, 1, 1, 2, 2, 1, 1),
+    (1, 5, 4, 2, 5, 5, 3, 2, 2, 3, 3, 0, 0),
+    (3, 3, 3, 16, 1, 1, 7, 0, 0, 1, 1, 0, 0),
+]
+
+
+def _torch_conv_trans(x, K, ph, pw, sh, sw, oph, opw):
+    import torch
+    import torch.nn.functional as F
+    y = F.conv_transpose2d(torch.from_numpy(x).permute(0, 3, 1, 2).double(),
+                           torch.from_numpy(K).permute(2, 3, 0, 1).double(), stride=(sh, sw),
+                           padding=(ph, pw), output_padding=(oph, opw))
+    return y.permute(0, 2, 3, 1).numpy()
+
+
+@pytest.mark.parametrize("case", CONV_TRANS_CASES)
+def test_conv_trans_vs_torch(case):
+    """Where the reference's tap skip cannot trigger ((h + 2ph - r) % sh < 2) the
+    operator is torch's conv_transpose2d with weight[f][c][r][s] = K[r][s][f][c]."""
+    n, h, w, f, r, s, c, ph, pw, sh, sw, oph, opw = case
+    assert (h + 2 * ph - r) % sh < 2 and (w + 2 * pw - s) % sw < 2
+    rng = np.random.default_rng(sum(case))
+    x = rng.integers(-3, 4, (n, h, w, f)).astype(np.float32)
+    K = rng.integers(-3, 4, (r, s, f, c)).astype(np.float32)
+    got = oracle.conv_trans(x, K, ph, pw, sh, sw, 1, 1, oph, opw)
+    np.testing.assert_array_equal(got, _torch_conv_trans(x, K, ph, pw, sh, sw, oph, opw))
+    xf = rng.standard_normal((n, h, w, f)).astype(np.float32)
+    Kf = rng.standard_normal((r, s, f, c)).astype(np.float32)
+    np.testing.assert_allclose(oracle.conv_trans(xf, Kf, ph, pw, sh, sw, 1, 1, oph, opw),
+                               _torch_conv_trans(xf, Kf, ph, pw, sh, sw, oph, opw), rtol=1e-5,
+                               atol=1e-5)
+
+
+def test_conv_trans_tap_skip_of_the_reference():
+    """src/Graph/operator.cc:953-956 leaves out the flipped taps rr > r - ah with
+    ah = (h + 2ph - r) % sh, i.e. the kernel rows t = r-1-rr < ah - 1: with stride 3,
+    h = 6, r = 4, ah = 2, that is kernel row 0. Pinned as torch's result on a kernel
+    whose row 0 is zero."""
+    rng = np.random.default_rng(3)
+    x = rng.integers(-3, 4, (1, 6, 5, 2)).astype(np.float32)
+    K = rng.integers(-3, 4, (4, 3, 2, 3)).astype(np.float32)
+    got = oracle.conv_trans(x, K, 0, 0, 3, 1)
+    Kz = K.copy()
+    Kz[0] = 0
+    np.testing.assert_array_equal(got, _torch_conv_trans(x, Kz, 0, 0, 3, 1, 0, 0))
+    assert not np.array_equal(got, _torch_conv_trans(x, K, 0, 0, 3, 1, 0, 0))
+
+
+def _band_dense(A, B, w, d):
+    """G2BMM from the dense product: C[b,i,j] = (A B^T)[b, i, i + d (j - w)], 0 outside."""
+    bs, m, _ = A.shape
+    full = np.einsum("bik,brk->bir", A.astype(np.float64), B.astype(np.float64))
+    out = np.zeros((bs, m, 2 * w + 1))
+    for i in range(m):
+        for j in range(2 * w + 1):
+            r = i + d * (j - w)
+            if 0 <= r < m:
+                out[:, i, j] = full[:, i, r]
+    return out
+
+
+@pytest.mark.parametrize("bs,m,k,w,d", [(2, 9, 5, 2, 1), (1, 17, 8, 3, 2), (3, 40, 16, 6, 4),
+                                        (1, 5, 3, 7, 1)])
+def test_g2bmm_gbmml_vs_dense_numpy(bs, m, k, w, d):
+    rng = np.random.default_rng(bs + m + k + w + d)
+    A = rng.integers(-3, 4, (bs, m, k)).astype(np.float32)
+    B = rng.integers(-3, 4, (bs, m, k)).astype(np.float32)
+    np.testing.assert_array_equal(oracle.g2bmm(A, B, w, d), _band_dense(A, B, w, d))
+    # GBMML: scatter the band into a dense [m, m] matrix and multiply
+    P = rng.integers(-3, 4, (bs, m, 2 * w + 1)).astype(np.float32)
+    V = rng.integers(-3, 4, (bs, m, k)).astype(np.float32)
+    dense = np.zeros((bs, m, m))
+    for i in range(m):
+        for j in range(2 * w + 1):
+            r = i + d * j - d * w
+            if 0 <= r < m:
+                dense[:, i, r] += P[:, i, j]
+    np.testing.assert_array_equal(oracle.gbmml(P, V, d), dense @ V.astype(np.float64))
+    # the uint32 tier agrees on non-negative data
+    Au, Bu = np.abs(A).astype(np.uint32), np.abs(B).astype(np.uint32)
+    np.testing.assert_array_equal(oracle.g2bmm(Au, Bu, w, d),
+                                  _band_dense(np.abs(A), np.abs(B), w, d).astype(np.uint32))

@@ -33,6 +33,8 @@ def max_rel_err(got, ref, mag):
     ref = ref.astype(np.float64)
     mag = mag.astype(np.float64)
     err = np.abs(got - ref)
-    elem = np.max(np.maximum(err - ULP * mag, 0.0) / np.maximum(np.abs(ref), FLOOR * mag))
+    # an output without terms (mag == 0) must be exactly 0: any error there divides by 1e-300
+    den = np.maximum(np.maximum(np.abs(ref), FLOOR * mag), 1e-300)
+    elem = np.max(np.maximum(err - ULP * mag, 0.0) / den)
     norm = np.max(err) / max(np.max(np.abs(ref)), 1e-300)
     return float(max(elem, norm))
