@@ -67,7 +67,14 @@ typedef enum pet_hip_call_flags {
      * which the readers' second ReLU does not change. */
     PET_HIP_CALL_DEFER_RELU = 2,
     PET_HIP_CALL_X_RELU = 4,   /* use max(x, 0) for x */
-    PET_HIP_CALL_RES_RELU = 8  /* use max(residual, 0) for the residual */
+    PET_HIP_CALL_RES_RELU = 8, /* use max(residual, 0) for the residual */
+    /* pet_hip_bmm_ex_f32 only. A holds one [m,k] (or [k,m]) matrix that every batch entry
+     * multiplies: an Extend of the lhs along dim 0 in front of a BatchMatmul (PET's matmul
+     * merge, src/Mutant/generator.cc:1495-1552) folded into the addressing. */
+    PET_HIP_CALL_A_SHARED = 16,
+    /* pet_hip_bmm_ex_f32 only. bias is [b, n], one vector per batch entry: the per-slab
+     * bias Adds that follow the Split of a merged BatchMatmul. */
+    PET_HIP_CALL_BIAS_PER_BATCH = 32
 } pet_hip_call_flags;
 
 /* Convolution algorithms, the counterpart of the cuDNN algorithm list ConvOp::perf
@@ -300,6 +307,24 @@ PET_HIP_API int pet_hip_g2bmm_f32(const float *A, const float *B, float *C, int 
                       int width, int dilation, pet_hip_stream_t stream);
 PET_HIP_API int pet_hip_gbmml_f32(const float *A, const float *B, float *C, int bs, int m, int width,
                       int n, int dilation, pet_hip_stream_t stream);
+
+/* Multi-head attention core in one launch: for each batch entry and head h,
+ * out[:, h*dh:(h+1)*dh] = softmax(scale * Q_h K_h^T) V_h, with Q, K, V [seq, heads*dh]
+ * matrices whose rows are ldq / ldk / ldv floats apart (so the three slabs of a merged
+ * projection, or three separate projections, are read in place) and out [seq, heads*dh]
+ * with row stride ldo; the stride_* are the distances between batch entries. scale is
+ * multiplied by *scale_dev when that is not NULL (a one-element tensor in the graph).
+ * It stands for the operator sequence Transpose (head split) x 3, Matmul(transB), Mul,
+ * Softmax, Matmul, Transpose (head merge), Reshape, i.e. MatmulOp::compute
+ * (src/Graph/operator.cc:620-654) twice around a row softmax; the reference emits those
+ * as cuBLAS calls and an inline softmax (src/Graph/code_engine.cc:1103-1169, 1707-1731).
+ * seq <= 512, dh in {32, 64, 96, 128}, Q and K rows 16-byte aligned; PET_HIP_ERR_UNSUPPORTED
+ * otherwise (callers then run the operators one by one). */
+PET_HIP_API int pet_hip_attention_f32(const float *q, const float *k, const float *v, float *out,
+                          int batch, int heads, int seq, int dh, int ldq, int ldk, int ldv,
+                          int ldo, long long stride_q, long long stride_k, long long stride_v,
+                          long long stride_o, float scale, const float *scale_dev,
+                          pet_hip_stream_t stream);
 
 /* ---- layout operators (bit-exact copies) ---------------------------------*/
 

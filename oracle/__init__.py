@@ -485,3 +485,19 @@ def layernorm(x, gamma, beta, eps=1e-5):
                                ctypes.c_size_t(x.size // cols),
                                ctypes.c_size_t(cols), ctypes.c_float(eps))
     return y
+
+
+def attention(q, k, v, heads, scale):
+    """The operator sequence a fused attention launch stands for, one reference operator at
+    a time: head split (Transpose), scores = Matmul(Q, K, transB), Mul by the scale, row
+    Softmax, Matmul with V, head merge (Transpose + Reshape). q, k, v: [seq, heads*dh]."""
+    seq, width = q.shape
+    dh = width // heads
+
+    def to_heads(t):  # [seq, heads*dh] -> [heads, seq, dh]
+        return transpose(_c(t), 1, [1, 0, -1], dh)
+
+    s = matmul(to_heads(q), to_heads(k), False, True)
+    s = eltwise("mul", [s, np.full((1,), scale, dtype=np.float32)], s.shape)
+    ctx = matmul(softmax(s), to_heads(v))
+    return transpose(ctx, -1, [1, 0, 2]).reshape(seq, width)

@@ -13,7 +13,7 @@ LIB_PATH = os.path.join(_HERE, "lib", "libpet_hip.so")
 ACT = {"none": 0, "relu": 1, "sigmoid": 2, "tanh": 3, "gelu": 4, None: 0}
 ELT = {"add": 0, "sub": 1, "mul": 2, "div": 3}
 # pet_hip_call_flags
-Y_INITIALISED, DEFER_RELU, X_RELU, RES_RELU = 1, 2, 4, 8
+Y_INITIALISED, DEFER_RELU, X_RELU, RES_RELU, A_SHARED, BIAS_PER_BATCH = 1, 2, 4, 8, 16, 32
 
 
 class Fill(ctypes.Structure):
@@ -73,6 +73,7 @@ SIGNATURES = {
     "pet_hip_conv_trans_f32": [_vp] * 4 + [_i] * 16 + [_vp],
     "pet_hip_g2bmm_f32": [_vp] * 3 + [_i] * 5 + [_vp],
     "pet_hip_gbmml_f32": [_vp] * 3 + [_i] * 5 + [_vp],
+    "pet_hip_attention_f32": [_vp] * 4 + [_i] * 8 + [ctypes.c_longlong] * 4 + [ctypes.c_float, _vp, _vp],
     "pet_hip_transpose": [_vp, _vp, _c_int_p, _c_int_p, _i, _vp],
     "pet_hip_trans_chain": [_vp, _vp, _c_int_p, _i, _c_int_p, _i, _c_int_p, _c_int_p, _c_int_p, _vp],
     "pet_hip_split": [_vp, ctypes.POINTER(_vp), _i, _c_int_p, _i, _i, _c_int_p, _vp],

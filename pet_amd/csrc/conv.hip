@@ -1142,7 +1142,7 @@ int try_launch_plane(const ConvParams &p, hipStream_t stream) {
     const long long w_bytes = 4ll * p.F * p.K;
     if (in_bytes >= (1ll << 31) || w_bytes >= (1ll << 31))
         return -1;
-    if (((uintptr_t)p.w & 15) != 0)
+    if (((uintptr_t)p.w & 15) != 0 || p.w_shared || p.bias_gstride)
         return -1;
     const bool is3d = p.T > 1 || p.KT > 1 || p.pt > 0 || p.st > 1;
     const int rs = p.R * p.S;
@@ -1324,6 +1324,8 @@ int bmm_as_grouped_1x1(const float *A, const float *B, float *C, const float *bi
                        unsigned flags, int *dry) {
     if (k % 32 != 0 || b > 65535)
         return -1;
+    const bool a_shared = (flags & PET_HIP_CALL_A_SHARED) != 0;
+    const bool bias_per_batch = (flags & PET_HIP_CALL_BIAS_PER_BATCH) != 0;
     // the group view holds b*k "channels" of n pixels and b*m "filters" of k taps: both
     // must stay inside 32-bit element counts and the 2 GiB range of a buffer resource
     if ((long long)b * k >= (1ll << 31) || (long long)b * m >= (1ll << 31) ||
@@ -1366,6 +1368,8 @@ int bmm_as_grouped_1x1(const float *A, const float *B, float *C, const float *bi
     p.fd_ohw = make_fastdiv((unsigned)n);
     p.fd_ow = make_fastdiv((unsigned)n);
     p.fd_splitk = make_fastdiv(1);
+    p.w_shared = a_shared;
+    p.bias_gstride = bias_per_batch ? n : 0;
     const int rc = try_launch_direct(p, stream);
     return rc >= 0 ? rc : try_launch_plane(p, stream);
 }

@@ -47,6 +47,9 @@ struct ConvParams {
                      // array (the entry point that allocates nothing); implies the ordered sum
     int res_first;   // accumulating launch into an initialised y: the workgroup that holds a
                      // tile's first K step adds the residual along with its partial sums
+    int w_shared;    // every group reads the filters of group 0 (a matmul whose A operand has
+                     // one batch entry: an Extend of the lhs folded into the addressing)
+    int bias_gstride; // bias_mode 2: floats between the groups' bias vectors (0: one for all)
     FastDiv fd_krs, fd_rs, fd_s;     // k -> (c, kt, r, s)
     FastDiv fd_opix, fd_ohw, fd_ow;  // pixel -> (n, ot, oh, ow)
 };

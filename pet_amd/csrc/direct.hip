@@ -92,7 +92,7 @@ __global__ __launch_bounds__(Cfg::NT) void conv_direct_kernel(ConvParams p) {
 #pragma unroll
     for (int tm = 0; tm < TM; ++tm)
         voffA[tm] = ((unsigned)min(m0 + tm * 32 + l32, p.M - 1) * (unsigned)p.K + hk * KH) * 4u;
-    const __amdgpu_buffer_rsrc_t ra = make_rsrc(p.w + (long long)g * p.M * p.K);
+    const __amdgpu_buffer_rsrc_t ra = make_rsrc(p.w + (p.w_shared ? 0ll : (long long)g * p.M * p.K));
 
     float a[TM][KH], b[TN][KH];
     floatx16 acc[TM][TN];
@@ -199,7 +199,7 @@ __global__ __launch_bounds__(Cfg::NT) void conv_direct_kernel(ConvParams p) {
         if (bias)
             v += bias[f];
         if (p.bias && p.bias_mode == 2)
-            v += p.bias[rem];
+            v += p.bias[(size_t)g * p.bias_gstride + rem];
         if (p.res) {
             const float rv = p.res[yi];
             v += p.res_relu ? fmaxf(rv, 0.f) : rv;
@@ -340,6 +340,8 @@ int try_launch_direct(const ConvParams &p0, hipStream_t stream) {
         c.splitk = p.force_splitk;
     const int nchunks = p.cpg / (rs9 ? 8 : 32);
     c.splitk = std::max(1, std::min(c.splitk, nchunks));
+    if (p.w_shared || p.bias_gstride) // the initialising launch knows one bias vector only
+        c.splitk = 1;
     const bool exists = (c.tm == 1 || c.tm == 2) && (c.tn == 1 || c.tn == 2) &&
                         (c.kw == 4 || c.kw == 8 || (c.kw == 16 && c.tm * c.tn == 1));
     if (!exists || (long long)p.G * c.splitk > 65535 ||

@@ -155,9 +155,12 @@ namespace {
 int bmm_common(int transA, int transB, int b, int m, int n, int k, const float *A, const float *B,
                float *C, const float *bias, const float *res, int act, pet_hip_stream_t stream,
                unsigned flags = 0, int *dry = nullptr) {
-    if (flags & ~(unsigned)(PET_HIP_CALL_Y_INITIALISED | 0xff00u))
+    if (flags & ~(unsigned)(PET_HIP_CALL_Y_INITIALISED | PET_HIP_CALL_A_SHARED |
+                            PET_HIP_CALL_BIAS_PER_BATCH | 0xff00u))
         return set_error(PET_HIP_ERR_INVALID,
-                         "matmul takes PET_HIP_CALL_Y_INITIALISED and an algorithm only");
+                         "matmul takes PET_HIP_CALL_Y_INITIALISED, PET_HIP_CALL_A_SHARED, "
+                         "PET_HIP_CALL_BIAS_PER_BATCH and an algorithm only");
+    const unsigned addressing = flags & (PET_HIP_CALL_A_SHARED | PET_HIP_CALL_BIAS_PER_BATCH);
     if (((flags >> 8) & 0xffu) >= PET_HIP_CONV_ALGO_COUNT)
         return set_error(PET_HIP_ERR_INVALID, "unknown algorithm %u", (flags >> 8) & 0xffu);
     if (dry) {
@@ -208,6 +211,20 @@ int bmm_common(int transA, int transB, int b, int m, int n, int k, const float *
                                     dry);
         if (rc >= 0)
             return rc;
+    }
+    if (addressing) {
+        // no kernel with that addressing applies: one product per batch entry
+        for (int i = 0; i < b; ++i) {
+            const float *Ai = (flags & PET_HIP_CALL_A_SHARED) ? A : A + (size_t)i * m * k;
+            const float *bi = bias && (flags & PET_HIP_CALL_BIAS_PER_BATCH) ? bias + (size_t)i * n
+                                                                            : bias;
+            int rc = bmm_common(transA, transB, 1, m, n, k, Ai, B + (size_t)i * k * n,
+                                C + (size_t)i * m * n, bi, res ? res + (size_t)i * m * n : nullptr,
+                                act, stream, flags & ~addressing, dry);
+            if (rc != PET_HIP_OK || dry)
+                return rc;
+        }
+        return PET_HIP_OK;
     }
     if (dry) // the general kernel never accumulates into C
         return PET_HIP_OK;

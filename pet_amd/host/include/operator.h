@@ -913,6 +913,7 @@ class SoftmaxOp : public Operator {
   public:
     SoftmaxOp(Tensor *input, Tensor *output, int axis);
     SoftmaxOp(const SoftmaxOp &rhs) : Operator(rhs), axis(rhs.axis) {}
+    int getAxis() const { return axis; }
     SoftmaxOp *clone() override { return new SoftmaxOp(*this); }
     Dim computeShape() override;
     double perf(PerfEngine *pe, int rounds = 200, int warmupRounds = 200) override;

@@ -316,6 +316,129 @@ LaunchPlan planLaunchFlags(const OpVec &order, const TensorVec &graphOutputs,
     return plan;
 }
 
+// The attention core as one launch: head-split Transposes of Q, K and V, Matmul(transB),
+// Mul by a one-element scale, Softmax over the last axis, Matmul with V and the head-merge
+// Transpose run as pet_hip_attention_f32 in place of the head merge, reading the
+// [seq, heads*dh] projections and writing the merged [seq, heads*dh] result; none of the
+// tensors in between is materialised. Everything in between must be used by this chain only.
+struct FusedAttention {
+    Tensor *q = nullptr, *k = nullptr, *v = nullptr; // [seq, heads*dh]
+    Tensor *scale = nullptr;                         // one element, or none
+    Tensor *out = nullptr;                           // [seq, heads, dh]
+    int heads = 0, seq = 0, dh = 0;
+};
+
+struct FusedAttentions {
+    std::set<const Operator *> absorbed;
+    std::map<const Operator *, FusedAttention> atMerge; // keyed by the head-merge transpose
+};
+
+bool swapsFirstTwoOfThree(TransposeOp *tr) {
+    auto ba = tr->getBeforeAndAfter();
+    return ba.second.asVector() == std::vector<int>{1, 0, 2} && tr->getPaddingSize().first == 0 &&
+           tr->getPaddingSize().second == 0;
+}
+
+FusedAttentions planAttention(const OpVec &order, const TensorVec &graphOutputs,
+                              const std::set<const Operator *> &skipped,
+                              const TransposeChains &rows) {
+    FusedAttentions plan;
+    static const bool off = getenv("PET_HOST_NO_ATTENTION_FUSION") != nullptr;
+    if (off)
+        return plan;
+    std::set<const Tensor *> outs(graphOutputs.begin(), graphOutputs.end());
+    auto soleUser = [&](Tensor *t) -> Operator * {
+        return t->getInputOf().size() == 1 && !outs.count(t) ? t->getInputOf()[0] : nullptr;
+    };
+    auto plainMatmul = [&](Operator *op, bool transB) -> MatmulOp * {
+        auto mm = dynamic_cast<MatmulOp *>(op);
+        if (!mm || skipped.count(op) || mm->getTransA() || mm->getTransB() != transB ||
+            mm->getBias() || mm->getAct() != Operator::None)
+            return nullptr;
+        return mm;
+    };
+    // [seq, heads*dh] --split the columns by dh, heads to the front--> [heads, seq, dh]
+    auto headSplit = [&](Tensor *t, int heads, int seq, int dh) -> Tensor * {
+        auto tr = dynamic_cast<TransposeOp *>(t->getOutputOf());
+        if (!tr || skipped.count(tr) || rows.folded.count(tr) || rows.chains.count(tr) ||
+            soleUser(t) == nullptr || tr->getSplit() != 1 || tr->getFactor() != dh ||
+            !swapsFirstTwoOfThree(tr))
+            return nullptr;
+        Tensor *src = tr->getInputs()[0];
+        if (src->getDims() != Dim{seq, heads * dh})
+            return nullptr;
+        Operator *prod = src->getOutputOf();
+        return prod && rows.folded.count(prod) ? nullptr : src;
+    };
+    for (auto op : order) {
+        auto sm = dynamic_cast<SoftmaxOp *>(op);
+        if (!sm || skipped.count(op))
+            continue;
+        Tensor *scores = op->getInputs()[0], *scale = nullptr;
+        const Dim sd = scores->getDims();
+        if (sd.size() != 3 || sd[1] != sd[2] || sm->getAxis() != 2 || soleUser(scores) != op)
+            continue;
+        Operator *mulOp = nullptr;
+        if (scores->getOutputOf() && scores->getOutputOf()->getType() == Operator::Mul &&
+            scores->getOutputOf()->getInputs().size() == 2 && !skipped.count(scores->getOutputOf())) {
+            mulOp = scores->getOutputOf();
+            Tensor *a = mulOp->getInputs()[0], *b = mulOp->getInputs()[1];
+            if (b->size() == 1 && a->size() == scores->size())
+                scale = b, scores = a;
+            else if (a->size() == 1 && b->size() == scores->size())
+                scale = a, scores = b;
+            else
+                continue;
+            if (soleUser(scores) != mulOp)
+                continue;
+        }
+        MatmulOp *m1 = plainMatmul(scores->getOutputOf(), true);
+        Tensor *probs = op->getOutputs()[0];
+        MatmulOp *m2 = plainMatmul(soleUser(probs), false);
+        if (!m1 || !m2 || m2->getInputs()[0] != probs)
+            continue;
+        const int heads = sd[0], seq = sd[1];
+        Tensor *qh = m1->getInputs()[0], *kh = m1->getInputs()[1], *vh = m2->getInputs()[1];
+        if (qh->getDims().size() != 3 || qh == kh || qh == vh || kh == vh)
+            continue;
+        const int dh = qh->getDims()[2];
+        if (qh->getDims() != Dim{heads, seq, dh} || kh->getDims() != qh->getDims() ||
+            vh->getDims() != qh->getDims() || seq > 512 ||
+            (dh != 32 && dh != 64 && dh != 96 && dh != 128))
+            continue;
+        FusedAttention f;
+        f.q = headSplit(qh, heads, seq, dh);
+        f.k = headSplit(kh, heads, seq, dh);
+        f.v = headSplit(vh, heads, seq, dh);
+        Tensor *ctx = m2->getOutputs()[0];
+        auto merge = dynamic_cast<TransposeOp *>(soleUser(ctx));
+        if (!f.q || !f.k || !f.v || !merge || skipped.count(merge) || rows.folded.count(merge) ||
+            rows.chains.count(merge) || merge->getSplit() >= 0 || !swapsFirstTwoOfThree(merge))
+            continue;
+        f.scale = scale;
+        f.out = merge->getOutputs()[0];
+        f.heads = heads;
+        f.seq = seq;
+        f.dh = dh;
+        for (Tensor *t : {qh, kh, vh})
+            plan.absorbed.insert(t->getOutputOf());
+        plan.absorbed.insert(m1);
+        if (mulOp)
+            plan.absorbed.insert(mulOp);
+        plan.absorbed.insert(op);
+        plan.absorbed.insert(m2);
+        plan.atMerge[merge] = f;
+    }
+    return plan;
+}
+
+int launchAttention(const FusedAttention &f, pet_hip_stream_t s) {
+    const int ld = f.heads * f.dh;
+    return pet_hip_attention_f32(f.q->devicePtr(), f.k->devicePtr(), f.v->devicePtr(),
+                                 f.out->devicePtr(), 1, f.heads, f.seq, f.dh, ld, ld, ld, ld, 0, 0,
+                                 0, 0, 1.0f, f.scale ? f.scale->devicePtr() : nullptr, s);
+}
+
 // Micro-ops of a row of transposes, lowered on the first one's input.
 bool lowerChain(const std::vector<TransposeOp *> &row, TransProgram &prog) {
     std::vector<std::shared_ptr<TransBasic>> all;
@@ -454,13 +577,19 @@ std::unique_ptr<GraphExec> CodeEngine::instantiate(std::shared_ptr<SubGraph> &gr
                                       [](const FusedTail &f) {
                                           return f.residual->devicePtr() != f.out->devicePtr();
                                       }); // asked for tails with a residual only
-    LaunchPlan lp = planLaunchFlags(order, graph->getOutputs(), plan.skipped, rows.folded, tails,
+    FusedAttentions att = planAttention(order, graph->getOutputs(), plan.skipped, rows);
+    std::set<const Operator *> inert = rows.folded; // operators that do not launch by themselves
+    inert.insert(att.absorbed.begin(), att.absorbed.end());
+    LaunchPlan lp = planLaunchFlags(order, graph->getOutputs(), plan.skipped, inert, tails,
                                     [](const Tensor *) { return true; });
     auto flagsOf = [&](const Operator *op) {
         auto it = lp.flags.find(op);
         return it == lp.flags.end() ? 0u : it->second;
     };
     auto launchOp = [&](Operator *op, pet_hip_stream_t st) -> int {
+        auto fa = att.atMerge.find(op);
+        if (fa != att.atMerge.end())
+            return launchAttention(fa->second, st);
         auto tail = tails.atAdd.find(op);
         if (tail != tails.atAdd.end()) {
             const FusedTail &f = tail->second;
@@ -514,7 +643,7 @@ std::unique_ptr<GraphExec> CodeEngine::instantiate(std::shared_ptr<SubGraph> &gr
         }
         if (weightOnly(op))
             continue;
-        if (rows.folded.count(op) || tails.absorbed.count(op)) {
+        if (rows.folded.count(op) || tails.absorbed.count(op) || att.absorbed.count(op)) {
             exec->nFoldedOps++;
             continue;
         }
@@ -541,8 +670,8 @@ std::unique_ptr<GraphExec> CodeEngine::instantiate(std::shared_ptr<SubGraph> &gr
             auto tail = tails.atAdd.find(prod);
             if (tail != tails.atAdd.end() && tail->second.out != t)
                 inside = true;
-            if (inside || lp.preAct.count(t)) // not there, or there without its ReLU
-                continue;
+            if (inside || lp.preAct.count(t) || att.absorbed.count(prod))
+                continue; // not there, or there without its ReLU
             t->deviceWritten();
             t->setComputed();
         }
@@ -683,7 +812,10 @@ std::string CodeEngine::genCode(std::shared_ptr<SubGraph> &graph) {
     FusedTails tails = planFusedTails(order, graph->getOutputs(), skipped, [&](const FusedTail &f) {
         return !viewOf.count(f.residual) && !viewOf.count(f.out);
     });
-    LaunchPlan lp = planLaunchFlags(order, graph->getOutputs(), skipped, rows.folded, tails,
+    FusedAttentions att = planAttention(order, graph->getOutputs(), skipped, rows);
+    std::set<const Operator *> inert = rows.folded;
+    inert.insert(att.absorbed.begin(), att.absorbed.end());
+    LaunchPlan lp = planLaunchFlags(order, graph->getOutputs(), skipped, inert, tails,
                                     [](const Tensor *) { return true; });
     auto flagsOf = [&](const Operator *op) {
         auto it = lp.flags.find(op);
@@ -706,7 +838,14 @@ std::string CodeEngine::genCode(std::shared_ptr<SubGraph> &graph) {
             tail = nullptr;
             return ok;
         }
-        if (auto conv = dynamic_cast<ConvOp *>(op)) {
+        if (att.atMerge.count(op)) {
+            const FusedAttention &f = att.atMerge.at(op);
+            const int ld = f.heads * f.dh;
+            c << "pet_hip_attention_f32(" << e.name(f.q) << ", " << e.name(f.k) << ", "
+              << e.name(f.v) << ", " << e.name(f.out) << ", 1, " << f.heads << ", " << f.seq << ", "
+              << f.dh << ", " << ld << ", " << ld << ", " << ld << ", " << ld
+              << ", 0, 0, 0, 0, 1.0f, " << nullable(e, f.scale) << ", s)";
+        } else if (auto conv = dynamic_cast<ConvOp *>(op)) {
             auto d = op->getInputs()[0]->getDims(), w = op->getInputs()[1]->getDims();
             const unsigned fl = flagsOf(op) | PET_HIP_CONV_ALGO(conv->getAlgo());
             c << (fl     ? "pet_hip_conv2d_ex_f32("
@@ -960,7 +1099,7 @@ std::string CodeEngine::genCode(std::shared_ptr<SubGraph> &graph) {
     }
     for (auto op : order)
         if (!weightOnly(op) && !skipped.count(op) && !rows.folded.count(op) &&
-            !tails.absorbed.count(op) && !emitOp(op))
+            !tails.absorbed.count(op) && !att.absorbed.count(op) && !emitOp(op))
             return "";
     e.line("    pet_hip_graph_t g; CHECK(pet_hip_graph_end_capture(s, &g));");
     e.line("    pet_hip_event_t st, ed; CHECK(pet_hip_event_create(&st)); "

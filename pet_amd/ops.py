@@ -146,9 +146,15 @@ def conv3d(x, w, pad, stride=(1, 1, 1), dil=(1, 1, 1), bias=None, act="none", ou
 def matmul(A, B, transA=False, transB=False, bias=None, act="none", out=None, residual=None,
            flags=0):
     """MatmulOp on [b, ., .] tensors (MatmulOp::computeShape, operator.cc:717-726);
-    with residual: act(A @ B + bias + residual)."""
+    with residual: act(A @ B + bias + residual). flags: pet_hip_call_flags (abi.A_SHARED:
+    A is [1, ., .] and multiplies every batch entry of B; abi.BIAS_PER_BATCH: bias [b, n])."""
     _chk(A, B, bias, out, residual)
-    b = A.shape[0]
+    b = B.shape[0] if flags & abi.A_SHARED else A.shape[0]
+    if flags & abi.A_SHARED and A.shape[0] != 1:
+        raise abi.PetHipError(1, "a shared lhs has one batch entry")
+    if flags & abi.BIAS_PER_BATCH and (bias is None or bias.numel() != b * (
+            B.shape[1] if transB else B.shape[2])):
+        raise abi.PetHipError(1, "a per-batch bias holds b * n values")
     m = A.shape[2] if transA else A.shape[1]
     k = A.shape[1] if transA else A.shape[2]
     n = B.shape[1] if transB else B.shape[2]
@@ -218,6 +224,27 @@ def gbmml(A, B, dilation=1, out=None):
         out = torch.empty((bs, m, n), device=A.device, dtype=torch.float32)
     abi.call("pet_hip_gbmml_f32", _ptr(A), _ptr(B), _ptr(out), bs, m, (band - 1) // 2, n,
              dilation, _stream())
+    return out
+
+
+def attention(q, k, v, heads, scale=1.0, scale_dev=None, out=None):
+    """softmax(scale * Q_h K_h^T) V_h for every head, on [seq, heads*dh] (or [batch, seq,
+    heads*dh]) matrices; q, k, v may be row-strided views (slabs of a merged projection)."""
+    abi.init(torch.cuda.current_device())
+    for t in (q, k, v):
+        if not (t.is_cuda and t.dtype == torch.float32 and t.stride(-1) == 1):
+            raise ValueError("expected fp32 device matrices with contiguous rows")
+    q3, k3, v3 = (t if t.dim() == 3 else t.unsqueeze(0) for t in (q, k, v))
+    batch, seq, width = q3.shape
+    if width % heads or tuple(k3.shape) != tuple(q3.shape) or tuple(v3.shape) != tuple(q3.shape):
+        raise abi.PetHipError(1, "attention operands do not agree")
+    if out is None:
+        out = torch.empty(tuple(q.shape), device=q.device, dtype=torch.float32)
+    o3 = out if out.dim() == 3 else out.unsqueeze(0)
+    abi.call("pet_hip_attention_f32", _ptr(q3), _ptr(k3), _ptr(v3), _ptr(o3), batch, heads, seq,
+             width // heads, q3.stride(1), k3.stride(1), v3.stride(1), o3.stride(1),
+             q3.stride(0), k3.stride(0), v3.stride(0), o3.stride(0), float(scale),
+             _ptr(scale_dev), _stream())
     return out
 
 

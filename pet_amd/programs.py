@@ -67,7 +67,28 @@ class GpuNS:
         return self._k(self.ops.trans_chain(x, chain))
 
     def split(self, x, dim, sizes=None, num=None):
+        if dim == 0:
+            # slabs of the input buffer, no copy (the graph runtime's storage sharing,
+            # src/Graph/code_engine.cc:133-144)
+            szs = self.ops.split_sizes(x.shape[0], sizes, num)
+            offs = np.concatenate([[0], np.cumsum(szs)]).astype(int)
+            return [x[int(offs[i]):int(offs[i + 1])] for i in range(len(szs))]
         return self._k(self.ops.split(x, dim, sizes, num))
+
+    def matmul_shared_lhs(self, x, W, bias=None):
+        """Extend(x, dim 0) -> BatchMatmul(., W) -> per-slab bias Add, as one launch: the
+        lhs is read in place by every batch entry, bias is [b, n]."""
+        from . import abi
+        flags = abi.A_SHARED | (abi.BIAS_PER_BATCH if bias is not None else 0)
+        return self._k(self.ops.matmul(x, W, bias=bias, flags=flags))
+
+    def attention(self, q, k, v, heads, scale):
+        """Head split x 3 -> Matmul(transB) -> Mul(scale) -> Softmax -> Matmul -> head
+        merge, as one launch on the [1, seq, hidden] projections; scale: one-element tensor."""
+        seq, hidden = q.shape[-2], q.shape[-1]
+        out = self.ops.attention(q.reshape(seq, hidden), k.reshape(seq, hidden),
+                                 v.reshape(seq, hidden), heads, 1.0, scale_dev=scale)
+        return self._k(out).view(1, seq, hidden)
 
     def concat(self, xs, dim):
         return self._k(self.ops.concat(xs, dim))
@@ -283,32 +304,26 @@ def run_c4(ns, p, transformed=False, T=None):
     scale = T["scale"]
     x = T["x"]
 
-    def to_heads(t):  # [1, seq, hidden] -> [heads, seq, dh]
-        return ns.transpose(ns.reshape(t, (seq, hidden)), 1, [1, 0, -1], dh)
-
     for l in range(layers):
         pre = "L%d." % l
         if transformed:
             # PET batch-matmul merge (generator.cc:1495-1552): the three projections
             # become one b=3 BatchMatmul; the lhs is repeated along dim 0, the
             # weights are concatenated on dim 0, the result is split on dim 0.
-            xa = ns.extend(x, 0, 2)
+            # On this backend the Extend and the three bias Adds ride in the BatchMatmul's
+            # addressing and epilogue, and the Split is storage sharing.
             if pre + "qkv.w" not in T:
                 T[pre + "qkv.w"] = ns.concat([T[pre + "q.w"], T[pre + "k.w"], T[pre + "v.w"]], 0)
-            qkv = ns.matmul(xa, T[pre + "qkv.w"])
+                T[pre + "qkv.b"] = ns.concat([ns.reshape(T[pre + n], (1, hidden))
+                                              for n in ("q.b", "k.b", "v.b")], 0)
+            qkv = ns.matmul_shared_lhs(x, T[pre + "qkv.w"], T[pre + "qkv.b"])
             q, k, v = ns.split(qkv, 0, num=3)
-            q = ns.add([q, T[pre + "q.b"]])
-            k = ns.add([k, T[pre + "k.b"]])
-            v = ns.add([v, T[pre + "v.b"]])
         else:
             q = ns.matmul(x, T[pre + "q.w"], bias=T[pre + "q.b"])
             k = ns.matmul(x, T[pre + "k.w"], bias=T[pre + "k.b"])
             v = ns.matmul(x, T[pre + "v.w"], bias=T[pre + "v.b"])
-        qh, kh, vh = to_heads(q), to_heads(k), to_heads(v)
-        s = ns.matmul(qh, kh, transB=True)                 # [heads, seq, seq]
-        s = ns.softmax(ns.mul([s, scale]))
-        ctx = ns.matmul(s, vh)                             # [heads, seq, dh]
-        ctx = ns.reshape(ns.transpose(ctx, -1, [1, 0, 2]), (1, seq, hidden))
+        # head split, scores, scale, softmax, probabilities x values, head merge
+        ctx = ns.attention(q, k, v, heads, scale)          # [1, seq, hidden]
         att = ns.matmul(ctx, T[pre + "o.w"], bias=T[pre + "o.b"], residual=x)
         x = ns.layernorm(att, T[pre + "ln1.g"], T[pre + "ln1.b"])
         h = ns.matmul(x, T[pre + "f1.w"], bias=T[pre + "f1.b"], act="gelu")

@@ -38,6 +38,20 @@ class OracleNS:
     def matmul(self, A, B, transA=False, transB=False, bias=None, act="none", residual=None):
         return self._tail(self.o.matmul(A, B, transA, transB), bias, act, residual, ch_axis=2)
 
+    def matmul_shared_lhs(self, x, W, bias=None):
+        """Extend -> BatchMatmul -> Split -> bias Add per slab -> (slabs side by side)."""
+        y = self.o.matmul(self.o.extend(x, 0, W.shape[0] - 1), W)
+        if bias is not None:
+            y = np.stack([self.o.eltwise("add", [y[i], bias[i]], y[i].shape)
+                          for i in range(W.shape[0])])
+        return y
+
+    def attention(self, q, k, v, heads, scale):
+        seq, hidden = q.shape[-2], q.shape[-1]
+        out = self.o.attention(q.reshape(seq, hidden), k.reshape(seq, hidden),
+                               v.reshape(seq, hidden), heads, float(scale.reshape(-1)[0]))
+        return out.reshape(1, seq, hidden)
+
     def permute_flat(self, x, flat, perm):
         return self.o.permute_flat(x, flat, perm)
 

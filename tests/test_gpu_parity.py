@@ -885,3 +885,26 @@ def test_graph_capture_replays_match_eager(ops):
             st.synchronize()
             assert torch.equal(out, eager)
         abi.call("pet_hip_graph_destroy", g)
+
+
+@pytest.mark.parametrize("b,m,n,k,tb", [(3, 128, 768, 768, False), (3, 16, 24, 20, False),
+                                        (4, 33, 40, 64, True), (2, 8, 8, 96, False)])
+def test_matmul_shared_lhs_and_per_batch_bias(ops, b, m, n, k, tb):
+    """PET's matmul merge (src/Mutant/generator.cc:1495-1552) as this backend runs it: the
+    Extend of the lhs along dim 0 and the per-slab bias Adds are addressing modes of the
+    BatchMatmul. Against the operators one by one: Extend, Matmul, Add per slab."""
+    from pet_amd import abi
+    rng = np.random.default_rng(b * 7 + m + n + k)
+    a = ints(rng, (1, m, k))
+    w = ints(rng, (b, n, k) if tb else (b, k, n))
+    bias = ints(rng, (b, n))
+    want = oracle.matmul(oracle.extend(a, 0, b - 1), w, False, tb)
+    got = host(ops.matmul(dev(a), dev(w), False, tb, flags=abi.A_SHARED))
+    np.testing.assert_array_equal(got, want)
+    want_b = want + bias[:, None, :]
+    got = host(ops.matmul(dev(a), dev(w), False, tb, bias=dev(bias),
+                          flags=abi.A_SHARED | abi.BIAS_PER_BATCH))
+    np.testing.assert_array_equal(got, want_b)
+    full = ints(rng, (b, m, k))
+    got = host(ops.matmul(dev(full), dev(w), False, tb, bias=dev(bias), flags=abi.BIAS_PER_BATCH))
+    np.testing.assert_array_equal(got, oracle.matmul(full, w, False, tb) + bias[:, None, :])
