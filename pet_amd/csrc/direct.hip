@@ -6,7 +6,11 @@
 // neither. Here a wave owns a (32 TM) x (32 TN) output tile and a share of K, and feeds
 // v_mfma_f32_32x32x2_f32 straight from global memory:
 //  * A (filters, K contiguous): lane (l32, hk) holds row m0 + l32, k = hk * KH + j for
-//    MFMA step j, i.e. a contiguous run of the row, loaded as 16-byte words.
+//    MFMA step j, i.e. a contiguous run of the row. Loaded that way every lane of a load
+//    would touch a cache line of its own (rows are K floats apart), which made the L1 the
+//    limit of the whole kernel; so a wave reads its 32 x KC tile as consecutive 16-byte
+//    words (a row is KC/4 neighbouring lanes), parks it in a private LDS region and reads
+//    it back in operand order. No barrier: only the wave itself touches the region.
 //  * B (im2col): lane (l32, hk) holds pixel n0 + l32; one K chunk is CB channels times the
 //    whole r*s plane, the upper half-wave takes the upper CB/2 channels, so a tap's offset
 //    and padding status are fixed per lane (computed once, 0x80000000 for a padding tap:
@@ -35,9 +39,16 @@ struct DirectCfg {
     static constexpr int CH = CB / 2;           // channels per half-wave
     static constexpr int NQ = KH / 4;           // 16-byte words of A per row and chunk
     static constexpr int NT = 64 * KW;
+    static constexpr int PPR = KC / 4;          // 16-byte words per row of a chunk's A tile
+    static constexpr int A_LD = KC + 4;         // LDS row stride of the parked tile (floats)
     static constexpr int NREG = TM * TN * 16;
+    // LDS per wave: the parked A tile during the K loop, its partial tile afterwards
+    static constexpr int WAVE_LDS =
+        TM * 32 * A_LD > NREG * 64 ? TM * 32 * A_LD : NREG * 64;
     static constexpr int RPW = NREG / KW;       // accumulator registers a wave finishes
-    static_assert(KH % 4 == 0 && NREG % KW == 0 && RPW >= 1, "bad direct tile");
+    static_assert(KH % 4 == 0 && NREG % KW == 0 && RPW >= 1 && (32 * PPR) % 64 == 0 &&
+                      32 * PPR / 64 == NQ,
+                  "bad direct tile");
 };
 
 template <class Cfg>
@@ -45,7 +56,8 @@ __global__ __launch_bounds__(Cfg::NT) void conv_direct_kernel(ConvParams p) {
     extern __shared__ __attribute__((aligned(16))) float lds[];
     constexpr int TM = Cfg::TM, TN = Cfg::TN, KW = Cfg::KW, RS = Cfg::RS;
     constexpr int CB = Cfg::CB, KC = Cfg::KC, KH = Cfg::KH, CH = Cfg::CH;
-    constexpr int NREG = Cfg::NREG, RPW = Cfg::RPW;
+    constexpr int NREG = Cfg::NREG, RPW = Cfg::RPW, NQ = Cfg::NQ, PPR = Cfg::PPR;
+    constexpr int A_LD = Cfg::A_LD, WAVE_LDS = Cfg::WAVE_LDS;
     constexpr int SW = RS == 9 ? 3 : 1, SR = RS / SW;
 
     const int tid = threadIdx.x;
@@ -87,14 +99,23 @@ __global__ __launch_bounds__(Cfg::NT) void conv_direct_kernel(ConvParams p) {
     }
     const int padoff = p.ph * p.W + p.pw;
     const __amdgpu_buffer_rsrc_t rb = make_rsrc(p.x + (long long)g * p.cpg * HW - padoff);
-    // ---- and of the A rows
-    unsigned voffA[TM];
+    // ---- and of the A tile: word i = q * 64 + lane is row i / PPR, floats 4 * (i % PPR) ..
+    unsigned voffA[TM][NQ];
+    int parkA[NQ]; // where that word is parked in the wave's LDS region (floats)
 #pragma unroll
-    for (int tm = 0; tm < TM; ++tm)
-        voffA[tm] = ((unsigned)min(m0 + tm * 32 + l32, p.M - 1) * (unsigned)p.K + hk * KH) * 4u;
+    for (int q = 0; q < NQ; ++q) {
+        const int i = q * 64 + lane, row = i / PPR, pc = i - row * PPR;
+        parkA[q] = row * A_LD + pc * 4;
+#pragma unroll
+        for (int tm = 0; tm < TM; ++tm)
+            voffA[tm][q] =
+                ((unsigned)min(m0 + tm * 32 + row, p.M - 1) * (unsigned)p.K + pc * 4) * 4u;
+    }
+    float *ldsA = lds + wave * WAVE_LDS;
     const __amdgpu_buffer_rsrc_t ra = make_rsrc(p.w + (p.w_shared ? 0ll : (long long)g * p.M * p.K));
 
     float a[TM][KH], b[TN][KH];
+    uintx4 stage[TM][NQ];
     floatx16 acc[TM][TN];
 #pragma unroll
     for (int tm = 0; tm < TM; ++tm)
@@ -106,15 +127,34 @@ __global__ __launch_bounds__(Cfg::NT) void conv_direct_kernel(ConvParams p) {
     const float lo = p.x_relu ? 0.f : -INFINITY; // max(x, lo): ReLU left to this reader, or x
 
     auto load_a = [&](int q, int chunk) __attribute__((always_inline)) {
-        const unsigned so = (unsigned)(chunk * KC + 4 * q) * 4u;
+        const unsigned so = (unsigned)(chunk * KC) * 4u;
 #pragma unroll
-        for (int tm = 0; tm < TM; ++tm) {
-            uintx4 v = __builtin_amdgcn_raw_buffer_load_b128(ra, voffA[tm], so, 0);
-            a[tm][4 * q] = __uint_as_float(v.x);
-            a[tm][4 * q + 1] = __uint_as_float(v.y);
-            a[tm][4 * q + 2] = __uint_as_float(v.z);
-            a[tm][4 * q + 3] = __uint_as_float(v.w);
-        }
+        for (int tm = 0; tm < TM; ++tm)
+            stage[tm][q] = __builtin_amdgcn_raw_buffer_load_b128(ra, voffA[tm][q], so, 0);
+    };
+    // the staged tile through the wave's LDS region into operand order
+    auto park_a = [&]() __attribute__((always_inline)) {
+#pragma unroll
+        for (int tm = 0; tm < TM; ++tm)
+#pragma unroll
+            for (int q = 0; q < NQ; ++q)
+                *reinterpret_cast<uintx4 *>(ldsA + tm * 32 * A_LD + parkA[q]) = stage[tm][q];
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+#pragma unroll
+        for (int tm = 0; tm < TM; ++tm)
+#pragma unroll
+            for (int q = 0; q < NQ; ++q) {
+                const float4 v = *reinterpret_cast<const float4 *>(
+                    ldsA + (tm * 32 + l32) * A_LD + hk * KH + 4 * q);
+                a[tm][4 * q] = v.x;
+                a[tm][4 * q + 1] = v.y;
+                a[tm][4 * q + 2] = v.z;
+                a[tm][4 * q + 3] = v.w;
+            }
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
     };
     auto load_b = [&](int j, int chunk) __attribute__((always_inline)) {
         const int cj = j / RS, t = j % RS; // channel inside the half-chunk, tap
@@ -135,27 +175,30 @@ __global__ __launch_bounds__(Cfg::NT) void conv_direct_kernel(ConvParams p) {
 
     if (cb < ce) {
 #pragma unroll
-        for (int j = 0; j < KH; ++j) {
-            if (j % 4 == 0)
-                load_a(j / 4, cb);
+        for (int q = 0; q < NQ; ++q)
+            load_a(q, cb);
+#pragma unroll
+        for (int j = 0; j < KH; ++j)
             load_b(j, cb);
-        }
+        park_a();
         for (int chunk = cb; chunk + 1 < ce; ++chunk) {
+#pragma unroll
+            for (int q = 0; q < NQ; ++q)
+                load_a(q, chunk + 1);
 #pragma unroll
             for (int j = 0; j < KH; ++j) {
                 mfma_step(j);
-                // refill what this step (and, for A, the three before it) has just read
-                load_b(j, chunk + 1);
-                if (j % 4 == 3)
-                    load_a(j / 4, chunk + 1);
+                load_b(j, chunk + 1); // refill what this step has just read
             }
+            park_a();
         }
 #pragma unroll
         for (int j = 0; j < KH; ++j)
             mfma_step(j);
     }
 
-    // ---- the KW partial tiles meet in LDS: part[wave][register][lane]
+    // ---- the KW partial tiles meet in LDS: each wave's tile in its own region,
+    // [register][lane]
     if (KW > 1) {
 #pragma unroll
         for (int tm = 0; tm < TM; ++tm)
@@ -163,7 +206,7 @@ __global__ __launch_bounds__(Cfg::NT) void conv_direct_kernel(ConvParams p) {
             for (int tn = 0; tn < TN; ++tn)
 #pragma unroll
                 for (int r = 0; r < 16; ++r)
-                    lds[(wave * NREG + (tm * TN + tn) * 16 + r) * 64 + lane] = acc[tm][tn][r];
+                    lds[wave * WAVE_LDS + ((tm * TN + tn) * 16 + r) * 64 + lane] = acc[tm][tn][r];
         __syncthreads();
     }
     const float *__restrict__ bias = (p.bias && p.bias_mode == 1) ? p.bias + g * p.M : nullptr;
@@ -174,7 +217,7 @@ __global__ __launch_bounds__(Cfg::NT) void conv_direct_kernel(ConvParams p) {
         if (KW > 1) {
 #pragma unroll
             for (int w2 = 0; w2 < KW; ++w2)
-                v += lds[(w2 * NREG + reg) * 64 + lane];
+                v += lds[w2 * WAVE_LDS + reg * 64 + lane];
         } else {
             // KW == 1: the wave keeps its own registers (reg is a compile-time constant)
             v = acc[i / (TN * 16)][(i / 16) % TN][i % 16];
@@ -260,7 +303,7 @@ DirectChoice choose_direct(const ConvParams &p, int rs, bool allow_split) {
 template <int TM, int TN, int KW, int RS>
 int launch_direct_cfg(const ConvParams &p, dim3 grid, hipStream_t stream) {
     using Cfg = DirectCfg<TM, TN, KW, RS>;
-    const size_t lds_bytes = KW > 1 ? (size_t)KW * Cfg::NREG * 64 * sizeof(float) : 0;
+    const size_t lds_bytes = (size_t)KW * Cfg::WAVE_LDS * sizeof(float);
     static int attr_status = [&] {
         if (lds_bytes <= 64 * 1024)
             return 0;

@@ -266,11 +266,12 @@ LaunchPlan planLaunchFlags(const OpVec &order, const TensorVec &graphOutputs,
             effs.push_back({op, op->getOutputs()[0], ownAct(op), false});
     }
     for (auto &e : effs) {
-        // Not the ones with a residual: the library can add it along with the partial sums,
-        // but measured that loses more than the launch it saves (ResNet-18 0.252 -> 0.271 ms,
-        // BERT-base 1.45 -> 1.54 ms): the first K share of every tile then ends on a
-        // dependent load, and its atomics meet lines that were written long before.
-        if (e.hasRes || !ownStorage(e.out) || !e.c->accumulates())
+        // With a residual the library adds it along with the partial sums of the first K
+        // share. That pays for the small 2-D layers and matmuls (ResNet-18 0.197 -> 0.189 ms,
+        // BERT-base 1.009 -> 0.990 ms: one launch less per block), not for the 3-D layers,
+        // whose tiles then end on a dependent load (ResNet3D-18 1.058 -> 1.070 ms).
+        if ((e.hasRes && e.c->getType() == Operator::Conv3d) || !ownStorage(e.out) ||
+            !e.c->accumulates())
             continue;
         const Dim &d = e.out->getDims();
         FillSpec f{e.out, ownBias(e.c), 0, 0, 0};

@@ -636,9 +636,10 @@ static bool test_launch_fusion_block() {
     CodeEngine ce;
     auto exec = ce.instantiate(s2);
     EXPECT(exec != nullptr);
-    // c1 and c3 have no residual: their initialisations are batched; the four launches
-    // left are the four convolutions (both Adds and all ReLUs ride in them)
-    EXPECT(exec->numHoistedFills() == 2);
+    // the initialisations of all four are batched (c2 and c4 add their residual along with
+    // their partial sums); the four launches left are the four convolutions (both Adds and
+    // all ReLUs ride in them)
+    EXPECT(exec->numHoistedFills() == 4);
     EXPECT(exec->numKernelOps() == 4);
     Tensor *o1 = s1->getOutputs()[0], *o2 = s2->getOutputs()[0];
     EXPECT(s1->getOutputs().size() == 1 && s2->getOutputs().size() == 1);
@@ -656,10 +657,10 @@ static bool test_launch_fusion_block() {
         EXPECT(!negative && big > 1.0 && worst <= 1e-5 * big);
     }
     std::string code = ce.genCode(s2);
-    EXPECT(code.find("pet_hip_bias_fill_batch(fills, 2, s)") != std::string::npos);
-    // c1: initialised + ReLU deferred (3); c2's tail: reads with ReLU, defers its own (6);
-    // c3: initialised, reads with ReLU, defers (7); c4's tail: input and residual with ReLU (12)
-    for (const char *f : {", 3u, s)", ", 6u, s)", ", 7u, s)", ", 12u, s)"})
+    EXPECT(code.find("pet_hip_bias_fill_batch(fills, 4, s)") != std::string::npos);
+    // c1: initialised + ReLU deferred (3); c2's tail and c3: initialised, read with ReLU,
+    // defer their own (7); c4's tail: initialised, input and residual with ReLU (13)
+    for (const char *f : {", 3u, s)", ", 7u, s)", ", 13u, s)"})
         EXPECT(code.find(f) != std::string::npos);
     return true;
 }
