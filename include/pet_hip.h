@@ -326,6 +326,60 @@ PET_HIP_API int pet_hip_attention_f32(const float *q, const float *k, const floa
                           long long stride_o, float scale, const float *scale_dev,
                           pet_hip_stream_t stream);
 
+/* ---- memory-bound operators given as an index expression ------------------------------
+ * MemBoundOp::compute (src/Graph/operator.cc:3601-3644) evaluates, for every output
+ * position, an expression tree (include/nnet/expr.h) with nnet::Interpreter
+ * (src/nnet/Visitor/Interpreter.cc:31-131); the emitted program runs a TVM kernel printed
+ * from the same tree (src/Graph/code_engine.cc:1752-1798). Here the tree is flattened into a
+ * program of 32-bit integers for a small stack machine with an integer stack (index
+ * arithmetic), a value stack (fp32) and iterator slots:
+ *
+ *   header  PET_HIP_EXPR_MAGIC, ntensors, {rank, extents...} per tensor, out_rank, extents...
+ *   body    instructions, below; execution starts with the output position (outermost dim
+ *           first) on the integer stack and ends at END with one value, the output element.
+ *
+ * ICONST v | IVAR slot: push. IADD ISUB IMUL IDIV IMOD: pop b, a, push a op b (C integer
+ * division). LOAD t: pop rank(t) indices (last dim on top), push the element, 0 outside the
+ * tensor (TensorNode::getData, src/nnet/expr.cc:62-72). I2F: move the integer top to the value
+ * stack. FADD FSUB FMUL FDIV FMOD: value arithmetic (FDIV truncates, the reference's values
+ * being integers). FRELU FTANH: in place. RANGE nloop skip {slot left right pad}*: pop nloop
+ * positions into the slots; when one lies outside [left, right) push 0 and continue at word
+ * `skip` (a range read in its padding, Interpreter.cc:63-72). SUM nsum {slot lo hi}*: set the
+ * slots to lo, push an accumulator 0. SUMEND nsum body {slot lo hi}*: pop v, add it to the
+ * accumulator below, step the iterators (last fastest); back to word `body` until they wrap,
+ * then the accumulator is the value of the sum. Limits: 8 tensors, 32 slots, stacks 16 deep. */
+#define PET_HIP_EXPR_MAGIC 0x50455401
+typedef enum pet_hip_expr_op {
+    PET_HIP_EXPR_END = 0,
+    PET_HIP_EXPR_ICONST,
+    PET_HIP_EXPR_IVAR,
+    PET_HIP_EXPR_IADD,
+    PET_HIP_EXPR_ISUB,
+    PET_HIP_EXPR_IMUL,
+    PET_HIP_EXPR_IDIV,
+    PET_HIP_EXPR_IMOD,
+    PET_HIP_EXPR_LOAD,
+    PET_HIP_EXPR_I2F,
+    PET_HIP_EXPR_FADD,
+    PET_HIP_EXPR_FSUB,
+    PET_HIP_EXPR_FMUL,
+    PET_HIP_EXPR_FDIV,
+    PET_HIP_EXPR_FMOD,
+    PET_HIP_EXPR_FRELU,
+    PET_HIP_EXPR_FTANH,
+    PET_HIP_EXPR_RANGE,
+    PET_HIP_EXPR_SUM,
+    PET_HIP_EXPR_SUMEND
+} pet_hip_expr_op;
+/* Checks a program and keeps a copy of it in device memory (release it with pet_hip_free). */
+PET_HIP_API int pet_hip_expr_program_create(const int *code, int ncode, int **device_code);
+/* out[position] = program(position) for every position of the output shape in the header;
+ * inputs[t] is tensor t of the header, contiguous. device_code comes from
+ * pet_hip_expr_program_create for the same code. */
+PET_HIP_API int pet_hip_expr_f32(const int *code, int ncode, const int *device_code,
+                     const float *const *inputs, int ninputs, float *out,
+                     pet_hip_stream_t stream);
+
 /* ---- layout operators (bit-exact copies) ---------------------------------*/
 
 /* TransposeOp::compute after the split has been resolved to flat dims,

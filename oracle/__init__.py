@@ -501,3 +501,18 @@ def attention(q, k, v, heads, scale):
     s = eltwise("mul", [s, np.full((1,), scale, dtype=np.float32)], s.shape)
     ctx = matmul(softmax(s), to_heads(v))
     return transpose(ctx, -1, [1, 0, 2]).reshape(seq, width)
+
+
+def expr(code, inputs):
+    """MemBoundOp: evaluate the index-expression program `code` (a list of ints, the format of
+    include/pet_hip.h) at every position of the output shape in its header."""
+    code = [int(c) for c in code]
+    at = 2
+    for _ in range(code[1]):
+        at += 1 + code[at]
+    shape = tuple(code[at + 1:at + 1 + code[at]])
+    ins = [_c(np.asarray(a, dtype=np.float32)) for a in inputs]
+    out = np.empty(shape, dtype=np.float32)
+    ptrs = (ctypes.c_void_p * max(1, len(ins)))(*[a.ctypes.data for a in ins])
+    rc = lib().oracle_expr_f32(_ints(code), len(code), ptrs, _p(out))
+    return None if rc else out

@@ -275,3 +275,147 @@ PET_ORACLE_EXPORT void oracle_layernorm_f32(const float *x, const float *gamma,
                             (beta ? (double)beta[j] : 0.0));
     }
 }
+
+
+/* ---- MemBoundOp: an index expression evaluated at every output position ------------
+ * MemBoundOp::compute, src/Graph/operator.cc:3601-3644, runs nnet::Interpreter
+ * (src/nnet/Visitor/Interpreter.cc) on the operator's expression tree for every output
+ * position: Subscript of a tensor reads 0 outside the tensor (TensorNode::getData,
+ * src/nnet/expr.cc:62-72), a RangeOp reached through a Subscript in its padding is 0
+ * (Interpreter.cc:63-72), sum iterators run over [lo, hi) with the last one fastest
+ * (:85-105), BinaryOp is C integer arithmetic on indices (:31-50). The tree arrives here
+ * flattened into the integer program of include/pet_hip.h (same opcodes, copied below so
+ * that this file needs nothing of the library); values are fp32, sums accumulate in fp64.
+ * Pinned by numpy index maps (tests/test_oracle.py) and, where the reference tree is
+ * present, by nnet::Interpreter itself on trees the reference builds
+ * (tests/cpp/membound_driver.cc). Returns 0, or 1 for a malformed program. */
+enum {
+    EX_END, EX_ICONST, EX_IVAR, EX_IADD, EX_ISUB, EX_IMUL, EX_IDIV, EX_IMOD, EX_LOAD, EX_I2F,
+    EX_FADD, EX_FSUB, EX_FMUL, EX_FDIV, EX_FMOD, EX_FRELU, EX_FTANH, EX_RANGE, EX_SUM, EX_SUMEND
+};
+
+PET_ORACLE_EXPORT int oracle_expr_f32(const int *code, int ncode, const float *const *in,
+                                      float *out) {
+    if (ncode < 4 || code[0] != 0x50455401)
+        return 1;
+    int at = 1, nt = code[at++];
+    int nd[8], shape_at[8];
+    if (nt < 0 || nt > 8)
+        return 1;
+    for (int t = 0; t < nt; ++t) {
+        nd[t] = code[at++];
+        shape_at[t] = at;
+        at += nd[t];
+    }
+    const int out_nd = code[at++];
+    const int *out_shape = code + at;
+    at += out_nd;
+    size_t total = 1;
+    for (int d = 0; d < out_nd; ++d)
+        total *= (size_t)out_shape[d];
+    const int pc0 = at;
+    int failed = 0;
+#pragma omp parallel for
+    for (size_t i = 0; i < total; ++i) {
+        int istack[32], vars[32], isp = 0, fsp = 0;
+        double fstack[32];
+        size_t t = i;
+        int pos[8];
+        for (int j = out_nd - 1; j >= 0; --j) {
+            pos[j] = (int)(t % (size_t)out_shape[j]);
+            t /= (size_t)out_shape[j];
+        }
+        for (int j = 0; j < out_nd; ++j)
+            istack[isp++] = pos[j];
+        int pc = pc0;
+        while (pc < ncode && code[pc] != EX_END) {
+            const int op = code[pc];
+            if (op == EX_ICONST) {
+                istack[isp++] = code[pc + 1];
+                pc += 2;
+            } else if (op == EX_IVAR) {
+                istack[isp++] = vars[code[pc + 1]];
+                pc += 2;
+            } else if (op >= EX_IADD && op <= EX_IMOD) {
+                int b = istack[--isp], a = istack[--isp];
+                istack[isp++] = op == EX_IADD   ? a + b
+                                : op == EX_ISUB ? a - b
+                                : op == EX_IMUL ? a * b
+                                : op == EX_IDIV ? (b ? a / b : 0)
+                                                : (b ? a % b : 0);
+                pc += 1;
+            } else if (op == EX_LOAD) {
+                const int tn = code[pc + 1], n = nd[tn];
+                const int *shape = code + shape_at[tn];
+                isp -= n;
+                size_t off = 0;
+                int inside = 1;
+                for (int d = 0; d < n; ++d) {
+                    int idx = istack[isp + d];
+                    if (idx < 0 || idx >= shape[d])
+                        inside = 0;
+                    off = off * (size_t)shape[d] + (size_t)(idx < 0 ? 0 : idx);
+                }
+                fstack[fsp++] = inside ? (double)in[tn][off] : 0.0;
+                pc += 2;
+            } else if (op == EX_I2F) {
+                fstack[fsp++] = (double)istack[--isp];
+                pc += 1;
+            } else if (op >= EX_FADD && op <= EX_FMOD) {
+                double b = fstack[--fsp], a = fstack[--fsp];
+                fstack[fsp++] = op == EX_FADD   ? a + b
+                                : op == EX_FSUB ? a - b
+                                : op == EX_FMUL ? a * b
+                                : op == EX_FDIV ? trunc(a / b)
+                                                : fmod(a, b);
+                pc += 1;
+            } else if (op == EX_FRELU) {
+                if (fstack[fsp - 1] < 0)
+                    fstack[fsp - 1] = 0;
+                pc += 1;
+            } else if (op == EX_FTANH) {
+                fstack[fsp - 1] = tanh(fstack[fsp - 1]);
+                pc += 1;
+            } else if (op == EX_RANGE) {
+                const int n = code[pc + 1], skip = code[pc + 2];
+                isp -= n;
+                int inside = 1;
+                for (int d = 0; d < n; ++d) {
+                    const int *it = code + pc + 3 + 4 * d;
+                    vars[it[0]] = istack[isp + d];
+                    if (istack[isp + d] < it[1] || istack[isp + d] >= it[2])
+                        inside = 0;
+                }
+                if (inside) {
+                    pc += 3 + 4 * n;
+                } else {
+                    fstack[fsp++] = 0.0;
+                    pc = skip;
+                }
+            } else if (op == EX_SUM) {
+                const int n = code[pc + 1];
+                for (int d = 0; d < n; ++d)
+                    vars[code[pc + 2 + 3 * d]] = code[pc + 3 + 3 * d];
+                fstack[fsp++] = 0.0;
+                pc += 2 + 3 * n;
+            } else if (op == EX_SUMEND) {
+                const int n = code[pc + 1], body = code[pc + 2];
+                double v = fstack[--fsp];
+                fstack[fsp - 1] += v;
+                int d = n - 1;
+                for (; d >= 0; --d) {
+                    const int *it = code + pc + 3 + 3 * d;
+                    if (++vars[it[0]] < it[2])
+                        break;
+                    vars[it[0]] = it[1];
+                }
+                pc = d >= 0 ? body : pc + 3 + 3 * n;
+            } else {
+                failed = 1;
+                break;
+            }
+        }
+        out[i] = fsp > 0 ? (float)fstack[fsp - 1] : 0.f;
+    }
+    return failed;
+}

@@ -74,6 +74,8 @@ SIGNATURES = {
     "pet_hip_g2bmm_f32": [_vp] * 3 + [_i] * 5 + [_vp],
     "pet_hip_gbmml_f32": [_vp] * 3 + [_i] * 5 + [_vp],
     "pet_hip_attention_f32": [_vp] * 4 + [_i] * 8 + [ctypes.c_longlong] * 4 + [ctypes.c_float, _vp, _vp],
+    "pet_hip_expr_program_create": [_c_int_p, _i, ctypes.POINTER(_vp)],
+    "pet_hip_expr_f32": [_c_int_p, _i, _vp, ctypes.POINTER(_vp), _i, _vp, _vp],
     "pet_hip_transpose": [_vp, _vp, _c_int_p, _c_int_p, _i, _vp],
     "pet_hip_trans_chain": [_vp, _vp, _c_int_p, _i, _c_int_p, _i, _c_int_p, _c_int_p, _c_int_p, _vp],
     "pet_hip_split": [_vp, ctypes.POINTER(_vp), _i, _c_int_p, _i, _i, _c_int_p, _vp],

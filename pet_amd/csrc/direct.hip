@@ -56,7 +56,7 @@ __global__ __launch_bounds__(Cfg::NT) void conv_direct_kernel(ConvParams p) {
     extern __shared__ __attribute__((aligned(16))) float lds[];
     constexpr int TM = Cfg::TM, TN = Cfg::TN, KW = Cfg::KW, RS = Cfg::RS;
     constexpr int CB = Cfg::CB, KC = Cfg::KC, KH = Cfg::KH, CH = Cfg::CH;
-    constexpr int NREG = Cfg::NREG, RPW = Cfg::RPW, NQ = Cfg::NQ, PPR = Cfg::PPR;
+    constexpr int RPW = Cfg::RPW, NQ = Cfg::NQ, PPR = Cfg::PPR;
     constexpr int A_LD = Cfg::A_LD, WAVE_LDS = Cfg::WAVE_LDS;
     constexpr int SW = RS == 9 ? 3 : 1, SR = RS / SW;
 

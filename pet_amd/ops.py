@@ -248,6 +248,37 @@ def attention(q, k, v, heads, scale=1.0, scale_dev=None, out=None):
     return out
 
 
+class ExprProgram:
+    """An index-expression program (see pet_hip.h) with its device copy."""
+
+    def __init__(self, code):
+        abi.init(torch.cuda.current_device())
+        self.code = abi.ints(code)
+        self.ncode = len(code)
+        dev = ctypes.c_void_p(0)
+        abi.call("pet_hip_expr_program_create", self.code, self.ncode, ctypes.byref(dev))
+        self.dev = dev
+        at = 2
+        for _ in range(code[1]):
+            at += 1 + code[at]
+        self.out_shape = tuple(code[at + 1:at + 1 + code[at]])
+
+    def __del__(self):
+        if getattr(self, "dev", None) is not None and self.dev.value:
+            abi.status("pet_hip_free", self.dev)
+
+
+def expr(program, inputs, out=None):
+    """MemBoundOp: out[pos] = program(pos) over the output shape in the program's header."""
+    _chk(out, *inputs)
+    if out is None:
+        out = torch.empty(program.out_shape, device=inputs[0].device, dtype=torch.float32)
+    ptrs = (ctypes.c_void_p * max(1, len(inputs)))(*[t.data_ptr() for t in inputs])
+    abi.call("pet_hip_expr_f32", program.code, program.ncode, program.dev, ptrs, len(inputs),
+             _ptr(out), _stream())
+    return out
+
+
 def transpose_params(in_dims, split, after, factor):
     """TransposeOp::setParam (include/operator.h:1124-1144) and the flat-dim
     rule of TransposeOp::computeShape (src/Graph/operator.cc:2340-2381).

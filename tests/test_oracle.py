@@ -583,3 +583,52 @@ def test_g2bmm_gbmml_vs_dense_numpy(bs, m, k, w, d):
     Au, Bu = np.abs(A).astype(np.uint32), np.abs(B).astype(np.uint32)
     np.testing.assert_array_equal(oracle.g2bmm(Au, Bu, w, d),
                                   _band_dense(np.abs(A), np.abs(B), w, d).astype(np.uint32))
+
+
+# ---- MemBound expressions -----------------------------------------------------------------
+
+def _membound_cases(rng):
+    """(tensor shapes, top range, inputs, expected) with the expected values from numpy."""
+    from expr_programs import C, I, R, RS, T, relu, tanh
+    cases = []
+    a = rng.integers(-3, 4, (4, 6)).astype(np.float32)
+    cases.append(("transpose", [(4, 6)], R([("i", 0, 6), ("j", 0, 4)], [], T(0, [I("j"), I("i")])),
+                  [a], a.T))
+    x = rng.integers(-3, 4, (2, 3, 6, 5)).astype(np.float32)
+    k = rng.integers(-3, 4, (4, 3, 3, 3)).astype(np.float32)
+    conv = R([("n", 0, 2), ("f", 0, 4), ("h", 0, 6), ("w", 0, 5)],
+             [("c", 0, 3), ("r", 0, 3), ("s", 0, 3)],
+             T(0, [I("n"), I("c"), I("h") + I("r") - 1, I("w") + I("s") - 1]) *
+             T(1, [I("f"), I("c"), I("r"), I("s")]))
+    cases.append(("conv as a sum over padded reads", [x.shape, k.shape], conv, [x, k],
+                  oracle.conv2d(x, k, 1, 1)))
+    # space-to-batch written with division and remainder: out[b, c, h, w] = x[0, c, 2h + b/2, 2w + b%2]
+    y = rng.integers(-3, 4, (1, 3, 8, 8)).astype(np.float32)
+    s2b = R([("b", 0, 4), ("c", 0, 3), ("h", 0, 4), ("w", 0, 4)], [],
+            T(0, [C(0), I("c"), I("h") * 2 + I("b") // 2, I("w") * 2 + I("b") % 2]))
+    want = y.reshape(3, 4, 2, 4, 2).transpose(2, 4, 0, 1, 3).reshape(4, 3, 4, 4)
+    cases.append(("space to batch", [y.shape], s2b, [y], want))
+    # a range read through a subscript, in and out of its padding, with ReLU inside and a
+    # value-level sum outside
+    v = rng.integers(-3, 4, (8,)).astype(np.float32)
+    inner = R([("p", 0, 8)], [], relu(T(0, [I("p")])), pads=[2])
+    outer = R([("i", 0, 12)], [], RS(inner, [I("i") - 2]) + T(0, [I("i")]))
+    cases.append(("nested range with padding", [(8,)], outer, [v],
+                  np.pad(np.maximum(v, 0), 2) + np.pad(v, (0, 4))))
+    # two stages: t[i] = sum_j m[i, j]; out[i] = tanh(t[i]) * i
+    m = rng.standard_normal((5, 7)).astype(np.float32)
+    stage = R([("i", 0, 5)], [("j", 0, 7)], T(0, [I("i"), I("j")]))
+    top = R([("i", 0, 5)], [], tanh(RS(stage, [I("i")])) * I("i"))
+    cases.append(("two stages, value times index", [(5, 7)], top, [m],
+                  np.tanh(m.astype(np.float64).sum(1)) * np.arange(5)))
+    return cases
+
+
+def test_membound_expression_interpreter_vs_numpy():
+    """MemBoundOp::compute (src/Graph/operator.cc:3601-3644 over nnet::Interpreter): the
+    restated interpreter against index maps written in numpy."""
+    from expr_programs import assemble
+    for name, shapes, top, inputs, want in _membound_cases(np.random.default_rng(9)):
+        got = oracle.expr(assemble(shapes, top), inputs)
+        assert got is not None and got.shape == want.shape, name
+        np.testing.assert_allclose(got, want, rtol=1e-6, atol=1e-6, err_msg=name)
