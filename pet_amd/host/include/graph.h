@@ -38,6 +38,11 @@ class GraphBase {
     void removeOps(OpVec &removed);
     // Operators in a topological order (Kahn, ties in insertion order).
     bool topoOrder(OpVec &order) const;
+    // The reference reads and writes model files through its embedded Python plug-in
+    // (src/Graph/graph.cc:1172-1187); this backend's file front end is
+    // pet_amd/onnx_import.py, so both report failure here.
+    bool exportOnnx(const char *path);
+    bool importOnnx(const char *net);
 };
 
 class Graph : public GraphBase {
@@ -125,8 +130,20 @@ class Graph : public GraphBase {
 
     void setInputs(TensorVec v) { inputs = std::move(v); }
     void setOutputs(TensorVec v) { outputs = std::move(v); }
+#ifdef PET_HAVE_NNET
+    // A memory-bound operator given by an expression of the reference's nnet tree
+    // (include/graph.h:176-180, src/Graph/graph.cc:603-613); only where that tree's
+    // headers are on the include path.
+    Operator *membound(const TensorVec &inputs, const TensorVec &outputs,
+                       const std::vector<nnet::Tensor> &nnetInputs, nnet::Expr expr,
+                       double exec_time, std::string hint = {}) {
+        // 0.001 ms for the launch, as upstream
+        double t = exec_time == 0 ? 0 : std::max(exec_time, 0.001);
+        return own(new MemBoundOp(inputs, outputs, nnetInputs, expr, t, hint));
+    }
+#endif
 
-  private:
+    // Takes ownership of an operator built elsewhere (and of the outputs it created).
     Operator *own(Operator *op);
 };
 
@@ -160,9 +177,23 @@ class SubGraph : public GraphBase {
     // Sum of op->perf() over the operators, in ms.
     double perf(PerfEngine *pe, bool withPenalty = true);
     uint64_t getHash();
+    // Key of the search engine's mutation archive: operator types, at level 1 also the
+    // extents of their inputs (src/Graph/graph.cc:901-924).
+    uint64_t getCacheIdx(int level);
     int print();
+    int printBrief();
     int getComputeOps(OpVec &out);
     void resetComputed();
+    // Gives the graph's inputs and outputs the identity (hash) of the given tensors, so
+    // that a mutant can take the place of the subgraph it was derived from.
+    int reset(std::vector<Tensor *> &input, std::vector<Tensor *> &output);
+    // The operators of `ops` as `slave`, all others as `master` (both cloned).
+    int split(std::shared_ptr<SubGraph> &master, std::shared_ptr<SubGraph> &slave,
+              std::vector<Operator *> &ops);
+    // This graph's operators plus the slave's, the slave's tensors replaced by this
+    // graph's where their hashes agree.
+    int merge(std::shared_ptr<SubGraph> &master, std::shared_ptr<SubGraph> &slave);
 };
 
 } // namespace tpm
+

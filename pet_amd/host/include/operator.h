@@ -9,6 +9,14 @@
 #include "tensor.h"
 #include "transpose.h"
 #include <sstream>
+// MemBoundOp is defined over the expression tree of the reference's search side
+// (include/nnet/expr.h). That tree is not part of this backend: where its headers are on
+// the include path (builds of the reference's mutators and search engine against this
+// directory) the class exists, elsewhere nothing here depends on it.
+#if __has_include("nnet/expr.h")
+#define PET_HAVE_NNET 1
+#include "nnet/expr.h"
+#endif
 
 namespace tpm {
 
@@ -152,6 +160,16 @@ class Operator {
     // buffers (used by compute(), by perf() and by the graph runtime).
     // Returns a pet_hip_status.
     virtual int launch(pet_hip_stream_t stream) = 0;
+    // For operators the emitter has no case of its own for: the C-ABI call that launches
+    // the operator on stream `s` in an emitted program, `name` giving a tensor's variable
+    // and `setup` taking lines that must precede the captured region. Empty: cannot be
+    // emitted.
+    virtual std::string emitLaunch(const std::function<std::string(const Tensor *)> &name,
+                                   std::vector<std::string> &setup) const {
+        (void)name;
+        (void)setup;
+        return "";
+    }
 
   protected:
     virtual bool checkValid(const TensorVec &inputs) = 0;
@@ -978,3 +996,7 @@ class IdentityOp : public ReshapeOp {
 };
 
 } // namespace tpm
+
+#ifdef PET_HAVE_NNET
+#include "membound.h"
+#endif

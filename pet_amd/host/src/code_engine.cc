@@ -1054,13 +1054,24 @@ std::string CodeEngine::genCode(std::shared_ptr<SubGraph> &graph) {
             c << "pet_hip_memcpy_d2d(" << out(0) << ", " << in(0) << ", "
               << op->getInputs()[0]->size() << " * sizeof(float), s)";
         } else {
-            return false;
+            std::vector<std::string> setup;
+            std::string call =
+                op->emitLaunch([&](const Tensor *t) { return e.name(t); }, setup);
+            if (call.empty())
+                return false;
+            c << call; // its set-up lines were written before the first launch
         }
         e.line("    CHECK(" + c.str() + "); // " + op->toString());
         return true;
     };
 
     e.line("    int odims[PET_HIP_MAX_RANK], orank = 0; (void)odims; (void)orank;");
+    for (auto op : order) { // what such operators need before their first launch
+        std::vector<std::string> setup;
+        op->emitLaunch([&](const Tensor *t) { return e.name(t); }, setup);
+        for (auto &l : setup)
+            e.line("    " + l);
+    }
     e.line("    // operators that only touch weights run once");
     for (auto op : order)
         if (weightOnly(op) && !skipped.count(op) && !rows.folded.count(op) &&

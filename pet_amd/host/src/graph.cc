@@ -3,6 +3,7 @@
 #include "perf_engine.h"
 
 #include <algorithm>
+#include <set>
 #include <functional>
 #include <unordered_map>
 
@@ -403,7 +404,16 @@ int SubGraph::findTensor(Tensor *tensor, int ntensor) {
 bool SubGraph::resetOps(OpVec oplist, size_t ntensor) {
     ntensor = ntensor == 0 ? tensors.size() : std::min(ntensor, tensors.size());
     hash = 2147483647;
-    cleanConnection();
+    // The operators of the previous list are borrowed and may be gone by now (the mutation
+    // generator deletes its candidate operators at the start of every run,
+    // src/Mutant/generator.cc:84-87, while its scratch graph still lists them): only the
+    // graph's own tensors are reset here, and the operators of the new list below.
+    for (auto t : tensors) {
+        t->setOutputOf(nullptr);
+        t->setInputOf({});
+    }
+    inputs.clear();
+    outputs.clear();
     ops = std::move(oplist);
     for (auto op : ops) {
         op->setPredecessors({});
@@ -529,6 +539,110 @@ int SubGraph::getComputeOps(OpVec &out) {
         if (op->isComputeOp())
             out.push_back(op);
     return (int)out.size();
+}
+
+} // namespace tpm
+
+namespace tpm {
+
+bool GraphBase::exportOnnx(const char *path) {
+    std::fprintf(stderr, "[pet] exportOnnx(%s): model files are written by the Python side of "
+                         "this backend, not by the host layer\n", path ? path : "");
+    return false;
+}
+
+bool GraphBase::importOnnx(const char *net) {
+    std::fprintf(stderr, "[pet] importOnnx(%s): use pet_amd.onnx_import.load, which builds the "
+                         "graph through the Python module\n", net ? net : "");
+    return false;
+}
+
+uint64_t SubGraph::getCacheIdx(int level) {
+    static const uint64_t factors[8] = {10000019, 10000079, 10000103, 10000121,
+                                        10000139, 10000141, 10000169, 10000189};
+    uint64_t h = 0;
+    for (auto op : ops) {
+        h = hashAppend(h, std::hash<uint64_t>()(op->getType()));
+        if (level != 1)
+            continue;
+        size_t l = 0;
+        for (auto in : op->getInputs()) {
+            uint64_t th = 0;
+            for (int d : in->getDims())
+                th = hashAppend(th, (uint64_t)d * factors[l++ % 8]);
+            h = hashAppend(h, th);
+        }
+    }
+    return h;
+}
+
+int SubGraph::printBrief() {
+    std::cout << "Subgraph[" << getHash() << "] brief\n    op num: " << ops.size()
+              << "\n    input: ";
+    for (auto t : inputs)
+        std::cout << t->getHash() << " ";
+    std::cout << "\n    output: ";
+    for (auto t : outputs)
+        if (t->isNotCounted())
+            std::cout << "(" << t->getHash() << ") ";
+        else
+            std::cout << t->getHash() << " ";
+    std::cout << std::endl;
+    return 0;
+}
+
+int SubGraph::reset(std::vector<Tensor *> &input, std::vector<Tensor *> &output) {
+    for (auto t : tensors)
+        t->refresh();
+    if (inputs.size() != input.size() || outputs.size() != output.size())
+        return 1;
+    for (size_t i = 0; i < input.size(); ++i)
+        inputs[i]->replace(*input[i]);
+    for (size_t i = 0; i < output.size(); ++i)
+        outputs[i]->replace(*output[i]);
+    return 0;
+}
+
+int SubGraph::split(std::shared_ptr<SubGraph> &master, std::shared_ptr<SubGraph> &slave,
+                    std::vector<Operator *> &slaveOps) {
+    std::set<Operator *> mine(ops.begin(), ops.end()), taken;
+    for (auto op : slaveOps) {
+        if (!mine.count(op)) {
+            std::cout << "ERROR: [SubGraph::split] slave op not in subgraph." << std::endl;
+            return 1;
+        }
+        taken.insert(op);
+    }
+    OpVec rest;
+    for (auto op : ops)
+        if (!taken.count(op))
+            rest.push_back(op);
+    master = std::make_shared<SubGraph>(rest);
+    slave = std::make_shared<SubGraph>(slaveOps);
+    return 0;
+}
+
+int SubGraph::merge(std::shared_ptr<SubGraph> &master, std::shared_ptr<SubGraph> &slave) {
+    std::unordered_map<uint64_t, Tensor *> byHash;
+    for (auto t : tensors)
+        byHash.emplace(t->getHash(), t);
+    OpVec all(ops.begin(), ops.end());
+    auto mine = [&](Tensor *t) {
+        auto it = byHash.find(t->getHash());
+        return it == byHash.end() ? t : it->second;
+    };
+    for (auto op : slave->getOperators()) {
+        TensorVec ins, outs;
+        for (auto t : op->getInputs())
+            ins.push_back(mine(t));
+        for (auto t : op->getOutputs())
+            outs.push_back(mine(t));
+        op->setInputs(ins);
+        op->setOutputs(outs);
+        all.push_back(op);
+    }
+    master = std::make_shared<SubGraph>(all);
+    return 0;
 }
 
 } // namespace tpm

@@ -316,6 +316,51 @@ def test_generator_candidates_run_and_are_ranked_on_the_device(args):
     assert res.returncode == 0
 
 
+SEARCH_DRIVER = os.path.join(LIB, "pet_search_driver")
+MEMBOUND_DRIVER = os.path.join(LIB, "pet_membound_driver")
+
+
+@pytest.mark.gpu
+@needs_refsearch
+@pytest.mark.parametrize("args", [
+    "1 64 56 56 64 3 1 1",         # benchmark configuration 1
+    "1 512 64 64 512 3 2 2",       # the 512 -> 512 layer of the dilated block
+])
+def test_reference_search_engine_runs_on_the_device(args):
+    """The reference's SearchEngine::run (src/Graph/search_engine.cc:54-118), compiled
+    unchanged with its mutation generator: candidates are ranked by Operator::perf on the
+    MI355X; the graph it returns costs no more than the input graph, its getPerf total is
+    SubGraph::perf, and it computes what the input graph computes."""
+    import re
+    assert os.path.exists(SEARCH_DRIVER), \
+        "run __graft_entry__.build() where the reference tree is present"
+    res = subprocess.run([SEARCH_DRIVER] + args.split(), capture_output=True, text=True,
+                         timeout=900)
+    print(res.stdout[-6000:])
+    print(res.stderr[-3000:])
+    assert res.returncode == 0
+    origin = re.findall(r"Origin Perf: ([0-9.eE+-]+)", res.stdout)
+    best = re.findall(r"Best Perf without correction: ([0-9.eE+-]+)", res.stdout)
+    assert origin and best and float(best[-1]) <= float(origin[0]) * 1.0001
+    assert "PET graph getPerf" in res.stdout and " op_time " in res.stdout   # the profile table
+    assert "driver: ok" in res.stdout
+
+
+@pytest.mark.gpu
+@needs_refsearch
+def test_membound_operator_agrees_with_the_reference_interpreter():
+    """MemBoundOp on the device against nnet::Interpreter (the reference's own evaluation,
+    compiled unchanged) on expressions the reference's pattern builders produce:
+    convolution, matmul, the band products, transposed convolution, layout moves."""
+    assert os.path.exists(MEMBOUND_DRIVER), \
+        "run __graft_entry__.build() where the reference tree is present"
+    res = subprocess.run([MEMBOUND_DRIVER], capture_output=True, text=True, timeout=300)
+    print(res.stdout[-4000:])
+    print(res.stderr[-2000:])
+    assert res.returncode == 0
+    assert res.stdout.count("[  OK  ]") >= 8 and "0 failed" in res.stdout
+
+
 # ---- the benchmark networks through Graph -> SubGraph -> CodeEngine ---------------
 RUN_MODEL = os.path.join(LIB, "pet_run_model")
 
