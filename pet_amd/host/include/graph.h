@@ -139,7 +139,9 @@ class Graph : public GraphBase {
                        double exec_time, std::string hint = {}) {
         // 0.001 ms for the launch, as upstream
         double t = exec_time == 0 ? 0 : std::max(exec_time, 0.001);
-        return own(new MemBoundOp(inputs, outputs, nnetInputs, expr, t, hint));
+        // the outputs are the caller's tensors (often another graph's): not adopted
+        ops.push_back(new MemBoundOp(inputs, outputs, nnetInputs, expr, t, hint));
+        return ops.back();
     }
 #endif
 

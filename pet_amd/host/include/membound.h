@@ -248,9 +248,16 @@ class MemBoundOp : public Operator {
     // 2051-2053); here the operator is launched and timed like every other one, so that the
     // search ranks by measured cost. Operators that only touch weights cost nothing, as
     // upstream: they run once, ahead of inference.
-    double perf(PerfEngine *, int rounds = 200, int warmupRounds = 200) override {
+    double perf(PerfEngine *pe, int rounds = 200, int warmupRounds = 200) override {
         if (isComputeWeight())
             return 0;
+        if (!expr) {
+            // A placeholder the reference's transforms leave for a layout move they only
+            // price (src/nnet/nmutator.cc:529-567: no expression, a time from the bytes moved
+            // at 200 GiB/s): the same bytes at this GPU's measured copy bandwidth.
+            const double bw = pe ? pe->layoutBandwidthGiBs() : 0.0;
+            return bw > 0 ? exec_time * 200.0 / bw : exec_time;
+        }
         if (measured < 0) {
             for (auto t : outputs)
                 if (t->devicePtr() == nullptr)

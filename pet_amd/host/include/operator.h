@@ -998,5 +998,6 @@ class IdentityOp : public ReshapeOp {
 } // namespace tpm
 
 #ifdef PET_HAVE_NNET
+#include "perf_engine.h"
 #include "membound.h"
 #endif

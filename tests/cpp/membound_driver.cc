@@ -9,10 +9,12 @@
 #include "nnet/Visitor/Interpreter.h"
 #include "nnet/expr.h"
 #include "nnet/iterator_table.h"
+#include "nnet/nmutator.h"
 #include "operator.h"
 
 #include <cstdio>
 #include <cstdlib>
+#include <map>
 
 using namespace tpm;
 
@@ -88,6 +90,42 @@ static void check(const char *name, nnet::Expr expr, const std::vector<nnet::Ten
     }
 }
 
+// The reference's own conversion of an operator into a MemBound operator
+    // (NMutator::runSingleOpToNaiveMembound, src/nnet/nmutator.cc:42-58): the
+    // convolution and the MemBound operator that states it must agree on the device
+static void naiveMemboundOfAConvolution() {
+    Graph g;
+    Tensor *x = g.tensor({2, 4, 6, 6}), *k = g.tensor({8, 4, 3, 3});
+    g.conv(x, k, 1, 1);
+    g.updateConnection();
+    SubGraph in(g.getOperators());
+    int seed = 5;
+    for (auto t : in.getInputs())
+        t->dataRand(seed++);
+    NMutator mutator;
+    mutator.setToNaiveMembound();
+    std::vector<SubGraph *> outs;
+    mutator.run(&in, outs);
+    bool ok = outs.size() == 1 && outs[0]->getOperators().size() == 1 &&
+              outs[0]->getOperators()[0]->getType() == Operator::MemBound;
+    if (ok) {
+        std::map<uint64_t, Tensor *> byHash;
+        for (auto t : in.getInputs())
+            byHash[t->getHash()] = t;
+        for (auto t : outs[0]->getInputs())
+            t->setData(byHash.at(t->getHash())->getDataPtr());
+        ok = in.compute() && outs[0]->compute();
+        const Tensor *a = in.getOutputs()[0], *b = outs[0]->getOutputs()[0];
+        ok = ok && a->size() == b->size();
+        for (size_t i = 0; ok && i < a->size(); ++i)
+            ok = const_cast<Tensor *>(a)->getDataPtr()[i] ==
+                 const_cast<Tensor *>(b)->getDataPtr()[i];
+    }
+    std::printf("[ %s ] NMutator naive MemBound of a convolution equals the convolution\n",
+                ok ? " OK " : "FAIL");
+    failures += !ok;
+}
+
 #define VAR(name) auto name = nnet::make_ref<nnet::VarNode>(#name)
 
 int main() {
@@ -130,6 +168,7 @@ int main() {
         check("conv transpose 4x4 / 2", ConvTransPattern::getExpr(A, K, N, C, H, W, F, R, S),
               {A, K});
     }
+    naiveMemboundOfAConvolution();
     std::printf("%d failed\n", failures);
     std::fflush(stdout);
     std::_Exit(failures ? 1 : 0);

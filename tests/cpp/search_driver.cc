@@ -3,7 +3,12 @@
 // SearchEngine::run on one convolution, every candidate ranked by Operator::perf on the
 // MI355X, then the chosen program is executed next to the original and compared.
 //
-//   pet_search_driver n c h w f r pad dilation
+//   pet_search_driver n c h w f r pad dilation [nnet]
+//
+// With "nnet" the mutation engine is the reference's NMutator (src/nnet/nmutator.cc)
+// instead of its Generator. Its transforms leave MemBound placeholders without an
+// expression for layout moves they only price; a best graph that holds one is costed but
+// cannot be executed, and the comparison of outputs is left out for it.
 //
 // Prints what SearchEngine::run prints (its getPerf profile tables among it), the cost of
 // the original and of bestGraph through SearchEngine::getPerf, and the agreement of the two
@@ -12,6 +17,7 @@
 // computes what the original computes.
 #include "generator.h"
 #include "graph.h"
+#include "nnet/nmutator.h"
 #include "operator.h"
 #include "perf_engine.h"
 #include "search_engine.h"
@@ -24,6 +30,7 @@
 #include <unistd.h>
 #include <cstdlib>
 #include <map>
+#include <string>
 
 using namespace tpm;
 
@@ -53,8 +60,13 @@ int main(int argc, char **argv) {
     g->updateConnection();
     auto graph = std::make_shared<SubGraph>(g->getOperators());
 
-    auto generator = std::make_shared<Generator>();
-    SearchEngine engine(std::static_pointer_cast<Mutator>(generator));
+    const bool useNnet = argc > 9 && std::string(argv[9]) == "nnet";
+    std::shared_ptr<Mutator> mutator;
+    if (useNnet)
+        mutator = std::make_shared<NMutator>();
+    else
+        mutator = std::make_shared<Generator>();
+    SearchEngine engine(mutator);
     std::shared_ptr<SubGraph> best;
     int err = engine.run(graph, best);
     std::fflush(stdout);
@@ -77,6 +89,16 @@ int main(int argc, char **argv) {
     ok = ok && std::isfinite(viaGraph) && viaGraph > 0 &&
          std::fabs(viaGraph - chosen) <= 0.5 * std::max(viaGraph, chosen);
 
+    bool runnable = true;
+    for (auto op : best->getOperators())
+        if (auto mb = dynamic_cast<MemBoundOp *>(op))
+            runnable = runnable && mb->getExpr() != nullptr;
+    if (!runnable) {
+        std::printf("driver: bestGraph holds priced-only MemBound placeholders: not executed\n");
+        std::printf("driver: %s\n", ok ? "ok" : "FAILED");
+        std::fflush(stdout);
+        std::_Exit(ok ? 0 : 1);
+    }
     // run both programs on the same inputs
     int seed = 1;
     std::map<uint64_t, Tensor *> byHash;

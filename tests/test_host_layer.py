@@ -325,6 +325,7 @@ MEMBOUND_DRIVER = os.path.join(LIB, "pet_membound_driver")
 @pytest.mark.parametrize("args", [
     "1 64 56 56 64 3 1 1",         # benchmark configuration 1
     "1 512 64 64 512 3 2 2",       # the 512 -> 512 layer of the dilated block
+    "1 512 64 64 512 3 2 2 nnet",  # the same with the reference's NMutator as mutation engine
 ])
 def test_reference_search_engine_runs_on_the_device(args):
     """The reference's SearchEngine::run (src/Graph/search_engine.cc:54-118), compiled
@@ -358,7 +359,8 @@ def test_membound_operator_agrees_with_the_reference_interpreter():
     print(res.stdout[-4000:])
     print(res.stderr[-2000:])
     assert res.returncode == 0
-    assert res.stdout.count("[  OK  ]") >= 8 and "0 failed" in res.stdout
+    assert res.stdout.count("[  OK  ]") >= 9 and "0 failed" in res.stdout
+    assert "NMutator naive MemBound of a convolution equals the convolution" in res.stdout
 
 
 # ---- the benchmark networks through Graph -> SubGraph -> CodeEngine ---------------
