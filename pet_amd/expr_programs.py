@@ -1,5 +1,6 @@
-"""A small assembler for the index-expression programs of include/pet_hip.h, used by the
-tests to write MemBound operators down as expressions:
+"""A small assembler for the index-expression programs of include/pet_hip.h: MemBound
+operators written down as expressions (the C++ host layer flattens the reference's nnet
+trees into the same format):
 
     I("h") + 1, I("w") % 2, C(3)            index expressions (iterators, constants)
     T(0, [idx, ...])                         tensor 0 read at the indices, 0 outside

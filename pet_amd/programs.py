@@ -123,6 +123,14 @@ class GpuNS:
     def reshape(self, x, shape):
         return x.view(shape)
 
+    def expr(self, code, inputs):
+        """MemBound operator: the index-expression program `code` over `inputs`."""
+        key = tuple(code)
+        progs = self.__dict__.setdefault("_progs", {})
+        if key not in progs:
+            progs[key] = self.ops.ExprProgram(list(code))
+        return self._k(self.ops.expr(progs[key], list(inputs)))
+
 
 def _table(ns, p, T):
     """Device copies of the parameters, made on first use and kept in ``T`` so
@@ -240,6 +248,29 @@ def run_c3(ns, p, transformed=False, T=None):
             pre = "l%d.b%d" % (li + 1, bi)
             stride = 2 if (bi == 0 and li > 0) else 1
             has_ds = (pre + ".ds.w") in p
+            if has_ds and transformed and li >= 2:
+                # 1x1 conv -> GEMM (nmutator.cc:641-668: reshape the image to [c, pixels],
+                # Matmul(W[f, c], .), reshape back; at batch 1 no transpose is needed). The
+                # stride-2 downsample reads every second row and column, so a MemBound
+                # gather stands where the reference has its reshape. The 1x1 conv's bias
+                # joins the bias of the conv whose residual it feeds (a weight-side Add).
+                from .expr_programs import C, I, R, T as Tn, assemble
+                _, cin, hh, ww = tuple(x.shape)
+                oh, ow = hh // 2, ww // 2
+                fo = p[pre + ".ds.w"].shape[0]
+                gather = assemble([(1, cin, hh, ww)],
+                                  R([("b", 0, 1), ("c", 0, cin), ("p", 0, oh * ow)], [],
+                                    Tn(0, [C(0), I("c"), (I("p") // ow) * 2, (I("p") % ow) * 2])))
+                if pre + ".c2ds.b" not in T:
+                    T[pre + ".c2ds.b"] = ns.add([T[pre + ".c2.b"], T[pre + ".ds.b"]])
+                y = ns.conv2d(x, T[pre + ".c1.w"], 1, 1, stride, stride,
+                              bias=T[pre + ".c1.b"], act="relu")
+                xa = ns.expr(gather, [x])                                   # [1, c, oh*ow]
+                idn = ns.matmul(ns.reshape(T[pre + ".ds.w"], (1, fo, cin)), xa)
+                idn = ns.reshape(idn, (1, fo, oh, ow))
+                x = ns.conv2d(y, T[pre + ".c2.w"], 1, 1, bias=T[pre + ".c2ds.b"], residual=idn,
+                              act="relu")
+                continue
             if has_ds and transformed:
                 # PET merge of the two convs that read the same tensor
                 # (generator.cc:1236-1325, MAX variant): the 1x1/s2 filter is

@@ -52,6 +52,9 @@ class OracleNS:
                                v.reshape(seq, hidden), heads, float(scale.reshape(-1)[0]))
         return out.reshape(1, seq, hidden)
 
+    def expr(self, code, inputs):
+        return self.o.expr(code, inputs)
+
     def permute_flat(self, x, flat, perm):
         return self.o.permute_flat(x, flat, perm)
 

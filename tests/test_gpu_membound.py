@@ -5,7 +5,7 @@ import pytest
 import torch
 
 import oracle
-from expr_programs import C, I, OPS, R, T, assemble
+from pet_amd.expr_programs import C, I, OPS, R, T, assemble
 from test_oracle import _membound_cases
 
 pytestmark = pytest.mark.gpu

@@ -589,7 +589,7 @@ def test_g2bmm_gbmml_vs_dense_numpy(bs, m, k, w, d):
 
 def _membound_cases(rng):
     """(tensor shapes, top range, inputs, expected) with the expected values from numpy."""
-    from expr_programs import C, I, R, RS, T, relu, tanh
+    from pet_amd.expr_programs import C, I, R, RS, T, relu, tanh
     cases = []
     a = rng.integers(-3, 4, (4, 6)).astype(np.float32)
     cases.append(("transpose", [(4, 6)], R([("i", 0, 6), ("j", 0, 4)], [], T(0, [I("j"), I("i")])),
@@ -627,7 +627,7 @@ def _membound_cases(rng):
 def test_membound_expression_interpreter_vs_numpy():
     """MemBoundOp::compute (src/Graph/operator.cc:3601-3644 over nnet::Interpreter): the
     restated interpreter against index maps written in numpy."""
-    from expr_programs import assemble
+    from pet_amd.expr_programs import assemble
     for name, shapes, top, inputs, want in _membound_cases(np.random.default_rng(9)):
         got = oracle.expr(assemble(shapes, top), inputs)
         assert got is not None and got.shape == want.shape, name
