@@ -315,6 +315,62 @@ def main():
                    "GB/s": odd_bytes / ms / 1e6, "frac_hbm": odd_bytes / ms / 1e6 / HBM_PEAK_GBS})
     del big, odd, padded
 
+    # the other operator families of the library, one launch each at a representative size:
+    # transposed convolution (the reference's perf-test shape, src/Test/transposeconv_test_1.cc,
+    # and a generator layer), the band matmuls at a long-sequence shape (12 heads, 4096
+    # tokens, window 2 x 256 + 1), the fused attention core at BERT-base's shape, and a
+    # MemBound expression (the stride-2 gather in front of ResNet-18's 1x1 downsample)
+    def family(name, fn, flop=None, nbytes=None, reps=20):
+        try:
+            ms = time_kernel(fn, reps=reps, warm=3)
+        except Exception as exc:  # report, do not lose the main measurement
+            per_op.append({"op": name, "error": str(exc)[:200]})
+            return
+        line = {"op": name, "ms": ms}
+        if flop:
+            line["TFLOP/s"] = flop / ms / 1e9
+            line["frac_mfma"] = flop / ms / 1e9 / MFMA_FP32_PEAK_TFLOPS
+        if nbytes:
+            line["GB/s"] = nbytes / ms / 1e6
+            line["frac_hbm"] = nbytes / ms / 1e6 / HBM_PEAK_GBS
+        per_op.append(line)
+
+    if not args.no_configs:
+        for (n_, h_, f_, r_, c_, p_, s_) in ((1, 2, 448, 4, 256, 0, 1), (16, 16, 256, 4, 128, 1, 2)):
+            xt = torch.randn((n_, h_, h_, f_), device=dev)
+            wt = torch.randn((r_, r_, f_, c_), device=dev) * 0.05
+            oh_ = ops.conv_trans_out_dim(h_, r_, p_, s_, 1, 0)
+            yt = torch.empty((n_, oh_, oh_, c_), device=dev)
+            family("conv_trans %dx%dx%dx%d, %dx%d filters -> %d, stride %d" % (n_, h_, h_, f_, r_, r_, c_, s_),
+                   lambda: ops.conv_trans(xt, wt, p_, p_, s_, s_, out=yt),
+                   flop=2.0 * n_ * h_ * h_ * f_ * r_ * r_ * c_,
+                   nbytes=4.0 * (xt.numel() + wt.numel() + yt.numel()))
+        for dil in (1, 4):
+            qa = torch.randn((12, 4096, 64), device=dev)
+            kb = torch.randn((12, 4096, 64), device=dev)
+            band = torch.empty((12, 4096, 513), device=dev)
+            family("g2bmm 12x4096x64, width 256, dilation %d" % dil,
+                   lambda: ops.g2bmm(qa, kb, 256, dil, out=band),
+                   flop=2.0 * 12 * 4096 * 513 * 64, nbytes=4.0 * (2 * qa.numel() + band.numel()))
+            ctx = torch.empty((12, 4096, 64), device=dev)
+            family("gbmml 12x4096x513 x 12x4096x64, dilation %d" % dil,
+                   lambda: ops.gbmml(band, kb, dil, out=ctx),
+                   flop=2.0 * 12 * 4096 * 513 * 64, nbytes=4.0 * (band.numel() + 2 * kb.numel()))
+        qkv = torch.randn((3, 128, 768), device=dev)
+        att = torch.empty((128, 768), device=dev)
+        family("attention 12 heads x 128 x 64 (scores, softmax, context)",
+               lambda: ops.attention(qkv[0], qkv[1], qkv[2], 12, 0.125, out=att),
+               flop=2.0 * 2 * 12 * 128 * 128 * 64, nbytes=4.0 * 4 * 128 * 768)
+        from pet_amd import expr_programs as ep
+        gx = torch.randn((1, 128, 28, 28), device=dev)
+        gy = torch.empty((1, 128, 196), device=dev)
+        gather = ops.ExprProgram(ep.assemble(
+            [(1, 128, 28, 28)],
+            ep.R([("b", 0, 1), ("c", 0, 128), ("p", 0, 196)], [],
+                 ep.T(0, [ep.C(0), ep.I("c"), (ep.I("p") // 14) * 2, (ep.I("p") % 14) * 2]))))
+        family("membound: stride-2 gather 1x128x28x28 -> 1x128x196",
+               lambda: ops.expr(gather, [gx], out=gy), nbytes=4.0 * 2 * gy.numel())
+
     # ---- the other configurations: batch-1 latency of the original network and of
     # its PET-transformed program, each replayed as one HIP graph
     other = {}
@@ -450,6 +506,16 @@ def main():
                                       if res.returncode == 0 else {"error": res.stderr[-200:]})
                 except Exception as exc:
                     host_path[key] = {"error": str(exc)[:200]}
+
+        # beside each configuration's plain call-by-call program: the same original network
+        # as the graph runtime launches it (aliases, folded tails, hoisted initialisations,
+        # fused attention)
+        for name, model in (("c3_resnet18", "resnet18"), ("c4_bert_base_seq128", "bert"),
+                            ("c5_resnet3d18", "resnet3d18")):
+            got = host_path.get(model, {})
+            if name in other and "ms" in got:
+                other[name]["graph_runtime_ms"] = got["ms"]
+                other[name]["graph_runtime_kernels"] = got.get("kernels")
 
     dom_flop = conv_flop(DIL * DIL, 512, hs, hs, 512, 3, 3)
     dom_ms = conv_ms[0]

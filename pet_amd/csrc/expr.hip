@@ -16,6 +16,7 @@ namespace {
 constexpr int kMaxTensors = 8;
 constexpr int kMaxVars = 32;
 constexpr int kStack = 16;
+constexpr int kMaxLdsCode = 4096; // program words kept in LDS
 
 struct ExprParams {
     const int *code; // device copy of the program
@@ -30,26 +31,45 @@ struct ExprParams {
     int out_shape[PET_HIP_MAX_RANK];
 };
 
+// Interpreter state lives in LDS, one column per thread ([slot][thread]: a wave's accesses
+// to one slot are consecutive banks); arrays indexed at run time would otherwise sit in
+// scratch memory, a round trip through the cache per push and pop. The program is copied to
+// LDS too when it fits (kMaxLdsCode words), so an instruction fetch is an LDS broadcast.
+template <bool CODE_IN_LDS>
 __global__ __launch_bounds__(256) void expr_kernel(ExprParams p) {
-    const unsigned i = blockIdx.x * 256u + threadIdx.x;
+    extern __shared__ __attribute__((aligned(16))) int smem[];
+    const int nt = blockDim.x, tid = threadIdx.x;
+    int *istack = smem + tid;                    // slot s at istack[s * nt]
+    int *fbits = smem + kStack * nt + tid;       // value stack, as bit patterns
+    int *vars = smem + 2 * kStack * nt + tid;
+    int *tab = smem + (2 * kStack + kMaxVars) * nt; // [nd x 8][shape_at x 8]
+    int *lcode = tab + 2 * kMaxTensors;
+    if (tid < kMaxTensors) {
+        tab[tid] = p.nd[tid];
+        tab[kMaxTensors + tid] = p.shape_at[tid];
+    }
+    if (CODE_IN_LDS)
+        for (int j = tid; j < p.ncode; j += nt)
+            lcode[j] = p.code[j];
+    __syncthreads();
+    const unsigned i = blockIdx.x * (unsigned)nt + tid;
     if (i >= p.total)
         return;
-    int istack[kStack];
-    float fstack[kStack];
-    int vars[kMaxVars];
+    const int *__restrict__ c = CODE_IN_LDS ? lcode : p.code;
+#define IS(s) istack[(s) * nt]
+#define FS(s) (*reinterpret_cast<float *>(&fbits[(s) * nt]))
+#define VAR(s) vars[(s) * nt]
     int isp = 0, fsp = 0;
     // the output position, outermost dim first, is what the outermost range pops
     {
         unsigned t = i;
-        int pos[PET_HIP_MAX_RANK];
         for (int j = p.out_nd - 1; j >= 0; --j) {
-            pos[j] = (int)(t % (unsigned)p.out_shape[j]);
-            t /= (unsigned)p.out_shape[j];
+            const unsigned e = (unsigned)c[p.pc0 - p.out_nd + j];
+            IS(j) = (int)(t % e);
+            t /= e;
         }
-        for (int j = 0; j < p.out_nd; ++j)
-            istack[isp++] = pos[j];
+        isp = p.out_nd;
     }
-    const int *__restrict__ c = p.code;
     int pc = p.pc0;
     for (;;) {
         const int op = c[pc];
@@ -57,11 +77,13 @@ __global__ __launch_bounds__(256) void expr_kernel(ExprParams p) {
             break;
         switch (op) {
         case PET_HIP_EXPR_ICONST:
-            istack[isp++] = c[pc + 1];
+            IS(isp) = c[pc + 1];
+            ++isp;
             pc += 2;
             break;
         case PET_HIP_EXPR_IVAR:
-            istack[isp++] = vars[c[pc + 1]];
+            IS(isp) = VAR(c[pc + 1]);
+            ++isp;
             pc += 2;
             break;
         case PET_HIP_EXPR_IADD:
@@ -69,7 +91,8 @@ __global__ __launch_bounds__(256) void expr_kernel(ExprParams p) {
         case PET_HIP_EXPR_IMUL:
         case PET_HIP_EXPR_IDIV:
         case PET_HIP_EXPR_IMOD: {
-            const int b = istack[--isp], a = istack[--isp];
+            const int b = IS(isp - 1), a = IS(isp - 2);
+            isp -= 2;
             int r;
             if (op == PET_HIP_EXPR_IADD)
                 r = a + b;
@@ -81,27 +104,41 @@ __global__ __launch_bounds__(256) void expr_kernel(ExprParams p) {
                 r = b != 0 ? a / b : 0;
             else
                 r = b != 0 ? a % b : 0;
-            istack[isp++] = r;
+            IS(isp) = r;
+            ++isp;
             pc += 1;
             break;
         }
         case PET_HIP_EXPR_LOAD: {
-            const int t = c[pc + 1], nd = p.nd[t];
-            const int *shape = c + p.shape_at[t];
+            const int t = c[pc + 1], nd = tab[t];
+            const int *shape = c + tab[kMaxTensors + t];
             isp -= nd;
             unsigned off = 0;
             bool inside = true;
             for (int d = 0; d < nd; ++d) {
-                const int idx = istack[isp + d];
-                inside = inside && (unsigned)idx < (unsigned)shape[d];
-                off = off * (unsigned)shape[d] + (unsigned)idx;
+                const int idx = IS(isp + d);
+                const unsigned e = (unsigned)shape[d];
+                inside = inside && (unsigned)idx < e;
+                off = off * e + (unsigned)idx;
             }
-            fstack[fsp++] = inside ? p.in[t][off] : 0.f;
+            float v = 0.f;
+            if (inside) {
+                // the tensor number is the same for every thread: a scalar select
+                const float *src = p.in[0];
+#pragma unroll
+                for (int k = 1; k < kMaxTensors; ++k)
+                    src = t == k ? p.in[k] : src;
+                v = src[off];
+            }
+            FS(fsp) = v;
+            ++fsp;
             pc += 2;
             break;
         }
         case PET_HIP_EXPR_I2F:
-            fstack[fsp++] = (float)istack[--isp];
+            --isp;
+            FS(fsp) = (float)IS(isp);
+            ++fsp;
             pc += 1;
             break;
         case PET_HIP_EXPR_FADD:
@@ -109,7 +146,8 @@ __global__ __launch_bounds__(256) void expr_kernel(ExprParams p) {
         case PET_HIP_EXPR_FMUL:
         case PET_HIP_EXPR_FDIV:
         case PET_HIP_EXPR_FMOD: {
-            const float b = fstack[--fsp], a = fstack[--fsp];
+            const float b = FS(fsp - 1), a = FS(fsp - 2);
+            fsp -= 2;
             float r;
             if (op == PET_HIP_EXPR_FADD)
                 r = a + b;
@@ -121,16 +159,17 @@ __global__ __launch_bounds__(256) void expr_kernel(ExprParams p) {
                 r = truncf(a / b); // the reference's values are integers
             else
                 r = fmodf(a, b);
-            fstack[fsp++] = r;
+            FS(fsp) = r;
+            ++fsp;
             pc += 1;
             break;
         }
         case PET_HIP_EXPR_FRELU:
-            fstack[fsp - 1] = fmaxf(fstack[fsp - 1], 0.f);
+            FS(fsp - 1) = fmaxf(FS(fsp - 1), 0.f);
             pc += 1;
             break;
         case PET_HIP_EXPR_FTANH:
-            fstack[fsp - 1] = tanhf(fstack[fsp - 1]);
+            FS(fsp - 1) = tanhf(FS(fsp - 1));
             pc += 1;
             break;
         case PET_HIP_EXPR_RANGE: {
@@ -140,14 +179,15 @@ __global__ __launch_bounds__(256) void expr_kernel(ExprParams p) {
             bool inside = true;
             for (int d = 0; d < n; ++d) {
                 const int *it = c + pc + 3 + 4 * d;
-                const int v = istack[isp + d];
-                vars[it[0]] = v;
+                const int v = IS(isp + d);
+                VAR(it[0]) = v;
                 inside = inside && v >= it[1] && v < it[2];
             }
             if (inside) {
                 pc += 3 + 4 * n;
             } else { // in the padding of the range: its value there is 0
-                fstack[fsp++] = 0.f;
+                FS(fsp) = 0.f;
+                ++fsp;
                 pc = skip;
             }
             break;
@@ -156,29 +196,36 @@ __global__ __launch_bounds__(256) void expr_kernel(ExprParams p) {
             // nsum, then (slot, lo, hi) per sum iterator
             const int n = c[pc + 1];
             for (int d = 0; d < n; ++d)
-                vars[c[pc + 2 + 3 * d]] = c[pc + 3 + 3 * d];
-            fstack[fsp++] = 0.f;
+                VAR(c[pc + 2 + 3 * d]) = c[pc + 3 + 3 * d];
+            FS(fsp) = 0.f;
+            ++fsp;
             pc += 2 + 3 * n;
             break;
         }
         default: { // PET_HIP_EXPR_SUMEND: nsum, body, then (slot, lo, hi) per sum iterator
             const int n = c[pc + 1], body = c[pc + 2];
-            const float v = fstack[--fsp];
-            fstack[fsp - 1] += v;
+            --fsp;
+            FS(fsp - 1) += FS(fsp);
             // advance the iterators, last one fastest
             int d = n - 1;
             for (; d >= 0; --d) {
                 const int *it = c + pc + 3 + 3 * d;
-                if (++vars[it[0]] < it[2])
+                const int v = VAR(it[0]) + 1;
+                if (v < it[2]) {
+                    VAR(it[0]) = v;
                     break;
-                vars[it[0]] = it[1];
+                }
+                VAR(it[0]) = it[1];
             }
             pc = d >= 0 ? body : pc + 3 + 3 * n;
             break;
         }
         }
     }
-    p.out[i] = fstack[fsp - 1];
+    p.out[i] = FS(fsp - 1);
+#undef IS
+#undef FS
+#undef VAR
 }
 
 } // namespace
@@ -379,7 +426,7 @@ int pet_hip_expr_f32(const int *code, int ncode, const int *device_code,
     PET_REQUIRE_INIT();
     if (!device_code || !out || (ninputs > 0 && !inputs))
         return set_error(PET_HIP_ERR_INVALID, "expr: null operand");
-    ExprParams p;
+    ExprParams p{};
     size_t in_elems[kMaxTensors], out_elems;
     if (int rc = expr_validate(code, ncode, ninputs, &p.pc0, p.nd, p.shape_at, in_elems, &p.out_nd,
                                p.out_shape, &out_elems))
@@ -395,8 +442,27 @@ int pet_hip_expr_f32(const int *code, int ncode, const int *device_code,
     p.ncode = ncode;
     p.out = out;
     p.total = (unsigned)out_elems;
-    const unsigned grid = (unsigned)((out_elems + 255) / 256);
-    hipLaunchKernelGGL(expr_kernel, dim3(grid), dim3(256), 0, as_stream(stream), p);
+    // small outputs go out as one-wave workgroups so that they still spread over the CUs
+    const unsigned nt = out_elems <= 64u * 2048u ? 64u : 256u;
+    const unsigned grid = (unsigned)((out_elems + nt - 1) / nt);
+    const bool in_lds = ncode <= kMaxLdsCode;
+    const size_t lds = sizeof(int) * ((size_t)(2 * kStack + kMaxVars) * nt + 2 * kMaxTensors +
+                                      (in_lds ? (size_t)ncode : 0));
+    static int attr_status = [] {
+        const hipError_t a = hipFuncSetAttribute(reinterpret_cast<const void *>(&expr_kernel<true>),
+                                                 hipFuncAttributeMaxDynamicSharedMemorySize,
+                                                 96 * 1024);
+        const hipError_t b = hipFuncSetAttribute(reinterpret_cast<const void *>(&expr_kernel<false>),
+                                                 hipFuncAttributeMaxDynamicSharedMemorySize,
+                                                 96 * 1024);
+        return a == hipSuccess && b == hipSuccess ? 0 : 1;
+    }();
+    if (attr_status)
+        return set_error(PET_HIP_ERR_RUNTIME, "expr: cannot size the LDS allocation");
+    if (in_lds)
+        hipLaunchKernelGGL(expr_kernel<true>, dim3(grid), dim3(nt), lds, as_stream(stream), p);
+    else
+        hipLaunchKernelGGL(expr_kernel<false>, dim3(grid), dim3(nt), lds, as_stream(stream), p);
     return check_launch("expr_kernel");
 }
 

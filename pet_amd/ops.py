@@ -264,7 +264,8 @@ class ExprProgram:
         self.out_shape = tuple(code[at + 1:at + 1 + code[at]])
 
     def __del__(self):
-        if getattr(self, "dev", None) is not None and self.dev.value:
+        # at interpreter exit the module globals may already be gone
+        if getattr(self, "dev", None) is not None and self.dev.value and abi is not None:
             abi.status("pet_hip_free", self.dev)
 
 

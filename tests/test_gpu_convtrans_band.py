@@ -96,6 +96,10 @@ BAND_CASES = [
     (2, 100, 64, 20, 1),
     (1, 257, 64, 33, 4),    # ragged row blocks in every residue class
     (8, 512, 64, 64, 1),    # a sliding-window attention head block
+    (2, 70, 96, 9, 2),      # three 32-wide chunks of the feature axis
+    (1, 64, 32, 40, 1),     # one chunk, band wider than the matrix
+    (32, 2048, 128, 8, 1),  # many tiles: a tile per wave, 64 output columns in GBMML
+    (32, 4096, 32, 4, 1),   # many tiles of 32 output columns
 ]
 
 
