@@ -496,7 +496,7 @@ def main():
         # plain, and with --tune: Operator::perf on every operator first, so that each
         # contraction runs with the algorithm that timed fastest for it (what PET's search
         # leaves in its PerfEngine)
-        for model in ("dilated:pet", "dilated", "resnet18", "bert", "resnet3d18"):
+        for model in ("dilated:pet", "dilated", "resnet18", "bert", "bert:pet", "resnet3d18"):
             for key, extra in ((model, []), (model + " tuned", ["--tune"])):
                 try:
                     res = subprocess.run([run_model, model, "--rounds", str(max(50, args.steps)),
@@ -516,6 +516,10 @@ def main():
             if name in other and "ms" in got:
                 other[name]["graph_runtime_ms"] = got["ms"]
                 other[name]["graph_runtime_kernels"] = got.get("kernels")
+            pet = host_path.get(model + ":pet", {})
+            if name in other and "ms" in pet:
+                other[name]["graph_runtime_pet_ms"] = pet["ms"]
+                other[name]["graph_runtime_pet_kernels"] = pet.get("kernels")
 
     dom_flop = conv_flop(DIL * DIL, 512, hs, hs, 512, 3, 3)
     dom_ms = conv_ms[0]

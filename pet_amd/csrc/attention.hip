@@ -8,12 +8,19 @@
 // through an inline kernel (src/Graph/code_engine.cc:1103-1169, 1707-1731).
 //
 // One workgroup owns 32 queries of one head; wave w owns keys 32w .. 32w+31:
-//   S_w = Q_blk K_w^T     32x32 tile, both operands contiguous along dh (16-byte loads)
-//   row max and row sum   across the 32 lanes of a half-wave, then across waves through LDS
-//   O_w = P_w V_w         P_w goes through LDS to become the row operand; V is read
-//                         across lanes along dh (coalesced)
-//   out = (sum_w O_w) / rowsum, the waves adding in wave order (results do not depend on
-//   timing).
+//   S_w^T = K_w Q_blk^T   32x32 tile, both operands contiguous along dh (16-byte loads). The
+//                         transposed product leaves a lane holding ONE query (its column)
+//                         and 16 of the 32 keys in its accumulator registers, so
+//   row max and row sum   are 16 in-register steps and one exchange between the half-waves,
+//                         then across waves through LDS, and
+//   O_w = P_w V_w         takes the accumulator registers directly as its row operand:
+//                         register r of half-wave hk is key (r/4)*8 + hk*4 + r%4, and the MFMA
+//                         steps are free to take the keys in that order; V is read across
+//                         lanes along dh (coalesced), and its loads are issued before the
+//                         first product so that they are there when the softmax is done.
+//   out = (sum_w O_w) / rowsum: the waves add their tiles into four LDS slots, wave w into
+//   slot w % 4 in rounds of four waves, and the slots are added in order (results do not
+//   depend on timing).
 // seq <= 512 (16 waves), dh a multiple of 32 up to 128.
 #include "mfma_common.h"
 
@@ -32,8 +39,13 @@ struct AttnParams {
     long long sq, sk, sv, so;        // batch strides in floats
 };
 
-template <int DH>
-__global__ __launch_bounds__(1024) void attention_kernel(AttnParams p) {
+constexpr int kSlots = 4; // partial output tiles in LDS
+
+// MAXT: 256 for up to four waves (seq <= 128; registers are plentiful), else 1024, where a
+// wave has 128 registers: V is then fetched after the softmax for dh > 64, and a 128-wide
+// head takes its S product in two halves.
+template <int DH, int MAXT>
+__global__ __launch_bounds__(MAXT) void attention_kernel(AttnParams p) {
     extern __shared__ __attribute__((aligned(16))) float lds[];
     constexpr int TN = DH / 32;
     constexpr int KH = DH / 2; // dh values per half-wave in the S product
@@ -45,102 +57,117 @@ __global__ __launch_bounds__(1024) void attention_kernel(AttnParams p) {
     const int head = blockIdx.y;
     const int b = blockIdx.z;
     const int k0 = wave * 32;
-    // LDS: [red: nw*32][sumred: nw*32][P: nw*32*33][O: 32*DH]
+    // LDS: [red: nw*32][sumred: nw*32][O slots: kSlots*32*DH]
     float *red = lds;
     float *sred = lds + nw * 32;
-    float *pbuf = lds + 2 * nw * 32 + wave * (32 * 33);
-    float *obuf = lds + 2 * nw * 32 + nw * (32 * 33);
+    float *obuf = lds + 2 * nw * 32;
 
     const float scale = p.scale * (p.scale_dev ? *p.scale_dev : 1.f);
     const float *qp = p.q + b * p.sq + (size_t)min(q0 + l32, p.seq - 1) * p.ldq + head * DH + hk * KH;
     const float *kp = p.k + b * p.sk + (size_t)min(k0 + l32, p.seq - 1) * p.ldk + head * DH + hk * KH;
+    constexpr bool EARLY_V = MAXT == 256 || DH <= 64;
+    constexpr int NJ = KH / 4, CJ = (MAXT == 1024 && NJ > 8) ? 8 : NJ; // float4 per operand and pass
+    float4 qv[CJ], kv[CJ];
+#pragma unroll
+    for (int j = 0; j < CJ; ++j) {
+        qv[j] = *reinterpret_cast<const float4 *>(qp + 4 * j);
+        kv[j] = *reinterpret_cast<const float4 *>(kp + 4 * j);
+    }
+    // V rows of this wave's keys in the order the accumulator registers hold them
+    const float *vp = p.v + b * p.sv + head * DH + l32;
+    float vv[16][TN];
+    auto load_v = [&]() __attribute__((always_inline)) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) {
+            const int key = k0 + (r / 4) * 8 + hk * 4 + (r % 4);
+            const float *vrow = vp + (size_t)min(key, p.seq - 1) * p.ldv;
+#pragma unroll
+            for (int tn = 0; tn < TN; ++tn)
+                vv[r][tn] = vrow[tn * 32];
+        }
+    };
+    if (EARLY_V)
+        load_v();
 
+    // S^T: rows = keys (operand A = K), columns = queries (operand B = Q)
     floatx16 s;
 #pragma unroll
     for (int r = 0; r < 16; ++r)
         s[r] = 0.f;
 #pragma unroll
-    for (int j = 0; j < KH; j += 4) {
-        const float4 a = *reinterpret_cast<const float4 *>(qp + j);
-        const float4 bb = *reinterpret_cast<const float4 *>(kp + j);
-        s = __builtin_amdgcn_mfma_f32_32x32x2f32(a.x, bb.x, s, 0, 0, 0);
-        s = __builtin_amdgcn_mfma_f32_32x32x2f32(a.y, bb.y, s, 0, 0, 0);
-        s = __builtin_amdgcn_mfma_f32_32x32x2f32(a.z, bb.z, s, 0, 0, 0);
-        s = __builtin_amdgcn_mfma_f32_32x32x2f32(a.w, bb.w, s, 0, 0, 0);
+    for (int c = 0; c < NJ; c += CJ) {
+        if (c > 0) {
+#pragma unroll
+            for (int j = 0; j < CJ; ++j) {
+                qv[j] = *reinterpret_cast<const float4 *>(qp + 4 * (c + j));
+                kv[j] = *reinterpret_cast<const float4 *>(kp + 4 * (c + j));
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < CJ; ++j) {
+            s = __builtin_amdgcn_mfma_f32_32x32x2f32(kv[j].x, qv[j].x, s, 0, 0, 0);
+            s = __builtin_amdgcn_mfma_f32_32x32x2f32(kv[j].y, qv[j].y, s, 0, 0, 0);
+            s = __builtin_amdgcn_mfma_f32_32x32x2f32(kv[j].z, qv[j].z, s, 0, 0, 0);
+            s = __builtin_amdgcn_mfma_f32_32x32x2f32(kv[j].w, qv[j].w, s, 0, 0, 0);
+        }
     }
-    // register r of a lane: query row (r/4)*8 + hk*4 + r%4, key column k0 + l32
-    const bool kvalid = k0 + l32 < p.seq;
-    float mx[16];
+    // register r of a lane: key k0 + (r/4)*8 + hk*4 + r%4, query q0 + l32
+    float mx = -INFINITY;
 #pragma unroll
     for (int r = 0; r < 16; ++r) {
+        const bool kvalid = k0 + (r / 4) * 8 + hk * 4 + (r % 4) < p.seq;
         s[r] = kvalid ? s[r] * scale : -INFINITY;
-        float m = s[r];
-#pragma unroll
-        for (int off = 1; off < 32; off <<= 1)
-            m = fmaxf(m, __shfl_xor(m, off));
-        mx[r] = m;
+        mx = fmaxf(mx, s[r]);
     }
-    if (l32 == 0) {
-#pragma unroll
-        for (int r = 0; r < 16; ++r)
-            red[wave * 32 + (r / 4) * 8 + hk * 4 + (r % 4)] = mx[r];
-    }
+    mx = fmaxf(mx, __shfl_xor(mx, 32));
+    if (hk == 0)
+        red[wave * 32 + l32] = mx;
     __syncthreads();
-    float sum[16];
+    float m = red[l32];
+    for (int w = 1; w < nw; ++w)
+        m = fmaxf(m, red[w * 32 + l32]);
+    float sum = 0.f;
 #pragma unroll
     for (int r = 0; r < 16; ++r) {
-        const int row = (r / 4) * 8 + hk * 4 + (r % 4);
-        float m = red[row];
-        for (int w = 1; w < nw; ++w)
-            m = fmaxf(m, red[w * 32 + row]);
-        const float e = kvalid ? expf(s[r] - m) : 0.f;
-        s[r] = e;
-        float t = e;
-#pragma unroll
-        for (int off = 1; off < 32; off <<= 1)
-            t += __shfl_xor(t, off);
-        sum[r] = t;
-        pbuf[row * 33 + l32] = e; // P_w as [query][key]
+        // a key past the end holds -inf: exp gives 0 (m is finite: key 0 is always valid)
+        s[r] = expf(s[r] - m);
+        sum += s[r];
     }
-    if (l32 == 0) {
-#pragma unroll
-        for (int r = 0; r < 16; ++r)
-            sred[wave * 32 + (r / 4) * 8 + hk * 4 + (r % 4)] = sum[r];
-    }
-    // O_w = P_w V_w: row operand from LDS (this wave's own region), V across lanes
+    sum += __shfl_xor(sum, 32);
+    if (hk == 0)
+        sred[wave * 32 + l32] = sum;
+    if (!EARLY_V)
+        load_v();
+
+    // O_w = P_w V_w: MFMA step r takes key (r/4)*8 + hk*4 + r%4 from both operands
     floatx16 o[TN];
 #pragma unroll
     for (int tn = 0; tn < TN; ++tn)
 #pragma unroll
         for (int r = 0; r < 16; ++r)
             o[tn][r] = 0.f;
-    const float *vp = p.v + b * p.sv + head * DH + l32;
-    // the wave's LDS writes above are visible to its own lanes after this wait
-    __builtin_amdgcn_s_waitcnt(0xc07f); // lgkmcnt(0)
-    __builtin_amdgcn_wave_barrier();
 #pragma unroll
-    for (int j = 0; j < 16; ++j) {
-        const int kk = hk * 16 + j; // key inside the wave's 32
-        const float a = pbuf[l32 * 33 + kk];
-        const float *vrow = vp + (size_t)min(k0 + kk, p.seq - 1) * p.ldv;
+    for (int r = 0; r < 16; ++r)
 #pragma unroll
         for (int tn = 0; tn < TN; ++tn)
-            o[tn] = __builtin_amdgcn_mfma_f32_32x32x2f32(a, vrow[tn * 32], o[tn], 0, 0, 0);
-    }
-    // sum of the waves' O tiles in wave order
-    for (int w = 0; w < nw; ++w) {
-        if (wave == w) {
+            o[tn] = __builtin_amdgcn_mfma_f32_32x32x2f32(s[r], vv[r][tn], o[tn], 0, 0, 0);
+
+    // the waves' O tiles into the slots, a round of kSlots waves at a time
+    float *slot = obuf + (wave % kSlots) * (32 * DH);
+    for (int round = 0; round * kSlots < nw; ++round) {
+        if (wave / kSlots == round) {
 #pragma unroll
             for (int tn = 0; tn < TN; ++tn)
 #pragma unroll
                 for (int r = 0; r < 16; ++r) {
                     const int row = (r / 4) * 8 + hk * 4 + (r % 4);
-                    float *dst = obuf + row * DH + tn * 32 + l32;
-                    *dst = w == 0 ? o[tn][r] : *dst + o[tn][r];
+                    float *dst = slot + row * DH + tn * 32 + l32;
+                    *dst = round == 0 ? o[tn][r] : *dst + o[tn][r];
                 }
         }
         __syncthreads();
     }
+    const int nslots = nw < kSlots ? nw : kSlots;
     // out[q0 + row][head*DH + d] = O / rowsum
     for (int i = threadIdx.x; i < 32 * DH; i += blockDim.x) {
         const int row = i / DH, d = i - row * DH;
@@ -149,16 +176,19 @@ __global__ __launch_bounds__(1024) void attention_kernel(AttnParams p) {
         float t = sred[row];
         for (int w = 1; w < nw; ++w)
             t += sred[w * 32 + row];
-        p.out[b * p.so + (size_t)(q0 + row) * p.ldo + head * DH + d] = obuf[i] / t;
+        float v = obuf[i];
+        for (int sl = 1; sl < nslots; ++sl)
+            v += obuf[sl * (32 * DH) + i];
+        p.out[b * p.so + (size_t)(q0 + row) * p.ldo + head * DH + d] = v / t;
     }
 }
 
-template <int DH>
-int launch_attention(const AttnParams &p, hipStream_t stream) {
+template <int DH, int MAXT>
+int launch_attention_as(const AttnParams &p, hipStream_t stream) {
     const int nw = (p.seq + 31) / 32;
-    const size_t lds_bytes = sizeof(float) * (2 * nw * 32 + nw * 32 * 33 + 32 * DH);
+    const size_t lds_bytes = sizeof(float) * (2 * nw * 32 + kSlots * 32 * DH);
     static int attr_status = [] {
-        return hipFuncSetAttribute(reinterpret_cast<const void *>(&attention_kernel<DH>),
+        return hipFuncSetAttribute(reinterpret_cast<const void *>(&attention_kernel<DH, MAXT>),
                                    hipFuncAttributeMaxDynamicSharedMemorySize,
                                    96 * 1024) == hipSuccess
                    ? 0
@@ -167,8 +197,14 @@ int launch_attention(const AttnParams &p, hipStream_t stream) {
     if (attr_status)
         return set_error(PET_HIP_ERR_RUNTIME, "attention: cannot size the LDS allocation");
     dim3 grid((unsigned)nw, (unsigned)p.heads, (unsigned)p.batch);
-    hipLaunchKernelGGL((attention_kernel<DH>), grid, dim3(64 * nw), lds_bytes, stream, p);
+    hipLaunchKernelGGL((attention_kernel<DH, MAXT>), grid, dim3(64 * nw), lds_bytes, stream, p);
     return check_launch("attention_kernel");
+}
+
+template <int DH>
+int launch_attention(const AttnParams &p, hipStream_t stream) {
+    return p.seq <= 128 ? launch_attention_as<DH, 256>(p, stream)
+                        : launch_attention_as<DH, 1024>(p, stream);
 }
 
 } // namespace

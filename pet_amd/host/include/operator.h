@@ -331,6 +331,15 @@ class MatmulOp : public Operator {
     int numInputs() override { return 2; }
     int numOutputs() override { return 1; }
     Tensor *getBias() const { return bias; }
+    // Set by the graph runtime when the lhs is `count` copies of one [1, m, k] tensor stacked
+    // on dim 0 (an Extend, or a Concat of the same tensor: the batch-matmul merge of
+    // src/Mutant/generator.cc:1495-1552 applied to projections of one input): the launch then
+    // reads that tensor for every batch entry and the stacked copy is never made.
+    void setSharedLhs(Tensor *src) { sharedLhs = src; }
+    Tensor *getSharedLhs() const { return sharedLhs; }
+    // A bias of b * n values is one row per batch entry (the merged projections' biases).
+    bool biasPerBatch() const;
+    unsigned operandFlags() const;
     void setAct(ActType a) { act = a; }
     ActType getAct() const { return act; }
     bool getTransA() const { return transA; }
@@ -346,6 +355,7 @@ class MatmulOp : public Operator {
     Tensor *bias;
     ActType act;
     int algo = 0;
+    Tensor *sharedLhs = nullptr;
 };
 
 // ---- ConvTrans -----------------------------------------------------------------------

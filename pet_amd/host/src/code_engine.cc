@@ -462,14 +462,53 @@ int launchChain(const std::vector<TransposeOp *> &row, pet_hip_stream_t s) {
 
 } // namespace
 
+// A Matmul whose lhs is one [1, m, k] tensor stacked b times on dim 0 (an Extend, or a Concat
+// of the same tensor) and read by nothing else reads that tensor directly: the stacking
+// operator is skipped and never launched. Returns the skipped operators.
+static std::set<const Operator *> planSharedLhs(const OpVec &order, const TensorVec &graphOutputs) {
+    std::set<const Operator *> skipped;
+    for (auto op : order) {
+        auto mm = dynamic_cast<MatmulOp *>(op);
+        if (!mm)
+            continue;
+        mm->setSharedLhs(nullptr);
+        if (mm->getTransA())
+            continue;
+        Tensor *A = mm->getInputs()[0];
+        Operator *prod = A->getOutputOf();
+        if (prod == nullptr || A->getInputOf().size() != 1 ||
+            std::find(graphOutputs.begin(), graphOutputs.end(), A) != graphOutputs.end())
+            continue;
+        Tensor *src = nullptr;
+        if (auto ex = dynamic_cast<ExtendOp *>(prod)) {
+            if (ex->getDim() == 0)
+                src = prod->getInputs()[0];
+        } else if (auto cat = dynamic_cast<ConcatOp *>(prod)) {
+            if (cat->getDim() == 0) {
+                src = prod->getInputs()[0];
+                for (auto in : prod->getInputs())
+                    if (in != src)
+                        src = nullptr;
+            }
+        }
+        if (src == nullptr || A->getDims().size() != 3 || src->size() * A->getDims()[0] != A->size() ||
+            src->size() != (size_t)A->getDims()[1] * A->getDims()[2])
+            continue;
+        mm->setSharedLhs(src);
+        skipped.insert(prod);
+    }
+    return skipped;
+}
+
 // Storage sharing, decided before anything is captured:
 //  * Split on dim 0: every output is a slab of the input buffer.
 //  * Concat on dim 0: every input that an operator of this graph produces (and
 //    that is used nowhere else in a conflicting way) is produced directly
 //    into its slab of the output buffer.
 //  * Reshape: the output is the input buffer.
-static AliasPlan planAliases(const OpVec &order) {
+static AliasPlan planAliases(const OpVec &order, const std::set<const Operator *> &alreadySkipped) {
     AliasPlan plan;
+    plan.skipped.insert(alreadySkipped.begin(), alreadySkipped.end());
     std::set<const Tensor *> aliased;
     // tensors whose buffer another tensor already points into: moving such a
     // buffer (into a concat's output) would leave those views on freed memory
@@ -572,7 +611,8 @@ std::unique_ptr<GraphExec> CodeEngine::instantiate(std::shared_ptr<SubGraph> &gr
                 t->devicePtr();
     }
     importAlgos(order);
-    AliasPlan plan = planAliases(order);
+    const std::set<const Operator *> stacked = planSharedLhs(order, graph->getOutputs());
+    AliasPlan plan = planAliases(order, stacked);
     TransposeChains rows = planTransposeChains(order, graph->getOutputs(), plan.skipped);
     FusedTails tails = planFusedTails(order, graph->getOutputs(), plan.skipped,
                                       [](const FusedTail &f) {
@@ -671,7 +711,7 @@ std::unique_ptr<GraphExec> CodeEngine::instantiate(std::shared_ptr<SubGraph> &gr
             auto tail = tails.atAdd.find(prod);
             if (tail != tails.atAdd.end() && tail->second.out != t)
                 inside = true;
-            if (inside || lp.preAct.count(t) || att.absorbed.count(prod))
+            if (inside || lp.preAct.count(t) || att.absorbed.count(prod) || stacked.count(prod))
                 continue; // not there, or there without its ReLU
             t->deviceWritten();
             t->setComputed();
@@ -747,7 +787,7 @@ std::string CodeEngine::genCode(std::shared_ptr<SubGraph> &graph) {
                 all.push_back(t);
     }
     std::set<const Tensor *> viewOf, viewBase;
-    std::set<const Operator *> skipped;
+    std::set<const Operator *> skipped = planSharedLhs(order, graph->getOutputs());
     // storage sharing, mirrored from instantiate(): split / concat on dim 0, reshape
     std::vector<std::string> aliasLines;
     for (auto op : order) {
@@ -912,12 +952,12 @@ std::string CodeEngine::genCode(std::shared_ptr<SubGraph> &graph) {
             bool ta, tb;
             int b, m, n, k;
             std::tie(ta, tb, b, m, n, k) = mm->getArgs();
-            const unsigned fl = flagsOf(op) | PET_HIP_CONV_ALGO(mm->getAlgo());
+            const unsigned fl = flagsOf(op) | mm->operandFlags() | PET_HIP_CONV_ALGO(mm->getAlgo());
             c << (fl     ? "pet_hip_bmm_ex_f32("
                   : tail ? "pet_hip_bmm_res_f32("
                          : "pet_hip_bmm_f32(")
               << ta << ", " << tb << ", " << b << ", " << m << ", " << n << ", " << k << ", "
-              << in(0) << ", " << in(1) << ", " << out(0) << ", " << nullable(e, mm->getBias())
+              << (mm->getSharedLhs() ? e.name(mm->getSharedLhs()) : in(0)) << ", " << in(1) << ", " << out(0) << ", " << nullable(e, mm->getBias())
               << ", "
               << (tail ? res : fl ? std::string("nullptr, ") : std::string())
               << actOf(mm->getAct()) << ", " << (fl ? std::to_string(fl) + "u, " : std::string())

@@ -114,7 +114,7 @@ Model resnet18(int hw, int width, int classes) {
     return finish("resnet18", std::move(g), b.macs);
 }
 
-Model bertBase(int layers, int seq, int hidden, int heads, int ffn) {
+Model bertBase(int layers, int seq, int hidden, int heads, int ffn, bool mergedQkv) {
     std::unique_ptr<Graph> g(new Graph());
     Builder b{*g};
     const int dh = hidden / heads;
@@ -128,8 +128,22 @@ Model bertBase(int layers, int seq, int hidden, int heads, int ffn) {
         return g->layernorm(t, b.fresh(), g->tensor({hidden}), g->tensor({hidden}))->getOutputs()[0];
     };
     for (int l = 0; l < layers; ++l) {
-        Tensor *q = toHeads(b.linear(x, hidden)), *k = toHeads(b.linear(x, hidden));
-        Tensor *v = toHeads(b.linear(x, hidden));
+        Tensor *q, *k, *v;
+        if (mergedQkv) {
+            // PET's batch-matmul merge (src/Mutant/generator.cc:1495-1552) of the three
+            // projections of x: lhs stacked on dim 0 (the same tensor three times), the
+            // weights and biases stacked the same way, one Matmul with b = 3, Split on dim 0
+            Tensor *x3 = g->concat({x, x, x}, 0)->getOutputs()[0];
+            Tensor *w3 = g->tensor({3, hidden, hidden});
+            w3->setType(Tensor::Weight);
+            Tensor *y3 = g->matmul(x3, w3, false, false, g->tensor({3, hidden}))->getOutputs()[0];
+            b.macs += 3.0 * seq * hidden * hidden;
+            const TensorVec &parts = g->split(y3, 0, 3)->getOutputs();
+            q = toHeads(parts[0]), k = toHeads(parts[1]), v = toHeads(parts[2]);
+        } else {
+            q = toHeads(b.linear(x, hidden)), k = toHeads(b.linear(x, hidden));
+            v = toHeads(b.linear(x, hidden));
+        }
         Tensor *s = b.bmm(q, k, true); // [heads, seq, seq]
         s = g->softmax(g->mul({s, scale})->getOutputs()[0], b.fresh(), 2)->getOutputs()[0];
         Tensor *ctx = b.bmm(s, v, false); // [heads, seq, dh]
@@ -138,7 +152,7 @@ Model bertBase(int layers, int seq, int hidden, int heads, int ffn) {
         Tensor *h = b.linear(b.linear(x, ffn, Operator::Gelu), hidden);
         x = norm(g->add({x, h})->getOutputs()[0]);
     }
-    return finish("bert", std::move(g), b.macs);
+    return finish(mergedQkv ? "bert:pet" : "bert", std::move(g), b.macs);
 }
 
 Model resnet3d18(int t, int hw, int width, int classes) {
@@ -173,6 +187,8 @@ bool byName(const std::string &name, Model &out) {
         out = resnet18();
     else if (name == "bert")
         out = bertBase();
+    else if (name == "bert:pet")
+        out = bertBase(12, 128, 768, 12, 3072, true);
     else if (name == "resnet3d18")
         out = resnet3d18();
     else

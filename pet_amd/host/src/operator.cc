@@ -795,11 +795,22 @@ Dim MatmulOp::computeShape() {
     return ret;
 }
 
+bool MatmulOp::biasPerBatch() const {
+    bool ta, tb;
+    int b, m, n, k;
+    std::tie(ta, tb, b, m, n, k) = getArgs();
+    return bias != nullptr && b > 1 && bias->size() == (size_t)b * n;
+}
+
+unsigned MatmulOp::operandFlags() const {
+    return (sharedLhs ? PET_HIP_CALL_A_SHARED : 0u) | (biasPerBatch() ? PET_HIP_CALL_BIAS_PER_BATCH : 0u);
+}
+
 int MatmulOp::launch(pet_hip_stream_t stream) {
     bool ta, tb;
     int b, m, n, k;
     std::tie(ta, tb, b, m, n, k) = getArgs();
-    if (algo != 0)
+    if (algo != 0 || operandFlags() != 0)
         return launchFused(stream, nullptr, act, outputs[0]->devicePtr(), 0);
     return pet_hip_bmm_f32(ta, tb, b, m, n, k, inputs[0]->devicePtr(), inputs[1]->devicePtr(),
                            outputs[0]->devicePtr(), bias ? bias->devicePtr() : nullptr, (int)act,
@@ -813,12 +824,15 @@ int MatmulOp::launchFused(pet_hip_stream_t stream, const float *residual, ActTyp
     bool ta, tb;
     int b, m, n, k;
     std::tie(ta, tb, b, m, n, k) = getArgs();
-    return pet_hip_bmm_ex_f32(ta, tb, b, m, n, k, inputs[0]->devicePtr(), inputs[1]->devicePtr(),
-                              out, bias ? bias->devicePtr() : nullptr, residual, (int)finalAct,
-                              flags | PET_HIP_CONV_ALGO(algo), stream);
+    const float *A = sharedLhs ? sharedLhs->devicePtr() : inputs[0]->devicePtr();
+    return pet_hip_bmm_ex_f32(ta, tb, b, m, n, k, A, inputs[1]->devicePtr(), out,
+                              bias ? bias->devicePtr() : nullptr, residual, (int)finalAct,
+                              flags | operandFlags() | PET_HIP_CONV_ALGO(algo), stream);
 }
 
 bool MatmulOp::accumulates() const {
+    if (operandFlags() != 0)
+        return false; // these forms never add partial sums into an initialised output
     bool ta, tb;
     int b, m, n, k, yes = 0;
     std::tie(ta, tb, b, m, n, k) = getArgs();

@@ -295,7 +295,9 @@ static bool test_code_engine_graph_runtime() {
     CodeEngine ce;
     auto exec = ce.instantiate(s2);
     EXPECT(exec != nullptr);
-    EXPECT(exec->numAliasedOps() == 2); // rhs concat and the split; lhs concat repeats `a`
+    // rhs concat and the split share storage; the lhs concat repeats `a`, which the matmul
+    // then reads for both batch entries
+    EXPECT(exec->numAliasedOps() == 3);
     for (int rep = 0; rep < 3; ++rep) {
         EXPECT(exec->launch() && exec->sync());
         Tensor *o1 = s1->getOutputs()[0], *o2 = s2->getOutputs()[0];
@@ -305,9 +307,10 @@ static bool test_code_engine_graph_runtime() {
     double ms = exec->time(5, 20);
     EXPECT(std::isfinite(ms) && ms > 0.0);
     std::string code = ce.genCode(s2);
-    EXPECT(code.find("pet_hip_bmm_f32(") != std::string::npos);
+    EXPECT(code.find("pet_hip_bmm_ex_f32(") != std::string::npos);
+    EXPECT(code.find(", 16u, s)") != std::string::npos); // lhs shared by the batch entries
     EXPECT(code.find("pet_hip_graph_begin_capture") != std::string::npos);
-    EXPECT(code.find("pet_hip_concat(") != std::string::npos); // the repeated-input concat
+    EXPECT(code.find("pet_hip_concat(") == std::string::npos); // neither concat runs
     EXPECT(code.find("pet_hip_split(") == std::string::npos);  // aliased away
     return true;
 }
@@ -919,6 +922,67 @@ static bool convTransCase(int h, int w, int f, int r, int s, int c, int p, int s
     return true;
 }
 
+// PET's batch-matmul merge of three projections of one tensor: Concat({x, x, x}, 0) ->
+// Matmul(b = 3, stacked weights, one bias row per batch entry) -> Split on dim 0. The graph
+// runtime reads x for every batch entry instead of making the stacked copy; the result
+// equals the operators run one by one and the oracle's matmul on the stacked operand.
+static bool test_merged_projections() {
+    const int m = 16, k = 64, n = 32;
+    Graph g;
+    Tensor *x = g.tensor({1, m, k});
+    Tensor *x3 = g.concat({x, x, x}, 0)->getOutputs()[0];
+    Tensor *w3 = g.tensor({3, k, n});
+    w3->setType(Tensor::Weight);
+    Tensor *b3 = g.tensor({3, n});
+    Tensor *y3 = g.matmul(x3, w3, false, false, b3)->getOutputs()[0];
+    for (auto part : g.split(y3, 0, 3)->getOutputs())
+        g.relu(part);
+    g.updateConnection();
+    x->dataRand(5);
+    w3->dataRand(6);
+    b3->dataRand(7);
+    auto s1 = std::make_shared<SubGraph>(g.getOperators());
+    auto s2 = std::make_shared<SubGraph>(g.getOperators());
+    for (auto sg : {s1, s2})
+        for (auto t : sg->getInputs())
+            for (auto orig : g.getTensors())
+                if (orig->getHash() == t->getHash())
+                    t->setData(orig->getDataPtr());
+    EXPECT(s1->compute());
+    CodeEngine ce;
+    auto exec = ce.instantiate(s2);
+    EXPECT(exec != nullptr);
+    EXPECT(exec->numAliasedOps() == 2); // the stacking Concat and the Split
+    EXPECT(exec->launch() && exec->sync());
+    // oracle: relu(X3 W3 + b3) with X3 the stacked operand
+    std::vector<float> X3(3 * m * k), C(3 * m * n);
+    for (int i = 0; i < 3; ++i)
+        std::copy(x->getDataPtr(), x->getDataPtr() + m * k, X3.begin() + i * m * k);
+    oracle_matmul_f32(X3.data(), w3->getDataPtr(), C.data(), 3, m, n, k, 0, 0);
+    for (int i = 0; i < 3; ++i)
+        for (int r = 0; r < m; ++r)
+            for (int c = 0; c < n; ++c) {
+                float &v = C[((size_t)i * m + r) * n + c];
+                v = std::max(v + b3->getDataPtr()[i * n + c], 0.f);
+            }
+    EXPECT(s1->getOutputs().size() == 3 && s2->getOutputs().size() == 3);
+    for (size_t o = 0; o < 3; ++o) {
+        Tensor *o1 = s1->getOutputs()[o], *o2 = s2->getOutputs()[o];
+        o2->deviceWritten();
+        EXPECT(equalArrays(o1->getDataPtr(), o2->getDataPtr(), o1->size()));
+        bool matched = false; // the outputs are the three batch entries in some order
+        for (int i = 0; i < 3 && !matched; ++i)
+            matched = std::equal(C.begin() + (size_t)i * m * n, C.begin() + (size_t)(i + 1) * m * n,
+                                 o2->getDataPtr());
+        EXPECT(matched);
+    }
+    std::string code = ce.genCode(s2);
+    EXPECT(code.find("pet_hip_bmm_ex_f32(") != std::string::npos);
+    EXPECT(code.find(", 48u, s)") != std::string::npos); // shared lhs + bias row per batch entry
+    EXPECT(code.find("pet_hip_concat(") == std::string::npos);
+    return true;
+}
+
 static bool test_convtrans_reference_vectors() {
     EXPECT(convTransCase(2, 2, 3, 4, 4, 2, 1, 2,
                          {190,  740,  770,  592,  992,  2704, 2836, 1832, 1184, 3232, 3364,
@@ -989,6 +1053,7 @@ int main(int argc, char **argv) {
         {"conv_merge_programs", test_conv_merge_programs},
         {"convtrans_reference_vectors", test_convtrans_reference_vectors},
         {"band_matmuls", test_band_matmuls},
+        {"merged_projections", test_merged_projections},
     };
     std::string only = argc > 1 ? argv[1] : "";
     if (argc > 2)

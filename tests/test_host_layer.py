@@ -20,7 +20,8 @@ CASES = ["conv_vs_oracle", "conv_invalid_groups", "transpose_n2h_h2n", "batch_ge
          "split_ratio_and_eltwise", "conv_merge_programs", "conv3d_prepacked_graph",
          "random_graphs_replay_equals_eager", "batchnorm_pow_div",
          "gather_reduce_mean", "launch_fusion_block", "alias_plan_shared_storage",
-         "two_conv_verification", "convtrans_reference_vectors", "band_matmuls"]
+         "two_conv_verification", "convtrans_reference_vectors", "band_matmuls",
+         "merged_projections"]
 
 
 def test_host_library_is_built_and_exports_the_operator_classes():
@@ -368,7 +369,8 @@ RUN_MODEL = os.path.join(LIB, "pet_run_model")
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("model", ["dilated", "dilated:pet", "resnet18", "bert", "resnet3d18"])
+@pytest.mark.parametrize("model", ["dilated", "dilated:pet", "resnet18", "bert", "bert:pet",
+                                   "resnet3d18"])
 def test_model_graph_replay_equals_operator_by_operator_run(model):
     """pet_run_model --check: the captured HIP graph (storage sharing, transposes in a
     row folded into one kernel, constant 3-D filters repacked) against
@@ -385,6 +387,9 @@ def test_model_graph_replay_equals_operator_by_operator_run(model):
     assert rec["ms"] > 0
     if model == "dilated:pet":
         assert rec["folded"] == 2 and rec["kernels"] == 8
+    if model == "bert:pet":
+        # per layer: one merged projection instead of three, the stacking Concat never runs
+        assert rec["kernels"] == 108 - 2 * 12
 
 
 @pytest.mark.gpu
@@ -483,7 +488,7 @@ def test_python_module_runs_a_graph_on_the_device():
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("model", ["resnet18", "resnet3d18", "bert"])
+@pytest.mark.parametrize("model", ["resnet18", "resnet3d18", "bert", "bert:pet"])
 def test_emitted_model_program_compiles_and_agrees_with_the_runtime(model, tmp_path):
     """CodeEngine::genCode for a whole network (fused block tails, kt-major filters,
     storage sharing): the emitted C++ builds against pet_hip.h alone, runs, and its
@@ -496,7 +501,9 @@ def test_emitted_model_program_compiles_and_agrees_with_the_runtime(model, tmp_p
     assert res.returncode == 0, res.stderr[-2000:]
     rec = json.loads(res.stdout.strip().splitlines()[-1])
     text = src.read_text()
-    if model != "bert":
+    if model == "bert:pet":
+        assert ", 48u, s)" in text and "pet_hip_concat(" not in text  # shared lhs, bias rows
+    if not model.startswith("bert"):
         # a block tail became one call, with the ReLU of what it reads applied on load
         assert re.search(r"pet_hip_conv[23]d_ex_f32\([^;]*, (1[0-5]|[4-9])u, s\)", text)
     else:
