@@ -382,6 +382,53 @@ __global__ __launch_bounds__(256) void softmax_kernel(const float *__restrict__ 
         yp[j] = expf(xp[j] - mx) * inv;
 }
 
+// Rows of 256 * NV floats (NV <= 8), 16-byte aligned: a lane holds NV 16-byte words of the
+// row, of gamma and of beta (a row of BERT's 768 columns is three loads per operand).
+template <int NV>
+__global__ __launch_bounds__(256) void layernorm_vec_kernel(const float *__restrict__ x,
+                                                            const float *__restrict__ gamma,
+                                                            const float *__restrict__ beta,
+                                                            float *__restrict__ y, size_t rows,
+                                                            float eps) {
+    constexpr int cols = 256 * NV;
+    const size_t row = (size_t)blockIdx.x * 4 + (threadIdx.x >> 6);
+    const int lane = threadIdx.x & 63;
+    if (row >= rows)
+        return;
+    const float4 *xp = reinterpret_cast<const float4 *>(x + row * cols);
+    float4 *yp = reinterpret_cast<float4 *>(y + row * cols);
+    float4 v[NV], gm[NV], bt[NV];
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+        v[i] = xp[lane + 64 * i];
+        gm[i] = gamma ? reinterpret_cast<const float4 *>(gamma)[lane + 64 * i]
+                      : make_float4(1.f, 1.f, 1.f, 1.f);
+        bt[i] = beta ? reinterpret_cast<const float4 *>(beta)[lane + 64 * i]
+                     : make_float4(0.f, 0.f, 0.f, 0.f);
+    }
+    float s = 0.f;
+#pragma unroll
+    for (int i = 0; i < NV; ++i)
+        s += (v[i].x + v[i].y) + (v[i].z + v[i].w);
+    const float mean = wave_sum(s) / (float)cols;
+    float q = 0.f;
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+        v[i].x -= mean, v[i].y -= mean, v[i].z -= mean, v[i].w -= mean;
+        q += (v[i].x * v[i].x + v[i].y * v[i].y) + (v[i].z * v[i].z + v[i].w * v[i].w);
+    }
+    const float inv = rsqrtf(wave_sum(q) / (float)cols + eps);
+#pragma unroll
+    for (int i = 0; i < NV; ++i) {
+        float4 o;
+        o.x = v[i].x * inv * gm[i].x + bt[i].x;
+        o.y = v[i].y * inv * gm[i].y + bt[i].y;
+        o.z = v[i].z * inv * gm[i].z + bt[i].z;
+        o.w = v[i].w * inv * gm[i].w + bt[i].w;
+        yp[lane + 64 * i] = o;
+    }
+}
+
 template <bool RESIDENT>
 __global__ __launch_bounds__(256) void layernorm_kernel(const float *__restrict__ x,
                                                         const float *__restrict__ gamma,
@@ -714,6 +761,28 @@ int pet_hip_layernorm(const float *x, const float *gamma, const float *beta, flo
         return set_error(PET_HIP_ERR_INVALID, "null pointer");
     if ((rows + 3) / 4 >= (1ull << 31))
         return set_error(PET_HIP_ERR_UNSUPPORTED, "too many rows");
+    const bool aligned = ((((uintptr_t)x) | ((uintptr_t)y) | ((uintptr_t)gamma) | ((uintptr_t)beta)) & 15) == 0;
+    const dim3 grid((unsigned)((rows + 3) / 4));
+    if (aligned && cols % 256 == 0 && cols <= 2048) {
+        hipStream_t st = as_stream(stream);
+        switch (cols / 256) {
+#define PET_LN_CASE(NV)                                                                            \
+    case NV:                                                                                       \
+        hipLaunchKernelGGL(layernorm_vec_kernel<NV>, grid, dim3(256), 0, st, x, gamma, beta, y,    \
+                           rows, eps);                                                             \
+        break;
+            PET_LN_CASE(1)
+            PET_LN_CASE(2)
+            PET_LN_CASE(3)
+            PET_LN_CASE(4)
+            PET_LN_CASE(5)
+            PET_LN_CASE(6)
+            PET_LN_CASE(7)
+            PET_LN_CASE(8)
+#undef PET_LN_CASE
+        }
+        return check_launch("layernorm_vec_kernel");
+    }
     if (cols <= 64 * (size_t)kRowRegs)
         hipLaunchKernelGGL(layernorm_kernel<true>, dim3((unsigned)((rows + 3) / 4)), dim3(256), 0,
                            as_stream(stream), x, gamma, beta, y, rows, cols, eps);

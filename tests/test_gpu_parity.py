@@ -823,10 +823,10 @@ def test_activation_pool_softmax_layernorm(ops):
                                oracle.layernorm(h, g, be), rtol=1e-4, atol=1e-5)
 
 
-@pytest.mark.parametrize("cols", [1, 63, 65, 700, 2048, 2049, 5000])
+@pytest.mark.parametrize("cols", [1, 63, 65, 256, 700, 768, 1792, 2048, 2049, 5000])
 def test_softmax_layernorm_row_lengths(ops, cols):
-    """Rows up to 2048 elements live in registers, longer ones stream; ragged
-    lengths on both sides of the switch."""
+    """Rows up to 2048 elements live in registers (multiples of 256 as 16-byte words),
+    longer ones stream; ragged lengths on both sides of the switch."""
     rng = np.random.default_rng(cols)
     s = rng.standard_normal((5, cols)).astype(np.float32)
     np.testing.assert_allclose(host(ops.softmax(dev(s))), oracle.softmax(s), rtol=1e-5, atol=1e-7)
