@@ -490,6 +490,12 @@ PET_HIP_API int pet_hip_bias_act(const float *x, const float *bias, float *y, si
 PET_HIP_API int pet_hip_pool2d(const float *x, float *y, int n, int c, int h, int w, int kh, int kw,
                    int ph, int pw, int sh, int sw, int dh, int dw, int mode,
                    pet_hip_stream_t stream);
+/* The same with pet_hip_call_flags: PET_HIP_CALL_X_RELU pools max(x, 0) (the ReLU of the
+ * convolution that produced x, left to this reader; cuDNN's fused activation has no such
+ * hand-over, src/Graph/code_engine.cc:955-977 applies it in the producer). */
+PET_HIP_API int pet_hip_pool2d_ex(const float *x, float *y, int n, int c, int h, int w, int kh, int kw,
+                      int ph, int pw, int sh, int sw, int dh, int dw, int mode, unsigned flags,
+                      pet_hip_stream_t stream);
 
 /* Row softmax over the last axis of a [rows, cols] view; replaces
  * online_softmax (src/Graph/code_engine.cc:424-486, 1707-1731). */

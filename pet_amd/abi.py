@@ -91,6 +91,7 @@ SIGNATURES = {
     "pet_hip_batchnorm": [_vp] * 6 + [_sz, _sz, _sz, ctypes.c_float, _vp],
     "pet_hip_bias_act": [_vp, _vp, _vp, _sz, _sz, _sz, _i, _vp],
     "pet_hip_pool2d": [_vp, _vp] + [_i] * 13 + [_vp],
+    "pet_hip_pool2d_ex": [_vp, _vp] + [_i] * 13 + [ctypes.c_uint, _vp],
     "pet_hip_softmax": [_vp, _vp, _sz, _sz, _vp],
     "pet_hip_layernorm": [_vp, _vp, _vp, _vp, _sz, _sz, ctypes.c_float, _vp],
 }

@@ -264,7 +264,7 @@ __global__ __launch_bounds__(256) void pool2d_kernel(const float *__restrict__ x
                                                      float *__restrict__ y, int nc, int h, int w,
                                                      int kh, int kw, int ph, int pw, int sh,
                                                      int sw, int dh, int dw, int oh, int ow,
-                                                     int mode) {
+                                                     int mode, float lo) {
     size_t total = (size_t)nc * oh * ow;
     size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
     const size_t step = (size_t)gridDim.x * 256;
@@ -283,7 +283,7 @@ __global__ __launch_bounds__(256) void pool2d_kernel(const float *__restrict__ x
                 int iw = j * sw + s * dw - pw;
                 if (iw < 0 || iw >= w)
                     continue;
-                float v = xp[(size_t)ih * w + iw];
+                float v = fmaxf(xp[(size_t)ih * w + iw], lo); // lo = 0: ReLU on the way in
                 acc = mode == 0 ? fmaxf(acc, v) : acc + v;
                 ++taps;
             }
@@ -309,7 +309,7 @@ __device__ __forceinline__ float wave_max(float v) {
 // Global average pooling: one wave per (n, c) plane.
 __global__ __launch_bounds__(256) void global_avgpool_kernel(const float *__restrict__ x,
                                                              float *__restrict__ y, int nc,
-                                                             int hw) {
+                                                             int hw, float lo) {
     int plane = blockIdx.x * 4 + (threadIdx.x >> 6);
     int lane = threadIdx.x & 63;
     if (plane >= nc)
@@ -317,7 +317,7 @@ __global__ __launch_bounds__(256) void global_avgpool_kernel(const float *__rest
     const float *xp = x + (size_t)plane * hw;
     float acc = 0.f;
     for (int i = lane; i < hw; i += 64)
-        acc += xp[i];
+        acc += fmaxf(xp[i], lo);
     acc = wave_sum(acc);
     if (lane == 0)
         y[plane] = acc / (float)hw;
@@ -711,7 +711,16 @@ int pet_hip_bias_act(const float *x, const float *bias, float *y, size_t outer, 
 
 int pet_hip_pool2d(const float *x, float *y, int n, int c, int h, int w, int kh, int kw, int ph,
                    int pw, int sh, int sw, int dh, int dw, int mode, pet_hip_stream_t stream) {
+    return pet_hip_pool2d_ex(x, y, n, c, h, w, kh, kw, ph, pw, sh, sw, dh, dw, mode, 0, stream);
+}
+
+int pet_hip_pool2d_ex(const float *x, float *y, int n, int c, int h, int w, int kh, int kw, int ph,
+                      int pw, int sh, int sw, int dh, int dw, int mode, unsigned flags,
+                      pet_hip_stream_t stream) {
     PET_REQUIRE_INIT();
+    if (flags & ~(unsigned)PET_HIP_CALL_X_RELU)
+        return set_error(PET_HIP_ERR_INVALID, "pooling takes PET_HIP_CALL_X_RELU only");
+    const float lo = (flags & PET_HIP_CALL_X_RELU) ? 0.f : -INFINITY;
     if (n < 0 || c < 0 || h <= 0 || w <= 0 || kh <= 0 || kw <= 0 || sh <= 0 || sw <= 0 ||
         dh <= 0 || dw <= 0 || ph < 0 || pw < 0 || (mode != 0 && mode != 1))
         return set_error(PET_HIP_ERR_INVALID, "bad pooling arguments");
@@ -727,11 +736,11 @@ int pet_hip_pool2d(const float *x, float *y, int n, int c, int h, int w, int kh,
     if (mode == 1 && kh == h && kw == w && ph == 0 && pw == 0 && dh == 1 && dw == 1) {
         int nc = n * c;
         hipLaunchKernelGGL(global_avgpool_kernel, dim3((nc + 3) / 4), dim3(256), 0,
-                           as_stream(stream), x, y, nc, h * w);
+                           as_stream(stream), x, y, nc, h * w, lo);
         return check_launch("global_avgpool_kernel");
     }
     hipLaunchKernelGGL(pool2d_kernel, dim3(grid_for(total)), dim3(256), 0, as_stream(stream), x, y,
-                       n * c, h, w, kh, kw, ph, pw, sh, sw, dh, dw, oh, ow, mode);
+                       n * c, h, w, kh, kw, ph, pw, sh, sw, dh, dw, oh, ow, mode, lo);
     return check_launch("pool2d_kernel");
 }
 

@@ -905,6 +905,9 @@ class PoolOp : public Operator {
     Dim computeShape() override;
     double perf(PerfEngine *pe, int rounds = 200, int warmupRounds = 200) override;
     int launch(pet_hip_stream_t stream) override;
+    // flags: PET_HIP_CALL_X_RELU only (the producer's ReLU applied on the way in)
+    int launchFused(pet_hip_stream_t stream, const float *residual, ActType finalAct, float *out,
+                    unsigned flags) override;
     std::string toString() const override;
     int numInputs() override { return 1; }
     int numOutputs() override { return 1; }

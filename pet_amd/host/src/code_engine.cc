@@ -299,6 +299,8 @@ LaunchPlan planLaunchFlags(const OpVec &order, const TensorVec &graphOutputs,
                 ok = false;
             } else if (isConvOp(u) && u->getInputs()[0] == e.out && u->getInputs()[1] != e.out) {
                 want[u] |= PET_HIP_CALL_X_RELU;
+            } else if (dynamic_cast<PoolOp *>(u) != nullptr && tail == tails.atAdd.end()) {
+                want[u] |= PET_HIP_CALL_X_RELU; // pooling applies it on the way in
             } else if (tail != tails.atAdd.end() && tail->second.residual == e.out &&
                        isConvOp(tail->second.contraction) &&
                        tail->second.contraction->getInputs()[1] != e.out) {
@@ -1082,10 +1084,12 @@ std::string CodeEngine::genCode(std::shared_ptr<SubGraph> &graph) {
             int kh, kw, ph, pw, sh, sw, dh, dw;
             std::tie(kh, kw, ph, pw, sh, sw, dh, dw) = pool->getArgs();
             auto d = op->getInputs()[0]->getDims();
-            c << "pet_hip_pool2d(" << in(0) << ", " << out(0) << ", " << d[0] << ", " << d[1]
-              << ", " << d[2] << ", " << d[3] << ", " << kh << ", " << kw << ", " << ph << ", "
-              << pw << ", " << sh << ", " << sw << ", " << dh << ", " << dw << ", "
-              << (op->getType() == Operator::MaxPool ? 0 : 1) << ", s)";
+            const unsigned fl = flagsOf(op);
+            c << (fl ? "pet_hip_pool2d_ex(" : "pet_hip_pool2d(") << in(0) << ", " << out(0) << ", "
+              << d[0] << ", " << d[1] << ", " << d[2] << ", " << d[3] << ", " << kh << ", " << kw
+              << ", " << ph << ", " << pw << ", " << sh << ", " << sw << ", " << dh << ", " << dw
+              << ", " << (op->getType() == Operator::MaxPool ? 0 : 1)
+              << (fl ? ", " + std::to_string(fl) + "u" : std::string()) << ", s)";
         } else if (dynamic_cast<SoftmaxOp *>(op)) {
             size_t cols = (size_t)op->getInputs()[0]->getDims().back();
             c << "pet_hip_softmax(" << in(0) << ", " << out(0) << ", "

@@ -1804,6 +1804,15 @@ int PoolOp::launch(pet_hip_stream_t stream) {
                           in[3], kh, kw, ph, pw, sh, sw, dh, dw, type == MaxPool ? 0 : 1, stream);
 }
 
+int PoolOp::launchFused(pet_hip_stream_t stream, const float *residual, ActType finalAct,
+                        float *out, unsigned flags) {
+    if (residual != nullptr || finalAct != None)
+        return PET_HIP_ERR_INVALID;
+    const Dim &in = inputs[0]->getDims();
+    return pet_hip_pool2d_ex(inputs[0]->devicePtr(), out, in[0], in[1], in[2], in[3], kh, kw, ph,
+                             pw, sh, sw, dh, dw, type == MaxPool ? 0 : 1, flags, stream);
+}
+
 double PoolOp::perf(PerfEngine *pe, int rounds, int warmupRounds) {
     PoolArgs args = getArgs();
     if (pe && pe->checkOpPerf(type, args))

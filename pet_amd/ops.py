@@ -536,15 +536,16 @@ def bias_act(x, bias, act="none", ch_axis=1, out=None):
     return out
 
 
-def pool2d(x, kh, kw, ph, pw, sh, sw, dh=1, dw=1, mode="max", out=None):
+def pool2d(x, kh, kw, ph, pw, sh, sw, dh=1, dw=1, mode="max", out=None, flags=0):
+    """flags: abi.X_RELU pools max(x, 0)."""
     _chk(x, out)
     n, c, h, w = x.shape
     oh = (h + 2 * ph - dh * (kh - 1) - 1) // sh + 1
     ow = (w + 2 * pw - dw * (kw - 1) - 1) // sw + 1
     if out is None:
         out = torch.empty((n, c, oh, ow), device=x.device, dtype=torch.float32)
-    abi.call("pet_hip_pool2d", _ptr(x), _ptr(out), n, c, h, w, kh, kw, ph, pw, sh, sw, dh, dw,
-             0 if mode == "max" else 1, _stream())
+    abi.call("pet_hip_pool2d_ex", _ptr(x), _ptr(out), n, c, h, w, kh, kw, ph, pw, sh, sw, dh, dw,
+             0 if mode == "max" else 1, flags, _stream())
     return out
 
 

@@ -823,6 +823,21 @@ def test_activation_pool_softmax_layernorm(ops):
                                oracle.layernorm(h, g, be), rtol=1e-4, atol=1e-5)
 
 
+def test_pooling_applies_a_deferred_relu_on_load(ops):
+    """pet_hip_pool2d_ex with PET_HIP_CALL_X_RELU: max / average pooling of max(x, 0), for a
+    producer that left its ReLU to this reader; bit-equal to ReLU followed by pooling."""
+    from pet_amd import abi
+    rng = np.random.default_rng(77)
+    x = rng.standard_normal((2, 5, 13, 11)).astype(np.float32)
+    relu = np.maximum(x, 0)
+    for mode, args in (("max", (3, 3, 1, 1, 2, 2)), ("avg", (2, 3, 1, 0, 1, 2)),
+                       ("avg", (13, 11, 0, 0, 1, 1))):  # the last one is global pooling
+        want = host(ops.pool2d(dev(relu), *args, mode=mode))
+        got = host(ops.pool2d(dev(x), *args, mode=mode, flags=abi.X_RELU))
+        np.testing.assert_array_equal(got, want)
+        np.testing.assert_allclose(want, oracle.pool2d(relu, *args, mode=mode), rtol=1e-6, atol=1e-7)
+
+
 @pytest.mark.parametrize("cols", [1, 63, 65, 256, 700, 768, 1792, 2048, 2049, 5000])
 def test_softmax_layernorm_row_lengths(ops, cols):
     """Rows up to 2048 elements live in registers (multiples of 256 as 16-byte words),
