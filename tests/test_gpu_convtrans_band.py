@@ -47,6 +47,10 @@ CONV_TRANS_CASES = [
     (1, 6, 6, 4, 3, 3, 4, 1, 1, 2, 2, 2, 2, 0, 0),       # dilated taps, as the loop nest reads
     (4, 16, 16, 64, 4, 4, 33, 1, 1, 2, 2, 1, 1, 0, 0),   # several pixel tiles per phase
     (16, 7, 7, 128, 4, 4, 64, 1, 1, 2, 2, 1, 1, 0, 0),   # a DCGAN / InfoGAN generator layer
+    # few pixels, many features: the waves of a workgroup share the feature axis
+    (1, 2, 2, 448, 4, 4, 256, 0, 0, 1, 1, 1, 1, 0, 0),   # src/Test/transposeconv_test_1.cc
+    (1, 3, 3, 68, 3, 3, 40, 1, 1, 2, 2, 1, 1, 0, 0),     # the same without 16-byte loads
+    (2, 5, 4, 96, 3, 3, 33, 1, 1, 2, 2, 1, 1, 1, 0),     # ragged pixel and channel tiles
 ]
 
 
@@ -73,6 +77,13 @@ def test_conv_trans_bias_and_activation(ops):
     x = rng.integers(-3, 4, (2, 4, 4, 8)).astype(np.float32)
     K = rng.integers(-3, 4, (4, 4, 8, 6)).astype(np.float32)
     b = rng.integers(-3, 4, 6).astype(np.float32)
+    want = np.maximum(oracle.conv_trans(x, K, 1, 1, 2, 2) + b, 0)
+    got = host(ops.conv_trans(dev(x), dev(K), 1, 1, 2, 2, bias=dev(b), act="relu"))
+    np.testing.assert_array_equal(got, want)
+    # the form in which waves share the feature axis has its own epilogue
+    x = rng.integers(-3, 4, (1, 3, 3, 128)).astype(np.float32)
+    K = rng.integers(-3, 4, (3, 3, 128, 37)).astype(np.float32)
+    b = rng.integers(-3, 4, 37).astype(np.float32)
     want = np.maximum(oracle.conv_trans(x, K, 1, 1, 2, 2) + b, 0)
     got = host(ops.conv_trans(dev(x), dev(K), 1, 1, 2, 2, bias=dev(b), act="relu"))
     np.testing.assert_array_equal(got, want)
