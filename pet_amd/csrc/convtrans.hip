@@ -13,6 +13,7 @@
 // one pixel (16-byte loads along f) and one channel (coalesced dword loads across lanes);
 // no LDS staging. A wave owns 32 pixels x 32*TN channels, a workgroup four pixel tiles.
 #include "mfma_common.h"
+#include <algorithm>
 #include <type_traits>
 
 using namespace pet;
@@ -28,6 +29,8 @@ struct ConvTransParams {
     int OH, OW;
     int ah, aw; // taps rr > R - ah (ss > S - aw) are left out, as the reference does
     int PT, KW; // pixel tiles and feature shares per workgroup
+    int nfast;  // pixel numbering, see the kernel
+    int KS;     // workgroups sharing a tile's taps (their sums meet in y as float atomics)
     int act;
 };
 
@@ -50,7 +53,8 @@ __global__ __launch_bounds__(SPLIT ? 1024 : 256) void conv_trans_kernel(ConvTran
     const int OHq = qh < p.OH ? (p.OH - qh + p.sh - 1) / p.sh : 0;
     const int OWq = qw < p.OW ? (p.OW - qw + p.sw - 1) / p.sw : 0;
     const int npix = p.N * OHq * OWq;
-    const int pix0 = (blockIdx.x * p.PT + pt) * 32;
+    const int ks = SPLIT ? (int)(blockIdx.x % (unsigned)p.KS) : 0; // this workgroup's taps
+    const int pix0 = ((SPLIT ? blockIdx.x / (unsigned)p.KS : blockIdx.x) * p.PT + pt) * 32;
     const bool active = pix0 < npix;
     if (!SPLIT && !active)
         return;
@@ -59,8 +63,11 @@ __global__ __launch_bounds__(SPLIT ? 1024 : 256) void conv_trans_kernel(ConvTran
     // this lane's pixel (rows past the end repeat the last pixel and are not stored)
     const int pix = max(min(pix0 + l32, npix - 1), 0);
     const int plane = max(OHq * OWq, 1);
-    const int n = pix / plane;
-    const int rem = pix - n * plane;
+    // pixels of a phase are numbered image-major, or (nfast) with the image number running
+    // fastest: with 32 images or more the lanes of a tile then sit at one output position and
+    // agree on which taps reach the input at all
+    const int n = p.nfast ? pix % p.N : pix / plane;
+    const int rem = p.nfast ? pix / p.N : pix - n * plane;
     const int pi = rem / max(OWq, 1), pj = rem - pi * max(OWq, 1);
     const int ybase = pix0 + l32 < npix
                           ? ((n * p.OH + qh + pi * p.sh) * p.OW + qw + pj * p.sw) * p.C
@@ -93,13 +100,18 @@ __global__ __launch_bounds__(SPLIT ? 1024 : 256) void conv_trans_kernel(ConvTran
             continue;
         const int ih = th / p.sh + pi;
         for (int ss = 0; ss < p.S; ++ss) {
-            if (p.S - p.aw < ss)
+            // (every sh-th row and sw-th column of taps reaches a phase: numbering them by
+            // rr / sh and ss / sw deals a phase's taps evenly)
+            if (p.S - p.aw < ss ||
+                (SPLIT && ((rr / p.sh) * ((p.S + p.sw - 1) / p.sw) + ss / p.sw) % p.KS != ks))
                 continue;
             const int tw = qw + ss * p.dw - (p.S - p.pw - 1);
             if (tw % p.sw != 0)
                 continue;
             const int iw = tw / p.sw + pj;
             const bool inside = ih >= 0 && ih < p.H && iw >= 0 && iw < p.W;
+            if (__builtin_amdgcn_ballot_w64(inside) == 0)
+                continue; // no lane of the wave has an input pixel under this tap
             const float *xp =
                 p.x + (size_t)((n * p.H + (inside ? ih : 0)) * p.W + (inside ? iw : 0)) * p.F;
             const float *wp = p.w + (size_t)((p.R - 1 - rr) * p.S + (p.S - 1 - ss)) * p.F * p.C;
@@ -110,9 +122,11 @@ __global__ __launch_bounds__(SPLIT ? 1024 : 256) void conv_trans_kernel(ConvTran
 #pragma unroll
                 for (int u = 0; u < U; ++u) {
                     const int fk = (ch + u) * 8 + hk * 4; // this half-wave's four k values
+                    // VEC: F is a multiple of 4, so the four are all inside or all outside
+                    const bool fin = fk < p.F;
                     if (VEC) {
-                        float4 v = inside ? *reinterpret_cast<const float4 *>(xp + fk)
-                                          : make_float4(0.f, 0.f, 0.f, 0.f);
+                        float4 v = inside && fin ? *reinterpret_cast<const float4 *>(xp + fk)
+                                                 : make_float4(0.f, 0.f, 0.f, 0.f);
                         a[u][0] = v.x;
                         a[u][1] = v.y;
                         a[u][2] = v.z;
@@ -126,7 +140,7 @@ __global__ __launch_bounds__(SPLIT ? 1024 : 256) void conv_trans_kernel(ConvTran
                     for (int j = 0; j < 4; ++j)
 #pragma unroll
                         for (int tn = 0; tn < TN; ++tn) {
-                            const bool ok = cok[tn] && (VEC || fk + j < p.F);
+                            const bool ok = cok[tn] && (VEC ? fin : fk + j < p.F);
                             b[u][tn][j] = ok ? wp[(size_t)(fk + j) * p.C + cc[tn]] : 0.f;
                         }
                 }
@@ -196,6 +210,10 @@ __global__ __launch_bounds__(SPLIT ? 1024 : 256) void conv_trans_kernel(ConvTran
         if (yo < 0 || c0 + j >= p.C)
             continue;
         float v = tile[e];
+        if (p.KS > 1) { // y holds the bias already; the activation follows in a launch of its own
+            unsafeAtomicAdd(p.y + (size_t)yo + c0 + j, v);
+            continue;
+        }
         if (p.bias)
             v += p.bias[c0 + j];
         p.y[(size_t)yo + c0 + j] = apply_act(v, p.act);
@@ -243,6 +261,7 @@ int pet_hip_conv_trans_f32(const float *x, const float *w, const float *bias, fl
     p.ah = (h + 2 * ph - r) % sh;
     p.aw = (wd + 2 * pw - s) % sw;
     p.act = act;
+    p.nfast = n >= 32;
     if (p.OH <= 0 || p.OW <= 0)
         return set_error(PET_HIP_ERR_INVALID, "conv_trans: empty output %d x %d", p.OH, p.OW);
     const long long xin = (long long)n * h * wd * f, yout = (long long)n * p.OH * p.OW * c,
@@ -270,12 +289,29 @@ int pet_hip_conv_trans_f32(const float *x, const float *w, const float *bias, fl
     const bool split = p.KW > 1;
     if (!split)
         p.PT = 4;
-    dim3 grid((unsigned)((tiles + p.PT - 1) / p.PT), (unsigned)((c + 32 * tn - 1) / (32 * tn)),
-              (unsigned)(sh * sw));
+    // still far from a wave per SIMD (2x2 pixels, 448 features): the taps are dealt to KS
+    // workgroups as well, whose sums meet in y as float atomics: y is initialised with the
+    // bias before and activated after. Not in reproducible mode.
+    p.KS = 1;
+    if (split && !deterministic()) {
+        const long long now = waves * p.KW;
+        const int taps = ((r + sh - 1) / sh) * ((s + sw - 1) / sw); // per phase
+        int ks = (int)std::min<long long>((1024 + now - 1) / now, 16);
+        ks = std::min(ks, taps / 2);
+        if (ks >= 2)
+            p.KS = ks;
+    }
+    dim3 grid((unsigned)((tiles + p.PT - 1) / p.PT) * (unsigned)p.KS,
+              (unsigned)((c + 32 * tn - 1) / (32 * tn)), (unsigned)(sh * sw));
     if (grid.y > 65535)
         return set_error(PET_HIP_ERR_UNSUPPORTED, "conv_trans: %d output channels", c);
-    const bool vec = f % 8 == 0 && ((uintptr_t)x & 15) == 0;
+    const bool vec = f % 4 == 0 && ((uintptr_t)x & 15) == 0;
     hipStream_t st = as_stream(stream);
+    if (p.KS > 1) {
+        pet_hip_fill fill{y, bias, (size_t)n * p.OH * p.OW, (size_t)c, 1};
+        if (int rc = pet_hip_bias_fill_batch(&fill, 1, stream))
+            return rc;
+    }
     const dim3 block(64u * p.PT * p.KW);
     const size_t lds = split ? sizeof(float) * p.PT * (32 * 32 * tn + 32) : 0;
     auto launch = [&](auto tn_, auto vec_) {
@@ -292,7 +328,11 @@ int pet_hip_conv_trans_f32(const float *x, const float *w, const float *bias, fl
         vec ? launch(two{}, std::true_type{}) : launch(two{}, std::false_type{});
     else
         vec ? launch(one{}, std::true_type{}) : launch(one{}, std::false_type{});
-    return check_launch("conv_trans_kernel");
+    if (int rc = check_launch("conv_trans_kernel"))
+        return rc;
+    if (p.KS > 1 && act != PET_HIP_ACT_NONE)
+        return pet_hip_activation(y, y, (size_t)yout, act, stream);
+    return PET_HIP_OK;
 }
 
 } // extern "C"

@@ -51,6 +51,9 @@ CONV_TRANS_CASES = [
     (1, 2, 2, 448, 4, 4, 256, 0, 0, 1, 1, 1, 1, 0, 0),   # src/Test/transposeconv_test_1.cc
     (1, 3, 3, 68, 3, 3, 40, 1, 1, 2, 2, 1, 1, 0, 0),     # the same without 16-byte loads
     (2, 5, 4, 96, 3, 3, 33, 1, 1, 2, 2, 1, 1, 1, 0),     # ragged pixel and channel tiles
+    # 32 images or more: pixels numbered with the image fastest, taps skipped per wave
+    (64, 1, 1, 100, 4, 4, 48, 0, 0, 1, 1, 1, 1, 0, 0),   # a generator's first layer (z = 100)
+    (37, 3, 2, 12, 3, 3, 5, 1, 0, 2, 1, 1, 1, 0, 0),
 ]
 
 
