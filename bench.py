@@ -405,6 +405,18 @@ def main():
                     entry[label + "_error"] = str(exc)[:200]
             if entry.get("pet_ms"):
                 entry["pet_TFLOP/s"] = gflop / entry["pet_ms"]
+            if name.startswith("c1"):
+                # a graph of one 7 us kernel mostly measures the replay's own launch cost:
+                # the same convolution launched on the stream, 50 in a row
+                try:
+                    ns, table = programs.GpuNS(keep=False), {}
+                    with torch.cuda.stream(stream):
+                        run(ns, params, False, T=table)
+                    entry["original_stream_launch_ms"] = time_kernel(
+                        lambda: run(ns, params, False, T=table))
+                    del ns, table
+                except Exception as exc:
+                    entry["original_stream_launch_error"] = str(exc)[:200]
             other[name] = entry
 
     # ---- every distinct contraction of the other configurations by itself: 20 launches
