@@ -116,8 +116,11 @@ int main(int argc, char **argv) {
             }
             else if (auto c3 = dynamic_cast<Conv3dOp *>(op))
                 tuned += c3->getAlgo() != 0;
-            else if (auto mm = dynamic_cast<MatmulOp *>(op))
+            else if (auto mm = dynamic_cast<MatmulOp *>(op)) {
                 tuned += mm->getAlgo() != 0;
+                if (mm->getAlgo() != 0 && getenv("PET_HOST_TRACE"))
+                    std::fprintf(stderr, "algo %d: %s\n", mm->getAlgo(), op->toString().c_str());
+            }
     }
     auto exec = ce.instantiate(sg);
     if (!exec) {
