@@ -36,6 +36,19 @@
  *       identity statistics (mean 0, var 1 - eps, scale 1, bias 0 -> y = x).
  *   trans_chain : numpy constructions of halo split / drop fuse / pad fuse /
  *       extr split on iota inputs, and conv equivalence (split+conv+fuse == conv).
+ *   conv_trans : the golden vectors of the reference's own tests
+ *       (src/Test/convtrans_test_1.cc:62-77, 120-135, convtrans_test_2.cc:81-82, 144-145),
+ *       reproduced exactly; torch.nn.functional.conv_transpose2d (CPU) on strided, padded
+ *       and output-padded shapes; the tap skip of src/Graph/operator.cc:957-960 as torch's
+ *       result on a kernel with the skipped rows zeroed. With dilation != 1 the reference's
+ *       loop keeps the undilated offset r - ph - 1 (:961-962) and is an operator of its
+ *       own: parity unpinned for dilated transposed convolution.
+ *   g2bmm, gbmml : band products cut out of numpy's dense matmul, from the definitions
+ *       of src/nnet/iterator_table.cc:596-630. The reference has no CPU compute for them
+ *       (src/Graph/operator.cc:1424-1598 are shape rules): parity unpinned by it; on a GPU
+ *       box the reference's nnet::Interpreter evaluates the same definitions.
+ *   expr (MemBound programs) : numpy index maps, gathers and sums; on a GPU box the
+ *       reference's nnet::Interpreter, compiled unchanged, on the same expressions.
  *   relu/sigmoid/tanh/gelu, bias_act, maxpool, avgpool, softmax, layernorm :
  *       parity unpinned by the reference (ActivationOp / MaxPoolOp / AvgPoolOp /
  *       SoftmaxOp::compute are assert(false), include/operator.h:1968-1977,

@@ -3,7 +3,8 @@
 Inputs are small integers (every contraction below stays exact in fp32), expected
 outputs come from routines that share no code with the oracle or the HIP library:
 torch's CPU convolutions and numpy's matmul / reshape / transpose / pad / split /
-concatenate / tile / take / mean and integer powers. The transposes are the reference's own closed form
+concatenate / tile / take / mean and integer powers, torch's conv_transpose2d, and band
+products cut out of numpy's dense matmul. The transposes are the reference's own closed form
 (reshape -> transpose -> reshape, src/Test/dat/transpose_test/transpose_ops.op:1-3
 and src/Test/transpose_test_2.py:4-31) on an iota input (src/Test/transpose_test_2.cc:24);
 the matmul triple is the reference's batch-GEMM merge case
@@ -102,6 +103,44 @@ def main():
     r = ints((2, 8, 4))
     out["rm_x"] = r
     out["rm_axis1"], out["rm_axis2"] = r.mean(axis=1, keepdims=True), r.mean(axis=2, keepdims=True)
+    # ---- transposed convolution (x NHWF, w RSFC, y NHWC) against torch's conv_transpose2d,
+    # which takes NCHW input and [in, out, kh, kw] filters. Dilation 1 only: with dilation the
+    # reference's loop nest (src/Graph/operator.cc:961-962) keeps the undilated offset
+    # r - ph - 1 and is an operator of its own, which no library routine restates.
+    # (n, h, w, f, r, s, c, ph, pw, sh, sw, dh, dw, oph, opw)
+    conv_trans = [
+        (1, 4, 5, 3, 3, 3, 4, 1, 1, 2, 2, 1, 1, 0, 0),
+        (2, 3, 3, 8, 4, 4, 5, 1, 1, 2, 2, 1, 1, 1, 1),
+        (1, 5, 4, 2, 3, 2, 3, 0, 1, 1, 1, 1, 1, 0, 0),
+    ]
+    for i, cs in enumerate(conv_trans):
+        n, h, w, f, r, s, c, ph, pw, sh, sw, dh, dw, oph, opw = cs
+        x, wt = ints((n, h, w, f)), ints((r, s, f, c))
+        y = F.conv_transpose2d(torch.from_numpy(x).double().permute(0, 3, 1, 2),
+                               torch.from_numpy(wt).double().permute(2, 3, 0, 1),
+                               stride=(sh, sw), padding=(ph, pw), output_padding=(oph, opw),
+                               dilation=(dh, dw)).permute(0, 2, 3, 1).contiguous().numpy()
+        out[f"convtrans_{i}_args"] = np.array(cs, np.int32)
+        out[f"convtrans_{i}_x"], out[f"convtrans_{i}_w"] = x, wt
+        out[f"convtrans_{i}_y"] = y.astype(np.float32)
+    # ---- band matmuls from the dense product: G2BMM[b,i,j] = (A B^T)[b, i, i + d (j - w)],
+    # GBMML[b,i,:] = sum_j band[b,i,j] B[b, i + d (j - w), :], rows outside the matrix are zero
+    # (bs, m, k, w, d)
+    for i, (bs, m, k, w, d) in enumerate([(2, 11, 6, 2, 1), (1, 13, 8, 3, 2), (2, 40, 32, 5, 3)]):
+        A, B = ints((bs, m, k)), ints((bs, m, k))
+        dense = np.matmul(A, B.transpose(0, 2, 1))
+        band = np.zeros((bs, m, 2 * w + 1), np.float32)
+        P = ints((bs, m, 2 * w + 1))
+        ctx = np.zeros((bs, m, k), np.float32)
+        for r_ in range(m):
+            for j in range(2 * w + 1):
+                col = r_ + d * (j - w)
+                if 0 <= col < m:
+                    band[:, r_, j] = dense[:, r_, col]
+                    ctx[:, r_, :] += P[:, r_, j:j + 1] * B[:, col, :]
+        out[f"band_{i}_args"] = np.array([bs, m, k, w, d], np.int32)
+        out[f"band_{i}_A"], out[f"band_{i}_B"], out[f"band_{i}_g2bmm"] = A, B, band
+        out[f"band_{i}_P"], out[f"band_{i}_gbmml"] = P, ctx
     np.savez_compressed(os.path.join(HERE, "golden.npz"), **out)
     print("wrote", os.path.join(HERE, "golden.npz"), len(out), "arrays")
 

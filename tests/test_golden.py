@@ -111,6 +111,17 @@ def check_all(be):
     r = be.put(G["rm_x"])
     eq(be.get(be.reduce_mean(r, 1)), G["rm_axis1"])
     eq(be.get(be.reduce_mean(r, 2)), G["rm_axis2"])
+    # transposed convolution (torch's conv_transpose2d) and the band matmuls (dense numpy)
+    for i in range(3):
+        n, h, w, f, r_, s, c, ph, pw, sh, sw, dh, dw, oph, opw = (
+            int(v) for v in G[f"convtrans_{i}_args"])
+        y = be.get(be.conv_trans(be.put(G[f"convtrans_{i}_x"]), be.put(G[f"convtrans_{i}_w"]),
+                                 ph, pw, sh, sw, dh, dw, oph, opw))
+        eq(y, G[f"convtrans_{i}_y"])
+        bs, m, k, w_, d = (int(v) for v in G[f"band_{i}_args"])
+        A, B, P = (be.put(G[f"band_{i}_{k_}"]) for k_ in ("A", "B", "P"))
+        eq(be.get(be.g2bmm(A, B, w_, d)), G[f"band_{i}_g2bmm"])
+        eq(be.get(be.gbmml(P, B, d)), G[f"band_{i}_gbmml"])
 
 
 def test_oracle_reproduces_golden_vectors():
