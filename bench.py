@@ -508,7 +508,8 @@ def main():
         # plain, and with --tune: Operator::perf on every operator first, so that each
         # contraction runs with the algorithm that timed fastest for it (what PET's search
         # leaves in its PerfEngine)
-        for model in ("dilated:pet", "dilated", "resnet18", "bert", "bert:pet", "resnet3d18"):
+        for model in ("dilated:pet", "dilated", "resnet18", "resnet18:pet", "bert", "bert:pet",
+                      "resnet3d18"):
             for key, extra in ((model, []), (model + " tuned", ["--tune"])):
                 try:
                     res = subprocess.run([run_model, model, "--rounds", str(max(50, args.steps)),

@@ -25,7 +25,7 @@ struct Model {
 // (src/nnet/nmutator.cc:529-567 of the reference).
 Model dilatedBlock(bool spaceToBatch, int hw = 64,
                    std::vector<int> channels = {512, 512, 512, 512, 256, 128, 64}, int d = 2);
-Model resnet18(int hw = 224, int width = 64, int classes = 1000);
+Model resnet18(int hw = 224, int width = 64, int classes = 1000, bool mergedShortcut = false);
 Model bertBase(int layers = 12, int seq = 128, int hidden = 768, int heads = 12, int ffn = 3072,
                bool mergedQkv = false);
 Model resnet3d18(int t = 16, int hw = 112, int width = 64, int classes = 400);

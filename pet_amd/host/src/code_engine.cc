@@ -502,8 +502,67 @@ static std::set<const Operator *> planSharedLhs(const OpVec &order, const Tensor
     return skipped;
 }
 
+// A Split along `dim` cuts a tensor into contiguous slabs when every dim before it has extent
+// 1 (dim 0 always; the channel dim of a batch-1 NCHW tensor).
+static bool splitsIntoSlabs(const Operator *op) {
+    if (op->getType() != Operator::Split)
+        return false;
+    const int dim = static_cast<const SplitOp *>(op)->getDim();
+    const Dim &d = op->getInputs()[0]->getDims();
+    for (int i = 0; i < dim && i < (int)d.size(); ++i)
+        if (d[i] != 1)
+            return false;
+    return true;
+}
+
+// A ReLU whose input does not come straight from a contraction (those ride in the
+// contraction's epilogue, planFusedTails) and whose result only convolutions and poolings read
+// as their input is left to those readers (PET_HIP_CALL_X_RELU): the activation does not run
+// and its output shares its input's storage. PET's merge of a block's first convolution with
+// its 1x1 shortcut produces this: Conv (both filter banks) -> Split -> ReLU on the first half.
+struct ReluIntoReaders {
+    std::set<const Operator *> folded;
+    std::map<const Operator *, unsigned> flags;
+};
+
+static ReluIntoReaders planReluIntoReaders(const OpVec &order, const TensorVec &graphOutputs,
+                                           const std::set<const Operator *> &skipped) {
+    ReluIntoReaders plan;
+    static const bool off = getenv("PET_HOST_NO_LAUNCH_FUSION") != nullptr;
+    if (off)
+        return plan;
+    for (auto op : order) {
+        auto act = dynamic_cast<ActivationOp *>(op);
+        if (act == nullptr || act->getActType() != Operator::Relu || skipped.count(op) ||
+            weightOnly(op))
+            continue;
+        Tensor *in = op->getInputs()[0], *out = op->getOutputs()[0];
+        Operator *prod = in->getOutputOf();
+        if (prod != nullptr && prod->canTakeResidual())
+            continue;
+        if (std::find(graphOutputs.begin(), graphOutputs.end(), out) != graphOutputs.end() ||
+            out->getInputOf().empty())
+            continue;
+        bool ok = true;
+        for (auto u : out->getInputOf()) {
+            const bool conv = u->getType() == Operator::Conv || u->getType() == Operator::Conv3d;
+            const bool pool = dynamic_cast<PoolOp *>(u) != nullptr;
+            if (skipped.count(u) || weightOnly(u) || !(conv || pool) || u->getInputs()[0] != out ||
+                (conv && u->getInputs()[1] == out))
+                ok = false;
+        }
+        if (!ok)
+            continue;
+        plan.folded.insert(op);
+        for (auto u : out->getInputOf())
+            plan.flags[u] |= PET_HIP_CALL_X_RELU;
+    }
+    return plan;
+}
+
 // Storage sharing, decided before anything is captured:
-//  * Split on dim 0: every output is a slab of the input buffer.
+//  * Split on dim 0 (or on a dim behind dims of extent 1 only): every output is a slab of
+//    the input buffer.
 //  * Concat on dim 0: every input that an operator of this graph produces (and
 //    that is used nowhere else in a conflicting way) is produced directly
 //    into its slab of the output buffer.
@@ -516,7 +575,7 @@ static AliasPlan planAliases(const OpVec &order, const std::set<const Operator *
     // buffer (into a concat's output) would leave those views on freed memory
     std::set<const Tensor *> bases;
     for (auto op : order) {
-        if (op->getType() == Operator::Split && static_cast<SplitOp *>(op)->getDim() == 0) {
+        if (splitsIntoSlabs(op)) {
             Tensor *in = op->getInputs()[0];
             bases.insert(in);
             float *base = in->devicePtr();
@@ -621,10 +680,16 @@ std::unique_ptr<GraphExec> CodeEngine::instantiate(std::shared_ptr<SubGraph> &gr
                                           return f.residual->devicePtr() != f.out->devicePtr();
                                       }); // asked for tails with a residual only
     FusedAttentions att = planAttention(order, graph->getOutputs(), plan.skipped, rows);
+    ReluIntoReaders relus = planReluIntoReaders(order, graph->getOutputs(), plan.skipped);
+    for (auto op : relus.folded) // the readers read the ReLU's input
+        op->getOutputs()[0]->aliasDevice(op->getInputs()[0]->devicePtr());
     std::set<const Operator *> inert = rows.folded; // operators that do not launch by themselves
     inert.insert(att.absorbed.begin(), att.absorbed.end());
+    inert.insert(relus.folded.begin(), relus.folded.end());
     LaunchPlan lp = planLaunchFlags(order, graph->getOutputs(), plan.skipped, inert, tails,
                                     [](const Tensor *) { return true; });
+    for (auto &f : relus.flags)
+        lp.flags[f.first] |= f.second;
     auto flagsOf = [&](const Operator *op) {
         auto it = lp.flags.find(op);
         return it == lp.flags.end() ? 0u : it->second;
@@ -686,7 +751,8 @@ std::unique_ptr<GraphExec> CodeEngine::instantiate(std::shared_ptr<SubGraph> &gr
         }
         if (weightOnly(op))
             continue;
-        if (rows.folded.count(op) || tails.absorbed.count(op) || att.absorbed.count(op)) {
+        if (rows.folded.count(op) || tails.absorbed.count(op) || att.absorbed.count(op) ||
+            relus.folded.count(op)) {
             exec->nFoldedOps++;
             continue;
         }
@@ -713,7 +779,8 @@ std::unique_ptr<GraphExec> CodeEngine::instantiate(std::shared_ptr<SubGraph> &gr
             auto tail = tails.atAdd.find(prod);
             if (tail != tails.atAdd.end() && tail->second.out != t)
                 inside = true;
-            if (inside || lp.preAct.count(t) || att.absorbed.count(prod) || stacked.count(prod))
+            if (inside || lp.preAct.count(t) || att.absorbed.count(prod) || stacked.count(prod) ||
+                relus.folded.count(prod))
                 continue; // not there, or there without its ReLU
             t->deviceWritten();
             t->setComputed();
@@ -789,17 +856,24 @@ std::string CodeEngine::genCode(std::shared_ptr<SubGraph> &graph) {
                 all.push_back(t);
     }
     std::set<const Tensor *> viewOf, viewBase;
+    // the buffer a view lives in (views of views resolve to the allocation at the bottom)
+    std::map<const Tensor *, const Tensor *> bufferOf;
+    auto buffer = [&](const Tensor *t) {
+        auto it = bufferOf.find(t);
+        return it == bufferOf.end() ? t : it->second;
+    };
     std::set<const Operator *> skipped = planSharedLhs(order, graph->getOutputs());
     // storage sharing, mirrored from instantiate(): split / concat on dim 0, reshape
     std::vector<std::string> aliasLines;
     for (auto op : order) {
-        if (op->getType() == Operator::Split && static_cast<SplitOp *>(op)->getDim() == 0) {
+        if (splitsIntoSlabs(op)) {
             size_t off = 0;
             viewBase.insert(op->getInputs()[0]);
             for (auto out : op->getOutputs()) {
                 aliasLines.push_back("    float *" + e.name(out) + " = " +
                                      e.name(op->getInputs()[0]) + " + " + std::to_string(off) + ";");
                 viewOf.insert(out);
+                bufferOf[out] = buffer(op->getInputs()[0]);
                 off += out->size();
             }
             skipped.insert(op);
@@ -807,6 +881,7 @@ std::string CodeEngine::genCode(std::shared_ptr<SubGraph> &graph) {
             aliasLines.push_back("    float *" + e.name(op->getOutputs()[0]) + " = " +
                                  e.name(op->getInputs()[0]) + ";");
             viewOf.insert(op->getOutputs()[0]);
+            bufferOf[op->getOutputs()[0]] = buffer(op->getInputs()[0]);
             viewBase.insert(op->getInputs()[0]);
             skipped.insert(op);
         }
@@ -828,10 +903,22 @@ std::string CodeEngine::genCode(std::shared_ptr<SubGraph> &graph) {
             aliasLines.push_back("    float *" + e.name(in) + " = " + e.name(op->getOutputs()[0]) +
                                  " + " + std::to_string(off) + ";");
             viewOf.insert(in);
+            bufferOf[in] = buffer(op->getOutputs()[0]);
             off += in->size();
         }
         skipped.insert(op);
     }
+    // a ReLU left to the convolutions that read it: its output is its input
+    ReluIntoReaders relus = planReluIntoReaders(order, graph->getOutputs(), skipped);
+    for (auto op : order)
+        if (relus.folded.count(op)) {
+            aliasLines.push_back("    float *" + e.name(op->getOutputs()[0]) + " = " +
+                                 e.name(op->getInputs()[0]) + ";");
+            viewOf.insert(op->getOutputs()[0]);
+            bufferOf[op->getOutputs()[0]] = buffer(op->getInputs()[0]);
+            viewBase.insert(op->getInputs()[0]);
+            skipped.insert(op);
+        }
     TransposeChains rows = planTransposeChains(order, graph->getOutputs(), skipped);
     uint64_t seed = 1;
     for (auto t : all) {
@@ -853,13 +940,15 @@ std::string CodeEngine::genCode(std::shared_ptr<SubGraph> &graph) {
 
     std::map<const Operator *, std::string> packedName; // Conv3d -> its kt-major filter copy
     FusedTails tails = planFusedTails(order, graph->getOutputs(), skipped, [&](const FusedTail &f) {
-        return !viewOf.count(f.residual) && !viewOf.count(f.out);
+        return buffer(f.residual) != buffer(f.out); // as instantiate(): different storage
     });
     FusedAttentions att = planAttention(order, graph->getOutputs(), skipped, rows);
     std::set<const Operator *> inert = rows.folded;
     inert.insert(att.absorbed.begin(), att.absorbed.end());
     LaunchPlan lp = planLaunchFlags(order, graph->getOutputs(), skipped, inert, tails,
                                     [](const Tensor *) { return true; });
+    for (auto &f : relus.flags)
+        lp.flags[f.first] |= f.second;
     auto flagsOf = [&](const Operator *op) {
         auto it = lp.flags.find(op);
         return it == lp.flags.end() ? 0u : it->second;

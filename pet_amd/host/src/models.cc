@@ -92,7 +92,7 @@ Model dilatedBlock(bool spaceToBatch, int hw, std::vector<int> channels, int d) 
     return finish("dilated:pet", std::move(g), b.macs);
 }
 
-Model resnet18(int hw, int width, int classes) {
+Model resnet18(int hw, int width, int classes, bool mergedShortcut) {
     std::unique_ptr<Graph> g(new Graph());
     Builder b{*g};
     Tensor *x = g->tensor({1, 3, hw, hw});
@@ -102,8 +102,23 @@ Model resnet18(int hw, int width, int classes) {
         int cout = width << stage;
         for (int block = 0; block < 2; ++block) {
             int stride = (block == 0 && stage > 0) ? 2 : 1;
-            Tensor *y = b.conv(x, cout, 3, stride, 1, 1, true);
-            Tensor *skip = stride == 2 ? b.conv(x, cout, 1, 2, 0, 1, false) : x;
+            Tensor *y, *skip;
+            if (stride == 2 && mergedShortcut) {
+                // PET's merge of two convolutions that read the same tensor
+                // (src/Mutant/generator.cc:1236-1381): the 1x1 shortcut's filters are padded
+                // to 3x3 and stacked under the first convolution's (weight-side work), one
+                // convolution computes both, Split on the channel dim hands them out. The
+                // ReLU belongs to the first half only and moves behind the Split.
+                const double before = b.macs;
+                Tensor *both = b.conv(x, 2 * cout, 3, 2, 1, 1, false);
+                b.macs = before + (double)both->size() / 2 * x->getDims()[1] * (9 + 1); // nominal work
+                const TensorVec &parts = g->split(both, 1, 2)->getOutputs();
+                y = g->relu(parts[0])->getOutputs()[0];
+                skip = parts[1];
+            } else {
+                y = b.conv(x, cout, 3, stride, 1, 1, true);
+                skip = stride == 2 ? b.conv(x, cout, 1, 2, 0, 1, false) : x;
+            }
             y = b.conv(y, cout, 3, 1, 1, 1, false);
             x = b.addRelu(y, skip);
         }
@@ -111,7 +126,7 @@ Model resnet18(int hw, int width, int classes) {
     int c = x->getDims()[1];
     x = g->avgpool(x, b.fresh())->getOutputs()[0];
     x = b.linear(b.reshape(x, {1, 1, c}), classes);
-    return finish("resnet18", std::move(g), b.macs);
+    return finish(mergedShortcut ? "resnet18:pet" : "resnet18", std::move(g), b.macs);
 }
 
 Model bertBase(int layers, int seq, int hidden, int heads, int ffn, bool mergedQkv) {
@@ -185,6 +200,8 @@ bool byName(const std::string &name, Model &out) {
         out = dilatedBlock(true);
     else if (name == "resnet18")
         out = resnet18();
+    else if (name == "resnet18:pet")
+        out = resnet18(224, 64, 1000, true);
     else if (name == "bert")
         out = bertBase();
     else if (name == "bert:pet")

@@ -983,6 +983,50 @@ static bool test_merged_projections() {
     return true;
 }
 
+// PET's merge of a block's first convolution with its 1x1 shortcut: one convolution with
+// both filter banks, Split on the channel dim (contiguous slabs at batch 1: a view), ReLU on
+// the first half only. The graph runtime leaves that ReLU to the convolution that reads it.
+static bool test_merged_shortcut_block() {
+    Graph g;
+    Tensor *x = g.tensor({1, 8, 12, 12});
+    Tensor *w1 = g.tensor({32, 8, 3, 3}), *w2 = g.tensor({16, 16, 3, 3});
+    w1->setType(Tensor::Weight);
+    w2->setType(Tensor::Weight);
+    Tensor *both = g.conv(x, w1, 1, 1, 2, 2, 1, 1)->getOutputs()[0]; // [1, 32, 6, 6]
+    const TensorVec &parts = g.split(both, 1, 2)->getOutputs();
+    Tensor *y = g.relu(parts[0])->getOutputs()[0];
+    y = g.conv(y, w2, 1, 1, 1, 1, 1, 1)->getOutputs()[0];
+    g.relu(g.add({y, parts[1]})->getOutputs()[0]);
+    g.updateConnection();
+    x->dataRand(3);
+    w1->dataRand(4);
+    w2->dataRand(5);
+    auto s1 = std::make_shared<SubGraph>(g.getOperators());
+    auto s2 = std::make_shared<SubGraph>(g.getOperators());
+    for (auto sg : {s1, s2})
+        for (auto t : sg->getInputs())
+            for (auto orig : g.getTensors())
+                if (orig->getHash() == t->getHash())
+                    t->setData(orig->getDataPtr());
+    EXPECT(s1->compute());
+    CodeEngine ce;
+    auto exec = ce.instantiate(s2);
+    EXPECT(exec != nullptr);
+    EXPECT(exec->numAliasedOps() == 1);  // the Split
+    EXPECT(exec->numKernelOps() == 2); // the two convolutions (the second with its tail)
+    for (int rep = 0; rep < 2; ++rep) {
+        EXPECT(exec->launch() && exec->sync());
+        Tensor *o1 = s1->getOutputs()[0], *o2 = s2->getOutputs()[0];
+        o2->deviceWritten();
+        EXPECT(equalArrays(o1->getDataPtr(), o2->getDataPtr(), o1->size()));
+    }
+    std::string code = ce.genCode(s2);
+    EXPECT(code.find("pet_hip_activation(") == std::string::npos);
+    EXPECT(code.find("pet_hip_split(") == std::string::npos);
+    EXPECT(code.find("pet_hip_conv2d_ex_f32(") != std::string::npos); // X_RELU on the reader
+    return true;
+}
+
 static bool test_convtrans_reference_vectors() {
     EXPECT(convTransCase(2, 2, 3, 4, 4, 2, 1, 2,
                          {190,  740,  770,  592,  992,  2704, 2836, 1832, 1184, 3232, 3364,
@@ -1054,6 +1098,7 @@ int main(int argc, char **argv) {
         {"convtrans_reference_vectors", test_convtrans_reference_vectors},
         {"band_matmuls", test_band_matmuls},
         {"merged_projections", test_merged_projections},
+        {"merged_shortcut_block", test_merged_shortcut_block},
     };
     std::string only = argc > 1 ? argv[1] : "";
     if (argc > 2)

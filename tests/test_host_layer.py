@@ -21,7 +21,7 @@ CASES = ["conv_vs_oracle", "conv_invalid_groups", "transpose_n2h_h2n", "batch_ge
          "random_graphs_replay_equals_eager", "batchnorm_pow_div",
          "gather_reduce_mean", "launch_fusion_block", "alias_plan_shared_storage",
          "two_conv_verification", "convtrans_reference_vectors", "band_matmuls",
-         "merged_projections"]
+         "merged_projections", "merged_shortcut_block"]
 
 
 def test_host_library_is_built_and_exports_the_operator_classes():
@@ -369,8 +369,8 @@ RUN_MODEL = os.path.join(LIB, "pet_run_model")
 
 
 @pytest.mark.gpu
-@pytest.mark.parametrize("model", ["dilated", "dilated:pet", "resnet18", "bert", "bert:pet",
-                                   "resnet3d18"])
+@pytest.mark.parametrize("model", ["dilated", "dilated:pet", "resnet18", "resnet18:pet", "bert",
+                                   "bert:pet", "resnet3d18"])
 def test_model_graph_replay_equals_operator_by_operator_run(model):
     """pet_run_model --check: the captured HIP graph (storage sharing, transposes in a
     row folded into one kernel, constant 3-D filters repacked) against
@@ -387,6 +387,9 @@ def test_model_graph_replay_equals_operator_by_operator_run(model):
     assert rec["ms"] > 0
     if model == "dilated:pet":
         assert rec["folded"] == 2 and rec["kernels"] == 8
+    if model == "resnet18:pet":
+        # three blocks run their shortcut inside their first convolution
+        assert rec["kernels"] == 23 - 3
     if model == "bert:pet":
         # per layer: one merged projection instead of three, the stacking Concat never runs
         assert rec["kernels"] == 108 - 2 * 12
