@@ -49,6 +49,20 @@ def test_attention_matches_the_operator_sequence(ops, heads, seq, dh):
     assert max_rel_err(got, ref, mag) <= REL_TOL
 
 
+def test_attention_over_a_batch_of_sequences(ops):
+    """[batch, seq, heads*dh] operands: every batch entry is an attention of its own."""
+    batch, heads, seq, dh = 3, 4, 70, 32
+    rng = np.random.default_rng(5)
+    q, k, v = (rng.standard_normal((batch, seq, heads * dh)).astype(np.float32) for _ in range(3))
+    scale = 1.0 / np.sqrt(dh)
+    got = host(ops.attention(dev(q), dev(k), dev(v), heads, scale))
+    assert got.shape == (batch, seq, heads * dh)
+    for b in range(batch):
+        ref = oracle.attention(q[b], k[b], v[b], heads, scale)
+        mag = oracle.attention(q[b], k[b], np.abs(v[b]), heads, scale)
+        assert max_rel_err(got[b], ref, mag) <= REL_TOL
+
+
 def test_attention_reads_the_slabs_of_a_merged_projection_in_place(ops):
     """Q, K and V as the three [seq, hidden] slabs of one [3, seq, hidden] tensor and as
     column blocks of one [seq, 3*hidden] tensor (row stride 3*hidden); the scale from a
