@@ -29,6 +29,13 @@ extern "C" {
 #define PET_HIP_API
 #endif
 
+/* Empty tensors. An empty batch (n, b or bs of 0, no rows) or an empty output is not an
+ * error: the call launches nothing, returns PET_HIP_OK and does not look at the pointers,
+ * which may then be NULL. The reference's loop nests do the same by not running
+ * (src/Graph/operator.cc:94-158, 620-654). A matmul over an empty k axis writes the bias
+ * (zeros without one), a pad around an empty tensor writes zeros. Negative extents, and a
+ * zero where the operator's shape rule needs a positive number (channels, filters, filter
+ * extents, strides), are PET_HIP_ERR_INVALID. */
 typedef enum pet_hip_status {
     PET_HIP_OK = 0,
     PET_HIP_ERR_INVALID = 1,     /* bad argument / shape the op rejects (reference: compute() == nullptr) */

@@ -217,10 +217,12 @@ int pet_hip_attention_f32(const float *q, const float *k, const float *v, float 
                           long long stride_o, float scale, const float *scale_dev,
                           pet_hip_stream_t stream) {
     PET_REQUIRE_INIT();
+    if (batch < 0 || heads <= 0 || seq <= 0 || dh <= 0)
+        return set_error(PET_HIP_ERR_INVALID, "attention: bad shape");
+    if (batch == 0)
+        return PET_HIP_OK; // no sequences
     if (!q || !k || !v || !out)
         return set_error(PET_HIP_ERR_INVALID, "attention: null operand");
-    if (batch <= 0 || heads <= 0 || seq <= 0 || dh <= 0)
-        return set_error(PET_HIP_ERR_INVALID, "attention: bad shape");
     const int width = heads * dh;
     if (ldq < width || ldk < width || ldv < width || ldo < width)
         return set_error(PET_HIP_ERR_INVALID, "attention: row stride below heads * dh");

@@ -448,13 +448,19 @@ __global__ __launch_bounds__(64 * kWavesPerBlock) void gbmml_staged_kernel(BandP
     }
 }
 
+// *empty: no batch entries or no rows, nothing to compute (pointers are not looked at).
 int check_band(const float *A, const float *B, float *C, int bs, int m, int x, int w, int d,
-               const char *what) {
-    if (!A || !B || !C)
-        return set_error(PET_HIP_ERR_INVALID, "%s: null operand", what);
-    if (bs <= 0 || m <= 0 || x <= 0 || w < 0 || d <= 0)
+               const char *what, bool *empty) {
+    *empty = false;
+    if (bs < 0 || m < 0 || x <= 0 || w < 0 || d <= 0)
         return set_error(PET_HIP_ERR_INVALID, "%s: bad shape bs=%d m=%d %d w=%d d=%d", what, bs, m,
                          x, w, d);
+    if (bs == 0 || m == 0) {
+        *empty = true;
+        return PET_HIP_OK;
+    }
+    if (!A || !B || !C)
+        return set_error(PET_HIP_ERR_INVALID, "%s: null operand", what);
     const long long band = 2ll * w + 1;
     if ((long long)bs * m * band >= (1ll << 31) || (long long)bs * m * x >= (1ll << 31))
         return set_error(PET_HIP_ERR_UNSUPPORTED, "%s: tensors of 2^31 elements or more", what);
@@ -486,8 +492,11 @@ extern "C" {
 int pet_hip_g2bmm_f32(const float *A, const float *B, float *C, int bs, int m, int k, int width,
                       int dilation, pet_hip_stream_t stream) {
     PET_REQUIRE_INIT();
-    if (int rc = check_band(A, B, C, bs, m, k, width, dilation, "g2bmm"))
+    bool empty;
+    if (int rc = check_band(A, B, C, bs, m, k, width, dilation, "g2bmm", &empty))
         return rc;
+    if (empty)
+        return PET_HIP_OK;
     BandParams p{A, B, C, bs, m, k, width, dilation, 0, 0, 0};
     p.mc = (m + dilation - 1) / dilation;
     // tiles from column i0 - w to i0 + 31 + w
@@ -518,8 +527,11 @@ int pet_hip_g2bmm_f32(const float *A, const float *B, float *C, int bs, int m, i
 int pet_hip_gbmml_f32(const float *A, const float *B, float *C, int bs, int m, int width, int n,
                       int dilation, pet_hip_stream_t stream) {
     PET_REQUIRE_INIT();
-    if (int rc = check_band(A, B, C, bs, m, n, width, dilation, "gbmml"))
+    bool empty;
+    if (int rc = check_band(A, B, C, bs, m, n, width, dilation, "gbmml", &empty))
         return rc;
+    if (empty)
+        return PET_HIP_OK;
     BandParams p{A, B, C, bs, m, 0, width, dilation, n, 0, 0};
     p.mc = (m + dilation - 1) / dilation;
     const unsigned iblocks = (unsigned)((p.mc + 31) / 32);

@@ -233,9 +233,7 @@ int pet_hip_conv_trans_f32(const float *x, const float *w, const float *bias, fl
                            int sw, int dh, int dw, int oph, int opw, int act,
                            pet_hip_stream_t stream) {
     PET_REQUIRE_INIT();
-    if (!x || !w || !y)
-        return set_error(PET_HIP_ERR_INVALID, "conv_trans: null operand");
-    if (n <= 0 || h <= 0 || wd <= 0 || f <= 0 || r <= 0 || s <= 0 || c <= 0 || sh <= 0 ||
+    if (n < 0 || h <= 0 || wd <= 0 || f <= 0 || r <= 0 || s <= 0 || c <= 0 || sh <= 0 ||
         sw <= 0 || dh <= 0 || dw <= 0 || ph < 0 || pw < 0 || oph < 0 || opw < 0)
         return set_error(PET_HIP_ERR_INVALID, "conv_trans: bad shape or parameter");
     ConvTransParams p;
@@ -264,6 +262,10 @@ int pet_hip_conv_trans_f32(const float *x, const float *w, const float *bias, fl
     p.nfast = n >= 32;
     if (p.OH <= 0 || p.OW <= 0)
         return set_error(PET_HIP_ERR_INVALID, "conv_trans: empty output %d x %d", p.OH, p.OW);
+    if (n == 0)
+        return PET_HIP_OK; // an empty batch: nothing to compute, as in the convolutions
+    if (!x || !w || !y)
+        return set_error(PET_HIP_ERR_INVALID, "conv_trans: null operand");
     const long long xin = (long long)n * h * wd * f, yout = (long long)n * p.OH * p.OW * c,
                     wel = (long long)r * s * f * c;
     if (xin >= (1ll << 31) || yout >= (1ll << 31) || wel >= (1ll << 31))

@@ -711,7 +711,11 @@ int launch_view_copy(const float *x, float *y, ViewDesc v, long long in_elems,
     if (total >= (1ll << 31) || in_elems >= (1ll << 31) || out_elems >= (1ll << 31))
         return set_error(PET_HIP_ERR_UNSUPPORTED,
                          "layout ops are limited to tensors below 2^31 elements");
-    if (!x || !y)
+    if (!y)
+        return set_error(PET_HIP_ERR_INVALID, "null tensor pointer");
+    if (in_elems == 0) // padding around an empty tensor: nothing to read, all zeros
+        return pet_hip_fill_f32(y, 0.f, (size_t)out_elems, (pet_hip_stream_t)stream);
+    if (!x)
         return set_error(PET_HIP_ERR_INVALID, "null tensor pointer");
     // does any element read at all? (a dim whose window is empty zero-fills)
     bool any_valid = true;
