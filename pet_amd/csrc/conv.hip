@@ -1183,8 +1183,11 @@ int launch_conv(ConvParams &p, hipStream_t stream) {
         return set_error(PET_HIP_ERR_UNSUPPORTED,
                          "kt-major filters are only read by the plane kernel; this shape does "
                          "not use it (pet_hip_conv3d_pack_filters would have said so)");
-    if (p.dry_atomic) // the general kernel never accumulates into y
+    if (p.dry_atomic) // the kernels below never accumulate into y
         return PET_HIP_OK;
+    rc = try_launch_stem(p, stream);
+    if (rc >= 0)
+        return rc;
     const bool veca = (p.K % 4 == 0) && (((uintptr_t)p.w & 15) == 0);
     switch (pick_tile(p.M, p.NPIX, p.G)) {
     case 0:

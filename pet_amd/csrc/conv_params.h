@@ -68,6 +68,10 @@ constexpr unsigned kOob = 0x80000000u; // voffset that the range check rejects
 // kernels), else a pet_hip_status.
 int try_launch_direct(const ConvParams &p, hipStream_t stream);
 
+// stem.hip: 7x7 stride-2 filters over three channels, input patch and filter bank staged in
+// LDS. Returns -1 when it does not apply, else a pet_hip_status.
+int try_launch_stem(const ConvParams &p, hipStream_t stream);
+
 // conv.hip: y = bias (+ residual) ahead of a launch that adds partial sums into y.
 int launch_accumulate_init(const ConvParams &p, hipStream_t stream);
 
