@@ -260,19 +260,22 @@ __global__ __launch_bounds__(256) void bias_act_kernel(const float *__restrict__
     }
 }
 
+// I: the index type, 32 bits when input and output have fewer than 2^31 elements (the three
+// divisions of an output index are most of this kernel's instructions in 64 bits).
+template <typename I>
 __global__ __launch_bounds__(256) void pool2d_kernel(const float *__restrict__ x,
                                                      float *__restrict__ y, int nc, int h, int w,
                                                      int kh, int kw, int ph, int pw, int sh,
                                                      int sw, int dh, int dw, int oh, int ow,
                                                      int mode, float lo) {
-    size_t total = (size_t)nc * oh * ow;
-    size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
-    const size_t step = (size_t)gridDim.x * 256;
-    for (; i < total; i += step) {
-        int j = (int)(i % ow);
-        int ii = (int)((i / ow) % oh);
-        size_t plane = i / ((size_t)ow * oh);
-        const float *xp = x + plane * (size_t)h * w;
+    const I total = (I)nc * (I)oh * (I)ow;
+    const I step = (I)gridDim.x * 256;
+    for (I i = (I)blockIdx.x * 256 + threadIdx.x; i < total; i += step) {
+        const int j = (int)(i % (I)ow);
+        const I rest = i / (I)ow;
+        const int ii = (int)(rest % (I)oh);
+        const I plane = rest / (I)oh;
+        const float *xp = x + plane * (I)h * (I)w;
         float acc = mode == 0 ? -INFINITY : 0.f;
         int taps = 0; // window positions inside the image: the divisor of an average
         for (int r = 0; r < kh; ++r) {
@@ -283,7 +286,7 @@ __global__ __launch_bounds__(256) void pool2d_kernel(const float *__restrict__ x
                 int iw = j * sw + s * dw - pw;
                 if (iw < 0 || iw >= w)
                     continue;
-                float v = fmaxf(xp[(size_t)ih * w + iw], lo); // lo = 0: ReLU on the way in
+                float v = fmaxf(xp[ih * w + iw], lo); // lo = 0: ReLU on the way in
                 acc = mode == 0 ? fmaxf(acc, v) : acc + v;
                 ++taps;
             }
@@ -733,14 +736,22 @@ int pet_hip_pool2d_ex(const float *x, float *y, int n, int c, int h, int w, int 
         return PET_HIP_OK;
     if (!x || !y)
         return set_error(PET_HIP_ERR_INVALID, "null pointer");
+    if ((long long)n * c >= (1ll << 31))
+        return set_error(PET_HIP_ERR_UNSUPPORTED, "pooling over 2^31 planes or more");
     if (mode == 1 && kh == h && kw == w && ph == 0 && pw == 0 && dh == 1 && dw == 1) {
         int nc = n * c;
         hipLaunchKernelGGL(global_avgpool_kernel, dim3((nc + 3) / 4), dim3(256), 0,
                            as_stream(stream), x, y, nc, h * w, lo);
         return check_launch("global_avgpool_kernel");
     }
-    hipLaunchKernelGGL(pool2d_kernel, dim3(grid_for(total)), dim3(256), 0, as_stream(stream), x, y,
-                       n * c, h, w, kh, kw, ph, pw, sh, sw, dh, dw, oh, ow, mode, lo);
+    if ((size_t)n * c * h * w < (1ull << 31) && total < (1ull << 31))
+        hipLaunchKernelGGL(pool2d_kernel<unsigned>, dim3(grid_for(total)), dim3(256), 0,
+                           as_stream(stream), x, y, n * c, h, w, kh, kw, ph, pw, sh, sw, dh, dw,
+                           oh, ow, mode, lo);
+    else
+        hipLaunchKernelGGL(pool2d_kernel<size_t>, dim3(grid_for(total)), dim3(256), 0,
+                           as_stream(stream), x, y, n * c, h, w, kh, kw, ph, pw, sh, sw, dh, dw,
+                           oh, ow, mode, lo);
     return check_launch("pool2d_kernel");
 }
 
