@@ -107,3 +107,28 @@ def test_stem_equals_the_general_kernel(ops):
     y = ops.conv2d(x, w, 3, 3, 2, 2)
     z = ops.conv2d(x, w, 3, 3, 2, 2, residual=torch.zeros_like(y))
     assert torch.equal(y, z)
+
+
+def test_stem_random_shapes(ops):
+    """Thirty seeded shapes, 2-D and 3-D, small integers, bit for bit against the oracle."""
+    rng = np.random.default_rng(2024)
+    for _ in range(30):
+        n, f = int(rng.integers(1, 4)), int(rng.integers(1, 140))
+        h, w = int(rng.integers(7, 70)), int(rng.integers(7, 70))
+        pad = int(rng.integers(0, 4))
+        if rng.random() < 0.5:
+            x = rng.integers(-3, 4, (n, 3, h, w)).astype(np.float32)
+            k = rng.integers(-3, 4, (f, 3, 7, 7)).astype(np.float32)
+            want = oracle.conv2d(x, k, pad, pad, 2, 2)
+            got = host(ops.conv2d(dev(x), dev(k), pad, pad, 2, 2))
+        else:
+            t, kt = int(rng.integers(1, 7)), int(rng.integers(1, 4))
+            pt, st = int(rng.integers(0, kt)), int(rng.integers(1, 3))
+            if t + 2 * pt < kt:
+                continue
+            x = rng.integers(-3, 4, (n, 3, t, h, w)).astype(np.float32)
+            k = rng.integers(-3, 4, (f, 3, kt, 7, 7)).astype(np.float32)
+            want = oracle.conv3d(x, k, (pt, pad, pad), (st, 2, 2))
+            got = host(ops.conv3d(dev(x), dev(k), (pt, pad, pad), (st, 2, 2)))
+        assert got.shape == want.shape
+        np.testing.assert_array_equal(got, want)
