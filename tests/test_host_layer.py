@@ -83,6 +83,10 @@ REFERENCE_PROGRAMS = [
     "transpose_test_1.cc", "transpose_test_2.cc", "transpose_test_3.cc", "transpose_test_4.cc",
     "transpose_test_5.cc",
 ]
+# ... and programs that also drive the generator, the search engine and the code engine:
+# they include the reference's own generator.h / search_engine.h (CMutator, nnet, ...),
+# so they are only compiled where the whole search is built (pet_amd/host/Makefile) and
+# run below, not syntax-checked here against empty stand-ins.
 REFERENCE_TESTS = "/root/reference/src/Test"
 
 
@@ -538,6 +542,67 @@ REFERENCE_OPERATOR_PROGRAMS = [
     "split_test_2", "tensor_test", "transpose_test_2", "transpose_test_3", "transpose_test_4",
     "transpose_test_5",
 ]
+
+
+# Programs of src/Test that build graphs and hand them to the reference's Generator,
+# SearchEngine (which times every candidate through Operator::perf on the device) and
+# CodeEngine: compiled unchanged, run to their own end. What they print is the search's
+# report; "Best Perf" can only be at or below "Origin Perf" (the search keeps the input graph
+# when nothing beats it). Left out, with the reason:
+#   convtrans_test_1 / _2     compare an NHWC output tensor, flat, with vectors written down in
+#                             NCHW order, and ConvTransOp::compute upstream takes its loop
+#                             bounds from the wrong dims (src/Graph/operator.cc:948): they
+#                             abort on the reference's own code too. The vectors themselves
+#                             are tests/golden/convtrans_reference_vectors.json, used with
+#                             the layout they were made in.
+#   transposeconv_test_1      its filter tensor is [f, r, s, c] and of type Input: the
+#                             reference's own ConvTransOp::checkValid (:1098-1111) rejects it
+#   graph_stat_test_2_batchmm copy-assigns a SubGraph, whose destructor frees the operators
+#                             both copies point at (src/Graph/graph.cc:12-19)
+#   SampleGraph1              a search of several minutes
+#   single_op_test_8_conv3d, gen_transpose    do not compile against the reference's own
+#                             headers at its head; import_onnx*: need .onnx files
+REFERENCE_SEARCH_PROGRAMS = {
+    # program: command-line arguments
+    "split_test_3": [], "fuse_activation": [], "eliminator_test_1": [],
+    "single_op_test_1": [], "single_op_test_2": [], "single_op_test_3": [],
+    "single_op_test_4": [], "single_op_test_5": [], "single_op_test_6": [],
+    "single_op_test_7_batch_gemm": [], "graph_stat_test_1_transpose_group": [],
+    "mutant_test_1": [], "mutant_test_3": [], "cache_test_1": [], "cache_test_2": [],
+    "cache_test_3": [], "SampleGraph2": [],
+    # the reference's own dilated-convolution benchmark: six 3x3 convolutions with ReLU at
+    # dilation 2 (configuration 1), batch 1; searches, then emits the program (res.cu)
+    "dilation_test": ["1", "1"],
+}
+
+
+# searches over a single convolution that time dozens of candidates (30-95 s each): run with
+# PET_SLOW_REFERENCE_PROGRAMS=1; the same path is covered by single_op_test_3 / _6 / _7
+SLOW_SEARCH_PROGRAMS = {"single_op_test_1", "single_op_test_2", "single_op_test_4",
+                        "single_op_test_5"}
+
+
+@pytest.mark.gpu
+@needs_refsearch
+@pytest.mark.parametrize("program", sorted(REFERENCE_SEARCH_PROGRAMS))
+def test_reference_search_program_runs_on_the_device(program, tmp_path):
+    import re
+    if program in SLOW_SEARCH_PROGRAMS and not os.environ.get("PET_SLOW_REFERENCE_PROGRAMS"):
+        pytest.skip("a search of 30-95 s: set PET_SLOW_REFERENCE_PROGRAMS=1")
+    exe = os.path.join(REFTESTS, program)
+    assert os.path.exists(exe), "run __graft_entry__.build() where the reference tree is present"
+    res = subprocess.run([exe] + REFERENCE_SEARCH_PROGRAMS[program], capture_output=True,
+                         text=True, timeout=600, cwd=str(tmp_path))
+    print(res.stdout[-2000:])
+    print(res.stderr[-1500:])
+    assert res.returncode == 0
+    origin = re.findall(r"Origin Perf: ([0-9.eE+-]+)", res.stdout)
+    best = re.findall(r"Best Perf with correction: ([0-9.eE+-]+)", res.stdout)
+    for o, b in zip(origin, best):
+        assert 0 < float(b) <= float(o) * 1.001
+    if program == "dilation_test":
+        emitted = (tmp_path / "res.cu").read_text()
+        assert emitted.count("pet_hip_conv2d") >= 6     # the six layers, ReLU fused
 
 
 @pytest.mark.gpu
