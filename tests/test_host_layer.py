@@ -559,7 +559,10 @@ REFERENCE_OPERATOR_PROGRAMS = [
 #                             reference's own ConvTransOp::checkValid (:1098-1111) rejects it
 #   graph_stat_test_2_batchmm copy-assigns a SubGraph, whose destructor frees the operators
 #                             both copies point at (src/Graph/graph.cc:12-19)
-#   SampleGraph1              a search of several minutes
+#   SampleGraph1              after 160 s of search it dies inside the reference's own
+#                             Generator::markTransType (src/Mutant/generator.cc:1953-1954: it
+#                             dereferences the producer of a convolution's input where that
+#                             input is the graph's input; the `if` above it, :1950, is empty)
 #   single_op_test_8_conv3d, gen_transpose    do not compile against the reference's own
 #                             headers at its head; import_onnx*: need .onnx files
 REFERENCE_SEARCH_PROGRAMS = {
