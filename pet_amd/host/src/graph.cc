@@ -551,12 +551,6 @@ bool GraphBase::exportOnnx(const char *path) {
     return false;
 }
 
-bool GraphBase::importOnnx(const char *net) {
-    std::fprintf(stderr, "[pet] importOnnx(%s): use pet_amd.onnx_import.load, which builds the "
-                         "graph through the Python module\n", net ? net : "");
-    return false;
-}
-
 uint64_t SubGraph::getCacheIdx(int level) {
     static const uint64_t factors[8] = {10000019, 10000079, 10000103, 10000121,
                                         10000139, 10000141, 10000169, 10000189};

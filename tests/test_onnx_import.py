@@ -307,3 +307,91 @@ def test_imported_resnet18_matches_torch():
     assert np.abs(got - want).max() <= 1e-4 * scale, (np.abs(got - want).max(), scale)
     assert ex.numKernelOps() <= 26
     assert 0.05 < ex.time(5, 20) < 5.0      # ms per inference
+
+
+# ---- the same files through the host layer's own reader (Graph::importOnnx, C++) ---------
+# pet_amd/lib/pet_onnx_driver (tests/cpp/onnx_driver.cc) imports a file, prints the operators
+# with the shapes of their outputs and, given an input, runs the graph on the device.
+DRIVER = os.path.join(ROOT, "pet_amd", "lib", "pet_onnx_driver")
+REFTESTS = os.path.join(ROOT, "pet_amd", "lib", "reftests")
+
+
+def _driver(*args, **kw):
+    import subprocess
+    assert os.path.exists(DRIVER), "run __graft_entry__.build()"
+    return subprocess.run([DRIVER] + [str(a) for a in args], capture_output=True, text=True,
+                          timeout=300, **kw)
+
+
+def test_native_importer_builds_the_same_graphs(tmp_path):
+    from pet_amd import onnx_import
+    for name, (data, _) in (("cnn", cnn(np.random.default_rng(0))),
+                            ("conv_bn", _conv_bn_model(np.random.default_rng(3))),
+                            ("resnet18", _resnet18(np.random.default_rng(18)))):
+        path = tmp_path / (name + ".onnx")
+        path.write_bytes(data)
+        res = _driver(path)
+        assert res.returncode == 0, res.stderr[-1000:]
+        lines = [ln for ln in res.stdout.splitlines() if "->" in ln]
+        want = [op.toString() for op in onnx_import.load(data).graph.getOperators()]
+        # the same operators with the same arguments, in the same order (tensor ids and the
+        # hashes derived from them differ between two processes: compare without them)
+        import re
+        strip = lambda s: re.sub(r"\[\d{5,}\]|(input|weight|output|in|out|A|B|C)=\d+,?", "", s)
+        assert [strip(ln.split("  ->")[0]) for ln in lines] == [strip(s) for s in want]
+    assert sum(ln.startswith("Conv") for ln in lines) == 20            # ResNet-18, BN folded
+    assert not any("BatchNorm" in ln for ln in lines)
+    assert lines[-1].endswith("[1,1,1000]")
+
+
+def test_native_importer_refuses_what_it_cannot_take(tmp_path):
+    bad = tmp_path / "einsum.onnx"
+    bad.write_bytes(ow.model([ow.node("Einsum", ["x"], ["y"])], {}, [("x", [2, 2])], [("y", [2, 2])]))
+    res = _driver(bad)
+    assert res.returncode == 2 and "Einsum is not supported" in res.stderr
+    cut = tmp_path / "cut.onnx"
+    cut.write_bytes(cnn(np.random.default_rng(0))[0][:-37])
+    res = _driver(cut)
+    assert res.returncode == 2 and "truncated" in res.stderr
+    res = _driver(tmp_path / "missing.onnx")
+    assert res.returncode == 2 and "cannot open" in res.stderr
+
+
+@pytest.mark.gpu
+def test_natively_imported_networks_match_torch(tmp_path):
+    for name, (data, w), shape, ref in (
+            ("cnn", cnn(np.random.default_rng(1)), (1, 3, 16, 16), cnn_reference),
+            ("resnet18", _resnet18(np.random.default_rng(18)), (1, 3, 224, 224), _resnet18_torch)):
+        x = np.random.default_rng(7).standard_normal(shape).astype(np.float32)
+        (tmp_path / (name + ".onnx")).write_bytes(data)
+        x.tofile(tmp_path / "in.bin")
+        res = _driver(tmp_path / (name + ".onnx"), tmp_path / "in.bin", tmp_path / "out.bin")
+        assert res.returncode == 0, res.stderr[-1000:]
+        want = ref(x, w)
+        got = np.fromfile(tmp_path / "out.bin", dtype=np.float32).reshape(want.shape)
+        assert np.abs(got - want).max() <= 1e-4 * np.abs(want).max()
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("program", ["import_onnx", "import_onnx_nnet", "import_onnx_cmutator"])
+def test_reference_import_programs_run_unchanged(program, tmp_path):
+    """src/Test/import_onnx*.cpp of the reference, compiled unchanged: Graph::importOnnx on a
+    model file, SearchEngine::run with the mutation generator / the nnet mutator / CMutator,
+    CodeEngine::genCode for the best graph (res.cu) and, in two of them, for the graph as
+    given (origin.cu). The reference's importOnnx calls into its Python plug-in and the `onnx`
+    package; here it is the host layer's own reader."""
+    import subprocess
+    exe = os.path.join(REFTESTS, program)
+    status = os.path.join(ROOT, "pet_amd", "lib", "refsearch_status.txt")
+    if os.path.exists(status) and open(status).read().strip() == "no-reference":
+        pytest.skip("the build had no reference tree to compile from")
+    assert os.path.exists(exe), "run __graft_entry__.build() where the reference tree is present"
+    (tmp_path / "cnn.onnx").write_bytes(cnn(np.random.default_rng(1))[0])
+    res = subprocess.run([exe, "cnn.onnx"], capture_output=True, text=True, timeout=600,
+                         cwd=str(tmp_path))
+    print(res.stdout[-2500:])
+    print(res.stderr[-1500:])
+    assert res.returncode == 0
+    assert "Graph Imported" in res.stdout
+    emitted = (tmp_path / "res.cu").read_text()
+    assert emitted.count("pet_hip_conv2d") >= 2 and "pet_hip_softmax" in emitted
