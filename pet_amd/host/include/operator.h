@@ -22,6 +22,14 @@ namespace tpm {
 
 class PerfEngine;
 
+// While one of these lives (on this thread), an operator constructor that finds its operands
+// invalid throws std::invalid_argument instead of asserting.
+struct InvalidOperandsThrow {
+    InvalidOperandsThrow();
+    ~InvalidOperandsThrow();
+    InvalidOperandsThrow(const InvalidOperandsThrow &) = delete;
+};
+
 class Operator {
   public:
     // Numbering as in the reference (include/operator.h:19-51); the ops this

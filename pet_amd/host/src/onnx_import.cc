@@ -367,7 +367,7 @@ void foldBatchnorm(Model &m) {
     std::set<const Node *> dropped;
     const std::set<std::string> outs(m.outputs.begin(), m.outputs.end());
     for (auto &nd : m.nodes) {
-        if (nd.op != "BatchNormalization" || nd.inputs.size() < 5)
+        if (nd.op != "BatchNormalization" || nd.inputs.size() < 5 || nd.outputs.empty())
             continue;
         bool constant = true;
         for (int i = 1; i < 5; ++i)
@@ -376,7 +376,8 @@ void foldBatchnorm(Model &m) {
         if (!constant || it == byOut.end())
             continue;
         Node *conv = it->second;
-        if (conv->op != "Conv" || users[conv->outputs[0]] != 1 || outs.count(conv->outputs[0]))
+        if (conv->op != "Conv" || conv->inputs.size() < 2 || users[conv->outputs[0]] != 1 ||
+            outs.count(conv->outputs[0]))
             continue;
         bool convConst = true;
         for (size_t i = 1; i < conv->inputs.size(); ++i)
@@ -387,8 +388,11 @@ void foldBatchnorm(Model &m) {
                     &me = m.inits[nd.inputs[3]], &va = m.inits[nd.inputs[4]];
         const double eps = nd.getf("epsilon", 1e-5);
         Array w = m.inits[conv->inputs[1]];
+        if (w.dims.empty() || w.dims[0] < 1 || w.size() % (size_t)w.dims[0] != 0)
+            continue;
         const size_t F = (size_t)w.dims[0], per = w.size() / F;
-        if (sc.size() != F || bi.size() != F || me.size() != F || va.size() != F)
+        if (sc.size() != F || bi.size() != F || me.size() != F || va.size() != F ||
+            (conv->inputs.size() > 2 && m.inits[conv->inputs[2]].size() != F))
             continue;
         Array b;
         b.dims = {(int64_t)F};
@@ -417,6 +421,19 @@ void foldBatchnorm(Model &m) {
 
 // ---------------------------------------------------------------- graph building
 
+Dim checkedDims(const std::vector<int64_t> &dims, const std::string &what) {
+    Dim out;
+    long long total = 1;
+    for (int64_t d : dims) {
+        if (d < 1 || d >= (1ll << 31) || (total *= d) >= (1ll << 31))
+            fail(what + ": a shape this backend does not take");
+        out.push_back((int)d);
+    }
+    if (out.size() > 8)
+        fail(what + ": more than 8 dims");
+    return out;
+}
+
 struct Builder {
     Graph *g;
     std::map<std::string, Tensor *> tensors;
@@ -431,13 +448,14 @@ struct Builder {
         auto c = consts.find(name);
         if (c == consts.end())
             fail("tensor " + name + " is neither computed nor a constant");
-        Dim dims;
-        for (int64_t d : c->second.dims)
-            dims.push_back((int)d);
+        Dim dims = checkedDims(c->second.dims, "constant " + name);
         if (dims.empty())
             dims.push_back(1);
         Tensor *t = g->tensor(dims);
         t->setType(Tensor::Weight);
+        if (t->size() != c->second.v.size())
+            fail("constant " + name + " holds " + std::to_string(c->second.v.size()) +
+                 " values for " + std::to_string(t->size()));
         std::vector<VType> host(c->second.v.begin(), c->second.v.end());
         if (!t->setData(host.data())) // host side; uploaded when an operator first needs it
             fail("cannot keep the values of " + name);
@@ -465,6 +483,8 @@ std::vector<int> symmetricPads(const Node &nd, int n) {
     for (int i = 0; i < n; ++i) {
         if (pads[i] != pads[i + n])
             fail(nd.op + ": asymmetric padding");
+        if (pads[i] < 0 || pads[i] > (1 << 20))
+            fail(nd.op + ": padding of " + std::to_string(pads[i]));
         out.push_back((int)pads[i]);
     }
     return out;
@@ -473,10 +493,14 @@ std::vector<int> symmetricPads(const Node &nd, int n) {
 std::vector<int> intsOr(const Node &nd, const char *key, int n, int dflt) {
     std::vector<int64_t> v = nd.getis(key);
     std::vector<int> out(n, dflt);
-    for (int i = 0; i < n && i < (int)v.size(); ++i)
+    for (int i = 0; i < n && i < (int)v.size(); ++i) {
+        if (v[i] < 1 || v[i] > (1 << 20))
+            fail(nd.op + ": " + key + " of " + std::to_string(v[i]));
         out[i] = (int)v[i];
+    }
     return out;
 }
+
 
 Tensor *resultOf(Operator *op) { return op ? op->getOutput() : nullptr; }
 
@@ -485,28 +509,32 @@ void build(Graph *g, Model &m) {
     for (auto &vi : m.inputs) {
         if (m.inits.count(vi.name))
             continue;
-        Dim dims;
-        for (int64_t d : vi.dims) {
+        for (int64_t d : vi.dims)
             if (d <= 0)
                 fail("input " + vi.name + " has a symbolic shape");
-            dims.push_back((int)d);
-        }
-        b.tensors[vi.name] = g->tensor(dims);
+        if (vi.dims.empty())
+            fail("input " + vi.name + " has no shape");
+        b.tensors[vi.name] = g->tensor(checkedDims(vi.dims, "input " + vi.name));
     }
     for (auto &nd : m.nodes) {
         const std::string &op = nd.op;
-        if (nd.outputs.empty() || nd.inputs.empty()) {
-            if (op == "Constant" && !nd.outputs.empty()) {
-                if (!nd.has("value"))
-                    fail("Constant without a value tensor");
-                b.consts[nd.outputs[0]] = nd.attrs.at("value").t;
-                continue;
-            }
-            fail("node " + nd.name + " (" + op + ") has no inputs or outputs");
-        }
-        if (op == "Constant") {
+        if (op == "Constant" && !nd.outputs.empty()) {
+            if (!nd.has("value") || nd.attrs.at("value").kind != Attr::Tensor)
+                fail("Constant without a value tensor");
             b.consts[nd.outputs[0]] = nd.attrs.at("value").t;
             continue;
+        }
+        if (nd.outputs.empty() || nd.inputs.empty())
+            fail("node " + nd.name + " (" + op + ") has no inputs or outputs");
+        {
+            // operands every form of the operator has
+            static const std::map<std::string, size_t> kOperands = {
+                {"Conv", 2}, {"Add", 2}, {"Mul", 2}, {"Sub", 2}, {"Div", 2}, {"MatMul", 2},
+                {"Gemm", 2}, {"Gather", 2}, {"Reshape", 2}, {"Pow", 2},
+                {"BatchNormalization", 5}, {"LayerNormalization", 2}};
+            auto need = kOperands.find(op);
+            if (need != kOperands.end() && nd.inputs.size() < need->second)
+                fail(op + " with " + std::to_string(nd.inputs.size()) + " inputs");
         }
         if (op == "Shape") {
             Array a;
@@ -533,6 +561,17 @@ void build(Graph *g, Model &m) {
             const std::vector<int> pads = symmetricPads(nd, nsp);
             const std::vector<int> st = intsOr(nd, "strides", nsp, 1);
             const std::vector<int> dil = intsOr(nd, "dilations", nsp, 1);
+            const Dim wdims = w->getDims();
+            const int64_t group = nd.geti("group", 1);
+            if ((int)wdims.size() != rank || group < 1 || wdims[1] * group != xd[1] ||
+                wdims[0] % group != 0)
+                fail("Conv: filters " + std::to_string(wdims.size()) + "-d / group " +
+                     std::to_string(group) + " do not fit the input");
+            for (int i = 0; i < nsp; ++i)
+                if (xd[2 + i] + 2 * pads[i] < dil[i] * (wdims[2 + i] - 1) + 1)
+                    fail("Conv: the filter is larger than the padded input");
+            if (bias && bias->size() != (size_t)wdims[0])
+                fail("Conv: the bias is not one value per filter");
             if (nsp == 2) {
                 out = resultOf(g->conv(x, w, pads[0], pads[1], st[0], st[1], dil[0], dil[1], bias));
             } else {
@@ -593,8 +632,11 @@ void build(Graph *g, Model &m) {
                 if (d != 1)
                     fail(op + ": dilated pooling is not supported");
             Dim od = {xd[0], xd[1]};
-            for (int i = 0; i < 2; ++i)
+            for (int i = 0; i < 2; ++i) {
+                if (k[i] < 1 || k[i] > xd[2 + i] + 2 * pads[i])
+                    fail(op + ": window of " + std::to_string(k[i]));
                 od.push_back((xd[2 + i] + 2 * pads[i] - (int)k[i]) / st[i] + 1);
+            }
             out = b.fresh(od);
             if (op == "MaxPool")
                 g->maxpool(x, out, (int)k[0], (int)k[1], 1, 1, pads[0], pads[1], st[0], st[1]);
@@ -623,12 +665,14 @@ void build(Graph *g, Model &m) {
                 fail("Gemm: C must be a vector of the output's last dim");
             out = resultOf(g->matmul(x, y, nd.geti("transA", 0) != 0, tb, bias));
         } else if (op == "Flatten") {
-            const int ax = (int)nd.geti("axis", 1);
+            const int64_t ax = nd.geti("axis", 1);
+            if (ax < 0 || ax > rank)
+                fail("Flatten: axis " + std::to_string(ax));
             int lead = 1, tail = 1;
             for (int i = 0; i < rank; ++i)
                 (i < ax ? lead : tail) *= xd[i];
             out = b.fresh({lead, tail});
-            g->flatten(x, out, ax);
+            g->flatten(x, out, (int)ax);
         } else if (op == "Reshape") {
             const Array &sh = b.constant(nd.inputs.at(1));
             Dim shape;
@@ -641,14 +685,19 @@ void build(Graph *g, Model &m) {
                         fail("Reshape: 0 beyond the input's rank");
                     v = xd[i];
                 }
-                if (v == -1)
+                if (v == -1 && hole < 0)
                     hole = (int)i;
-                else
-                    known *= v;
+                else if (v < 1 || (known *= v) > (long long)x->size())
+                    fail("Reshape: a shape that does not hold the input");
                 shape.push_back(v);
             }
             if (hole >= 0)
                 shape[hole] = (int)((long long)x->size() / std::max(known, 1ll));
+            long long total = 1;
+            for (int v : shape)
+                total *= v;
+            if (shape.empty() || total != (long long)x->size())
+                fail("Reshape: a shape that does not hold the input");
             out = b.fresh(shape);
             g->reshape(x, out);
         } else if (op == "Transpose") {
@@ -657,14 +706,30 @@ void build(Graph *g, Model &m) {
                 for (int i = rank - 1; i >= 0; --i)
                     perm.push_back(i);
             std::vector<PermItem> items;
-            for (int64_t p : perm)
+            std::vector<bool> seen(rank, false);
+            if ((int)perm.size() != rank)
+                fail("Transpose: perm of another rank");
+            for (int64_t p : perm) {
+                if (p < 0 || p >= rank || seen[p])
+                    fail("Transpose: perm is not a permutation");
+                seen[p] = true;
                 items.push_back(PermItem((int)p));
+            }
             out = resultOf(g->transpose(x, -1, Perm(items), 2));
         } else if (op == "Concat") {
             TensorVec ins;
-            for (auto &n : nd.inputs)
-                ins.push_back(b.in(n));
-            out = resultOf(g->concat(ins, axisOf(nd.geti("axis", 0))));
+            const int ax = axisOf(nd.geti("axis", 0));
+            for (auto &n : nd.inputs) {
+                Tensor *t = b.in(n);
+                Dim td = t->getDims();
+                if ((int)td.size() != rank)
+                    fail("Concat: inputs of different rank");
+                for (int i = 0; i < rank; ++i)
+                    if (i != ax && td[i] != xd[i])
+                        fail("Concat: inputs that differ off the axis");
+                ins.push_back(t);
+            }
+            out = resultOf(g->concat(ins, ax));
         } else if (op == "Split") {
             const int ax = axisOf(nd.geti("axis", 0));
             std::vector<int64_t> sizes = nd.getis("split");
@@ -673,6 +738,11 @@ void build(Graph *g, Model &m) {
                     sizes.push_back((int64_t)v);
             if (sizes.empty())
                 sizes.assign(nd.outputs.size(), xd[ax] / (int)nd.outputs.size());
+            int64_t sum = 0;
+            for (int64_t v : sizes)
+                sum += v < 1 ? (int64_t)1 << 40 : v;
+            if (sizes.size() != nd.outputs.size() || sum != xd[ax])
+                fail("Split: sizes that do not add up to the axis");
             Operator *sp = g->split(x, ax, std::vector<int>(sizes.begin(), sizes.end()));
             if (!sp)
                 fail("Split: the builder refused these sizes");
@@ -712,12 +782,15 @@ void build(Graph *g, Model &m) {
                     pads.push_back((int64_t)v);
             if (nd.gets("mode", "constant") != "constant" || (int)pads.size() != 2 * rank)
                 fail("Pad: constant mode with 2 * rank pads only");
+            for (int64_t v : pads)
+                if (v < 0 || v > (1 << 20))
+                    fail("Pad: a pad of " + std::to_string(v));
             out = resultOf(g->pad(x, Dim(pads.begin(), pads.begin() + rank),
                                   Dim(pads.begin() + rank, pads.end())));
         } else if (op == "Pow") {
             const Array &e = b.constant(nd.inputs.at(1));
             const double p = e.v.empty() ? -1 : e.v[0];
-            if (p != std::floor(p) || p < 0)
+            if (p != std::floor(p) || p < 0 || p > 64)
                 fail("Pow with a non-integer exponent");
             out = resultOf(g->pow(x, (int)p));
         } else {
@@ -745,6 +818,7 @@ bool GraphBase::importOnnx(const char *net) {
                                   std::istreambuf_iterator<char>());
         Model m = parse(data);
         foldBatchnorm(m);
+        InvalidOperandsThrow guard; // operands a builder rejects: a message, not an abort
         build(g, m);
     } catch (const std::exception &e) {
         std::fprintf(stderr, "[pet] importOnnx(%s): %s\n", net, e.what());

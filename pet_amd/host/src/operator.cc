@@ -2,8 +2,25 @@
 #include "perf_engine.h"
 
 #include <algorithm>
+#include <stdexcept>
+#include <string>
 
 namespace tpm {
+
+// The constructors assert the validity of their operands, as the reference's do. A front end
+// that builds operators from a file it does not control (Graph::importOnnx) asks for an
+// exception instead for the duration of its work.
+thread_local int invalidOperandsThrow = 0;
+InvalidOperandsThrow::InvalidOperandsThrow() { ++invalidOperandsThrow; }
+InvalidOperandsThrow::~InvalidOperandsThrow() { --invalidOperandsThrow; }
+#define PET_OPERANDS_VALID(cond)                                                               \
+    do {                                                                                       \
+        if (!(cond)) {                                                                         \
+            if (invalidOperandsThrow)                                                          \
+                throw std::invalid_argument(std::string(__func__) + ": operands it rejects");  \
+            assert(cond);                                                                      \
+        }                                                                                      \
+    } while (0)
 
 // ---- Operator base ------------------------------------------------------------
 
@@ -180,7 +197,7 @@ ConvOp::ConvOp(Tensor *input, Tensor *weight, Tensor *output, int ph, int pw, in
     : Operator(Conv, {input, weight}, {output}), ph(ph), pw(pw), sh(sh), sw(sw), dh(dh), dw(dw),
       bias(bias), act(act), padding(Other) {
     weight->setType(Tensor::Weight);
-    assert(checkValid({input, weight}));
+    PET_OPERANDS_VALID(checkValid({input, weight}));
     computeShape();
     setPaddingMode();
     initHash();
@@ -202,7 +219,7 @@ ConvOp::ConvOp(Tensor *input, Tensor *weight, Tensor *output, PaddingMode pm, in
       act(act), padding(pm) {
     assert(pm != Other);
     weight->setType(Tensor::Weight);
-    assert(checkValid({input, weight}));
+    PET_OPERANDS_VALID(checkValid({input, weight}));
     computeShape();
     initHash();
 }
@@ -414,7 +431,7 @@ ConvTransOp::ConvTransOp(Tensor *input, Tensor *weight, Tensor *output, int ph, 
     : Operator(ConvTrans, {input, weight}, {output}), ph(ph), pw(pw), sh(sh), sw(sw), dh(dh),
       dw(dw), oph(oph), opw(opw), bias(bias), act(act), padding(Other) {
     weight->setType(Tensor::Weight);
-    assert(checkValid({input, weight}));
+    PET_OPERANDS_VALID(checkValid({input, weight}));
     computeShape();
     setPaddingMode();
     initHash();
@@ -439,7 +456,7 @@ ConvTransOp::ConvTransOp(Tensor *input, Tensor *weight, Tensor *output, PaddingM
     : Operator(ConvTrans, {input, weight}, {output}), sh(sh), sw(sw), dh(dh), dw(dw), oph(oph),
       opw(opw), bias(bias), act(act), padding(pm) {
     weight->setType(Tensor::Weight);
-    assert(checkValid({input, weight}));
+    PET_OPERANDS_VALID(checkValid({input, weight}));
     computeShape();
     initHash();
 }
@@ -572,7 +589,7 @@ Conv3dOp::Conv3dOp(Tensor *input, Tensor *weight, Tensor *output, const Dim &pad
     : Operator(Conv3d, {input, weight}, {output}), pad(pad), stride(stride), dilation(dilation),
       bias(bias), act(act) {
     weight->setType(Tensor::Weight);
-    assert(checkValid({input, weight}));
+    PET_OPERANDS_VALID(checkValid({input, weight}));
     computeShape();
     initHash();
 }
@@ -731,7 +748,7 @@ MatmulOp::MatmulOp(Tensor *A, Tensor *B, Tensor *C, bool transA, bool transB, Te
     dimExtend(B);
     dimExtend(C);
     markWeight(A, B);
-    assert(checkValid({A, B}));
+    PET_OPERANDS_VALID(checkValid({A, B}));
     if (C->getDims().empty())
         computeShape();
     initHash();
@@ -900,7 +917,7 @@ std::string MatmulOp::toString() const {
 
 PadOp::PadOp(Tensor *input, Tensor *output, const Dim &begin, const Dim &end)
     : Operator(Pad, {input}, {output}), begin(begin), end(end) {
-    assert(checkValid({input}));
+    PET_OPERANDS_VALID(checkValid({input}));
     computeShape();
     initHash();
 }
@@ -949,7 +966,7 @@ std::string PadOp::toString() const {
 
 SliceOp::SliceOp(Tensor *input, Tensor *output, const Dim &begin, const Dim &end)
     : Operator(Slice, {input}, {output}), begin(begin), end(end) {
-    assert(checkValid({input}));
+    PET_OPERANDS_VALID(checkValid({input}));
     computeShape();
     initHash();
 }
@@ -1222,7 +1239,7 @@ TransposeOp::TransposeOp(Tensor *input, Tensor *output, const Perm &before, cons
             split = (int)i;
             break;
         }
-    assert(checkValid({input}));
+    PET_OPERANDS_VALID(checkValid({input}));
     initHash();
     computeShape();
 }
@@ -1233,7 +1250,7 @@ TransposeOp::TransposeOp(Tensor *input, Tensor *output, int split, const Perm &a
       factor(factor), trans_type(trans_type) {
     initHash();
     setParam((int)input->getDims().size());
-    assert(checkValid({input}));
+    PET_OPERANDS_VALID(checkValid({input}));
     computeShape();
 }
 
@@ -1490,7 +1507,7 @@ std::string ExtendOp::toString() const {
 
 EltwiseOp::EltwiseOp(OpType type, TensorVec ins, Tensor *output)
     : Operator(type, std::move(ins), {output ? output : new Tensor()}) {
-    assert(checkValid(inputs));
+    PET_OPERANDS_VALID(checkValid(inputs));
     if (outputs[0]->getDims().empty())
         computeShape();
     initHash();
@@ -1555,7 +1572,7 @@ std::string EltwiseOp::toString() const {
 // ---- Pow / BatchNorm ------------------------------------------------------------------
 
 PowOp::PowOp(Tensor *input, Tensor *output, int pow) : Operator(Pow, {input}, {output}), pow(pow) {
-    assert(checkValid(inputs));
+    PET_OPERANDS_VALID(checkValid(inputs));
     computeShape();
     initHash();
 }
@@ -1585,7 +1602,7 @@ BatchNormOp::BatchNormOp(Tensor *input, Tensor *scale, Tensor *bias, Tensor *mea
                          Tensor *output, float epsilon, float momentum)
     : Operator(BatchNorm, {input}, {output}), epsilon(epsilon), momentum(momentum), scale(scale),
       bias(bias), mean(mean), var(var) {
-    assert(checkValid(inputs));
+    PET_OPERANDS_VALID(checkValid(inputs));
     computeShape();
     initHash();
 }
@@ -1642,7 +1659,7 @@ std::string BatchNormOp::toString() const {
 
 GatherOp::GatherOp(Tensor *data, Tensor *indices, Tensor *output, int axis)
     : Operator(Gather, {data, indices}, {output}), axis(axis) {
-    assert(checkValid(inputs));
+    PET_OPERANDS_VALID(checkValid(inputs));
     computeShape();
     initHash();
 }
@@ -1692,7 +1709,7 @@ std::string GatherOp::toString() const {
 
 ReduceMeanOp::ReduceMeanOp(Tensor *input, Tensor *output, int axis)
     : Operator(ReduceMean, {input}, {output}), axis(axis) {
-    assert(checkValid(inputs));
+    PET_OPERANDS_VALID(checkValid(inputs));
     computeShape();
     initHash();
 }
@@ -1767,7 +1784,7 @@ PoolOp::PoolOp(OpType type, Tensor *input, Tensor *output, int kh, int kw, int d
                int pw, int sh, int sw)
     : Operator(type, {input}, {output}), kh(kh), kw(kw), dh(dh), dw(dw), ph(ph), pw(pw), sh(sh),
       sw(sw) {
-    assert(checkValid({input}));
+    PET_OPERANDS_VALID(checkValid({input}));
     computeShape();
     initHash();
 }
@@ -1832,7 +1849,7 @@ std::string PoolOp::toString() const {
 
 SoftmaxOp::SoftmaxOp(Tensor *input, Tensor *output, int axis)
     : Operator(Softmax, {input}, {output}), axis(axis) {
-    assert(checkValid({input}));
+    PET_OPERANDS_VALID(checkValid({input}));
     computeShape();
     initHash();
 }
@@ -1935,7 +1952,7 @@ G2BMMOp::G2BMMOp(Tensor *A, Tensor *B, Tensor *C, int width, int dilation, Tenso
     : Operator(G2BMM, {A, B}, {C}), width(width), dilation(dilation), bias(bias), act(act) {
     if (A->getType() == Tensor::Input && B->getType() == Tensor::Input)
         B->setType(Tensor::Weight);
-    assert(checkValid({A, B}));
+    PET_OPERANDS_VALID(checkValid({A, B}));
     computeShape();
     initHash();
 }
@@ -2021,7 +2038,7 @@ GBMMLOp::GBMMLOp(Tensor *A, Tensor *B, Tensor *C, int dilation, Tensor *bias, Ac
     : Operator(GBMML, {A, B}, {C}), dilation(dilation), bias(bias), act(act) {
     // both operands stay inputs: in attention neither is a constant
     // (src/Graph/operator.cc:1489-1493)
-    assert(checkValid({A, B}));
+    PET_OPERANDS_VALID(checkValid({A, B}));
     computeShape();
     initHash();
 }
