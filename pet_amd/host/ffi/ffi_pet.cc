@@ -56,6 +56,11 @@ void setTensorData(Tensor &t, py::array_t<float, py::array::c_style | py::array:
 
 PYBIND11_MODULE(cpp_module, m) {
     m.doc() = "PET host layer on the MI355X backend";
+    // From Python, operands a constructor rejects are a ValueError (pybind11 translates
+    // std::invalid_argument), not the assertion that ends a C++ program: in force on the
+    // importing thread for as long as the module lives.
+    static InvalidOperandsThrow *operandErrors = new InvalidOperandsThrow();
+    (void)operandErrors;
 
     py::class_<Tensor>(m, "Tensor")
         .def("getDims", [](const Tensor &t) { return t.getDims(); })

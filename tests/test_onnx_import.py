@@ -477,3 +477,19 @@ def test_native_importer_survives_damaged_files(tmp_path):
         assert res.returncode in (0, 2), (trial, res.returncode, res.stderr[-300:])
         outcomes[res.returncode] += 1
     assert outcomes[2] > 20 and outcomes[0] > 20, outcomes
+
+
+def test_operands_a_builder_rejects_are_a_python_error():
+    """The operator constructors assert on invalid operands, as the reference's do; through the
+    Python module that is a ValueError (a C++ assertion would end the interpreter)."""
+    from pet_amd import onnx_import
+    cm = onnx_import._module()
+    g = cm.Graph()
+    x, w = g.tensor([1, 3, 8, 8], "FLOAT"), g.tensor([4, 5, 3, 3], "FLOAT")
+    w.setWeight()
+    with pytest.raises(ValueError):
+        g.conv(x, w, 1, 1, 1, 1, 1, 1, None)      # 3 input channels, filters over 5
+    with pytest.raises(ValueError):                # the same through a model file
+        onnx_import.load(ow.model([ow.node("Conv", ["x", "w"], ["y"], pads=[1, 1, 1, 1])],
+                                  {"w": np.zeros((4, 5, 3, 3), np.float32)},
+                                  [("x", [1, 3, 8, 8])], [("y", [1, 4, 8, 8])]))
