@@ -200,7 +200,9 @@ PYBIND11_MODULE(cpp_module, m) {
         .def("setOutputs", &Graph::setOutputs)
         .def("getOperators", [](Graph &g) { return g.getOperators(); }, kRef)
         .def("getTensors", [](Graph &g) { return g.getTensors(); }, kRef)
-        .def("updateConnection", &Graph::updateConnection);
+        .def("updateConnection", &Graph::updateConnection)
+        .def("importOnnx", [](Graph &g, const std::string &path) { return g.importOnnx(path.c_str()); })
+        .def("exportOnnx", [](Graph &g, const std::string &path) { return g.exportOnnx(path.c_str()); });
 
     // dynamic attributes: Python code parks the Graph a SubGraph was cut from on it (the
     // SubGraph's operators keep pointing at that Graph's bias-like side tensors)
@@ -211,6 +213,8 @@ PYBIND11_MODULE(cpp_module, m) {
         .def("getOutputs", [](SubGraph &g) { return g.getOutputs(); }, kRef)
         .def("getOperators", [](SubGraph &g) { return g.getOperators(); }, kRef)
         .def("compute", py::overload_cast<>(&SubGraph::compute))
+        .def("exportOnnx",
+             [](SubGraph &g, const std::string &path) { return g.exportOnnx(path.c_str()); })
         .def("verification", &SubGraph::verification, "mutant"_a, "isFullComputing"_a = true)
         .def("perf",
              [](SubGraph &g, std::shared_ptr<PerfEngine> pe, bool withPenalty) {

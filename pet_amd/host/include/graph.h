@@ -39,10 +39,10 @@ class GraphBase {
     // Operators in a topological order (Kahn, ties in insertion order).
     bool topoOrder(OpVec &order) const;
     // The reference reads and writes model files through its embedded Python plug-in
-    // (src/Graph/graph.cc:1172-1187). Reading is native here (src/onnx_import.cc: the
-    // protobuf wire format read directly, one Graph builder call per node; false with a
-    // message on stderr for a file it cannot take; the object must be a Graph). Writing is
-    // not part of this backend: exportOnnx reports failure.
+    // (src/Graph/graph.cc:1172-1187). Both are native here, on the protobuf wire format
+    // directly: src/onnx_import.cc (one Graph builder call per node; the object must be a
+    // Graph) and src/onnx_export.cc (one or a few nodes per operator, weights written with
+    // their data). Each returns false with a message on stderr for what it cannot take.
     bool exportOnnx(const char *path);
     bool importOnnx(const char *net);
 };

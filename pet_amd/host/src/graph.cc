@@ -545,12 +545,6 @@ int SubGraph::getComputeOps(OpVec &out) {
 
 namespace tpm {
 
-bool GraphBase::exportOnnx(const char *path) {
-    std::fprintf(stderr, "[pet] exportOnnx(%s): model files are written by the Python side of "
-                         "this backend, not by the host layer\n", path ? path : "");
-    return false;
-}
-
 uint64_t SubGraph::getCacheIdx(int level) {
     static const uint64_t factors[8] = {10000019, 10000079, 10000103, 10000121,
                                         10000139, 10000141, 10000169, 10000189};

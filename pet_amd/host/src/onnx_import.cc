@@ -530,7 +530,7 @@ void build(Graph *g, Model &m) {
             // operands every form of the operator has
             static const std::map<std::string, size_t> kOperands = {
                 {"Conv", 2}, {"Add", 2}, {"Mul", 2}, {"Sub", 2}, {"Div", 2}, {"MatMul", 2},
-                {"Gemm", 2}, {"Gather", 2}, {"Reshape", 2}, {"Pow", 2},
+                {"Gemm", 2}, {"Gather", 2}, {"Reshape", 2}, {"Pow", 2}, {"Slice", 3},
                 {"BatchNormalization", 5}, {"LayerNormalization", 2}};
             auto need = kOperands.find(op);
             if (need != kOperands.end() && nd.inputs.size() < need->second)
@@ -787,6 +787,45 @@ void build(Graph *g, Model &m) {
                     fail("Pad: a pad of " + std::to_string(v));
             out = resultOf(g->pad(x, Dim(pads.begin(), pads.begin() + rank),
                                   Dim(pads.begin() + rank, pads.end())));
+        } else if (op == "Slice") {
+            // starts, ends, axes and steps as constants (opset 10 on); steps of 1 only
+            auto listOf = [&](size_t i) {
+                std::vector<double> v;
+                if (nd.inputs.size() > i && !nd.inputs[i].empty())
+                    v = b.constant(nd.inputs[i]).v;
+                return v;
+            };
+            const std::vector<double> starts = listOf(1), ends = listOf(2), steps = listOf(4);
+            std::vector<double> axes = listOf(3);
+            if (axes.empty())
+                for (size_t i = 0; i < starts.size(); ++i)
+                    axes.push_back((double)i);
+            if (starts.empty() || starts.size() != ends.size() || axes.size() != starts.size() ||
+                (int)starts.size() > rank)
+                fail("Slice: starts, ends and axes of different lengths");
+            for (double st : steps)
+                if (st != 1)
+                    fail("Slice with a step other than 1");
+            Dim begin(rank, 0), drop(rank, 0);
+            std::vector<bool> seen(rank, false);
+            for (size_t i = 0; i < axes.size(); ++i) {
+                if (axes[i] != std::floor(axes[i]) || axes[i] < -rank || axes[i] >= rank)
+                    fail("Slice: an axis out of range");
+                const int ax = axisOf((int64_t)axes[i]);
+                if (seen[ax])
+                    fail("Slice: an axis named twice");
+                seen[ax] = true;
+                const double n = xd[ax];
+                double lo = starts[i] < 0 ? starts[i] + n : starts[i];
+                double hi = ends[i] < 0 ? ends[i] + n : ends[i];
+                lo = std::min(std::max(lo, 0.0), n);
+                hi = std::min(std::max(hi, 0.0), n);
+                if (!(hi > lo))
+                    fail("Slice: an empty range");
+                begin[ax] = (int)lo;
+                drop[ax] = (int)(n - hi);
+            }
+            out = resultOf(g->slice(x, begin, drop));
         } else if (op == "Pow") {
             const Array &e = b.constant(nd.inputs.at(1));
             const double p = e.v.empty() ? -1 : e.v[0];

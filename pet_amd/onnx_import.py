@@ -448,6 +448,26 @@ def load(source, module=None, fold_bn=True):
                 raise ValueError("Pad: constant mode only")
             r = len(xd)
             out = g.pad(x, [int(p) for p in pads[:r]], [int(p) for p in pads[r:]]).getOutput()
+        elif op == "Slice":
+            lists = [np.asarray(const[n]).reshape(-1).tolist() if n else []
+                     for n in list(ins[1:5]) + [""] * (5 - len(ins))]
+            starts, ends, axes, steps = lists
+            axes = axes or list(range(len(starts)))
+            if not starts or not (len(starts) == len(ends) == len(axes)) or \
+                    len(set(int(ax) % len(xd) for ax in axes)) != len(axes):
+                raise ValueError("Slice: starts, ends and axes of different lengths")
+            if any(st != 1 for st in steps):
+                raise ValueError("Slice with a step other than 1")
+            begin, drop = [0] * len(xd), [0] * len(xd)
+            for lo, hi, ax in zip(starts, ends, axes):
+                ax = int(ax) % len(xd)
+                n = xd[ax]
+                lo = min(max(lo + n if lo < 0 else lo, 0), n)
+                hi = min(max(hi + n if hi < 0 else hi, 0), n)
+                if hi <= lo:
+                    raise ValueError("Slice: an empty range")
+                begin[ax], drop[ax] = int(lo), int(n - hi)
+            out = g.slice(x, begin, drop).getOutput()
         elif op == "Pow":
             p = float(np.asarray(const[ins[1]]).reshape(-1)[0])
             if p != int(p) or p < 0:

@@ -5,7 +5,10 @@
 //                                                 from raw float32, runs the graph on the
 //                                                 device (SubGraph::compute) and writes its
 //                                                 first output as raw float32
-// Exit code 2: the importer refused the file.
+//   onnx_driver <model.onnx> --export <out.onnx>  also writes the imported graph back with
+//                                                 GraphBase::exportOnnx (src/onnx_export.cc);
+//                                                 no device needed
+// Exit code 2: the importer refused the file; 3: the exporter refused the graph.
 #include "graph.h"
 #include "operator.h"
 #include "tensor.h"
@@ -13,13 +16,14 @@
 #include <cstdio>
 #include <fstream>
 #include <memory>
+#include <string>
 #include <vector>
 
 using namespace tpm;
 
 int main(int argc, char **argv) {
     if (argc != 2 && argc != 4) {
-        std::fprintf(stderr, "usage: %s model.onnx [in.bin out.bin]\n", argv[0]);
+        std::fprintf(stderr, "usage: %s model.onnx [in.bin out.bin | --export out.onnx]\n", argv[0]);
         return 1;
     }
     auto g = std::make_unique<Graph>();
@@ -40,6 +44,8 @@ int main(int argc, char **argv) {
     std::printf("operators: %zu\n", g->getOperators().size());
     if (argc == 2)
         return 0;
+    if (std::string(argv[2]) == "--export")
+        return g->exportOnnx(argv[3]) ? 0 : 3;
 
     // the whole model on the device
     TensorVec feeds;

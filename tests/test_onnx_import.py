@@ -344,6 +344,46 @@ def test_native_importer_builds_the_same_graphs(tmp_path):
     assert lines[-1].endswith("[1,1,1000]")
 
 
+def test_both_readers_take_slice_the_way_numpy_indexes(tmp_path):
+    """Slice (opset 10 on: starts / ends / axes / steps as constants): negative positions count
+    from the end, positions past the end are clamped, axes may be negative or left out."""
+    from pet_amd import onnx_import
+    shape = [2, 6, 9, 5]
+    probe = np.zeros(shape)
+    for starts, ends, axes, index in (
+            ([1, 2], [5, 2 ** 62], [1, 2], np.s_[:, 1:5, 2:, :]),
+            ([-4, 0], [-1, 3], [-2, -1], np.s_[:, :, -4:-1, 0:3]),
+            ([1, 0, 3, 2], [2, 6, 100, -1], None, np.s_[1:2, 0:6, 3:100, 2:-1])):
+        w = {"st": np.array(starts, dtype=np.int64), "en": np.array(ends, dtype=np.int64)}
+        ins = ["x", "st", "en"]
+        if axes is not None:
+            w["ax"] = np.array(axes, dtype=np.int64)
+            w["sp"] = np.ones(len(axes), dtype=np.int64)
+            ins += ["ax", "sp"]
+        want = probe[index].shape
+        data = ow.model([ow.node("Slice", ins, ["y"])], w, [("x", shape)], [("y", list(want))])
+        lo = [sl.indices(n)[0] for sl, n in zip(index, shape)]
+        drop = [n - sl.indices(n)[1] for sl, n in zip(index, shape)]
+        text = "Slice(begin=[%s],end=[%s])" % (",".join(map(str, lo)), ",".join(map(str, drop)))
+        m = onnx_import.load(data)
+        assert [op.toString() for op in m.graph.getOperators()] == [text]
+        assert tuple(m.tensors["y"].getDims()) == want
+        (tmp_path / "slice.onnx").write_bytes(data)
+        res = _driver(tmp_path / "slice.onnx")
+        assert res.returncode == 0, res.stderr
+        assert res.stdout.splitlines()[0] == text + "  -> [%s]" % ",".join(map(str, want))
+    for bad in ({"sp": np.array([2, 1], dtype=np.int64)}, {"en": np.array([1, 9], dtype=np.int64)}):
+        w = {"st": np.array([1, 2], dtype=np.int64), "en": np.array([5, 9], dtype=np.int64),
+             "ax": np.array([1, 2], dtype=np.int64), "sp": np.ones(2, dtype=np.int64)}
+        w.update(bad)
+        data = ow.model([ow.node("Slice", ["x", "st", "en", "ax", "sp"], ["y"])], w,
+                        [("x", shape)], [("y", shape)])
+        with pytest.raises(ValueError):
+            onnx_import.load(data)
+        (tmp_path / "slice.onnx").write_bytes(data)
+        assert _driver(tmp_path / "slice.onnx").returncode == 2
+
+
 def test_native_importer_refuses_what_it_cannot_take(tmp_path):
     bad = tmp_path / "einsum.onnx"
     bad.write_bytes(ow.model([ow.node("Einsum", ["x"], ["y"])], {}, [("x", [2, 2])], [("y", [2, 2])]))
@@ -407,6 +447,16 @@ def test_reference_import_programs_run_unchanged(program, tmp_path):
         return
     emitted = (tmp_path / "res.cu").read_text()
     assert emitted.count("pet_hip_conv2d") >= 2 and "pet_hip_softmax" in emitted
+    if program == "import_onnx":
+        # the program ends with bestGraph->exportOnnx("pet-optimization.onnx"): the file holds
+        # the optimised graph, or the exporter said on stderr which operator ONNX cannot say
+        written = tmp_path / "pet-optimization.onnx"
+        if "exportOnnx" in res.stderr:
+            assert "ONNX" in res.stderr and not written.exists()
+        else:
+            again = _driver(written)
+            assert again.returncode == 0, again.stderr[-1000:]
+            assert again.stdout.count("Conv") >= 2 and "Softmax" in again.stdout
 
 
 @pytest.mark.gpu
