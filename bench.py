@@ -70,6 +70,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--cpu-seconds", type=float, default=15.0)
+    ap.add_argument("--unfolded-layout", action="store_true",
+                    help="run space-to-batch and batch-to-space as launches of their own "
+                         "instead of as the neighbouring convolutions' addressing")
     ap.add_argument("--no-configs", action="store_true",
                     help="skip the latency table of the other four configurations")
     ap.add_argument("--config-only", default="", metavar="c1|c3|c4|c5[:pet]",
@@ -125,15 +128,34 @@ def main():
             fl |= _abi.X_RELU
         flags.append(fl)
 
+    # The two layout operators of the program are addressing modes of the convolutions next
+    # to them (pet_hip_conv2d_view_f32): the first convolution reads x through the strides of
+    # the space-to-batch Transpose, the last one writes through those of batch-to-space.
+    # --unfolded-layout keeps them as launches of their own.
+    folded = not args.unfolded_layout and \
+        ops.conv2d_view_supported((DIL * DIL, CHANNELS[0], hs, hs), tuple(ws[0].shape), 1, 1) and \
+        ops.conv2d_view_supported((DIL * DIL, CHANNELS[5], hs, hs), tuple(ws[5].shape), 1, 1)
+    view_in = ops.interleave_view(1, CHANNELS[0], hs, hs, DIL)
+    view_out = ops.interleave_view(1, CHANNELS[-1], hs, hs, DIL)
+    if folded and accum[5]:
+        fills[-1] = (t_out, None, 1, CHANNELS[-1], HW * HW)
+
     def optimised():
         if fills:
             ops.bias_fill_batch(fills)
-        ops.permute_flat(x, s2b_flat, s2b_perm, out=t_s2b)
-        cur = t_s2b
-        for i in range(6):
-            ops.conv2d(cur, ws[i], 1, 1, act="relu", out=t_act[i], flags=flags[i])
-            cur = t_act[i]
-        ops.permute_flat(cur, b2s_flat, b2s_perm, out=t_out)
+        if not folded:
+            ops.permute_flat(x, s2b_flat, s2b_perm, out=t_s2b)
+            cur = t_s2b
+            for i in range(6):
+                ops.conv2d(cur, ws[i], 1, 1, act="relu", out=t_act[i], flags=flags[i])
+                cur = t_act[i]
+            ops.permute_flat(cur, b2s_flat, b2s_perm, out=t_out)
+            return
+        ops.conv2d(x, ws[0], 1, 1, act="relu", out=t_act[0], flags=flags[0], x_view=view_in,
+                   x_shape=tuple(t_s2b.shape))
+        for i in range(1, 5):
+            ops.conv2d(t_act[i - 1], ws[i], 1, 1, act="relu", out=t_act[i], flags=flags[i])
+        ops.conv2d(t_act[4], ws[5], 1, 1, act="relu", out=t_out, flags=flags[5], y_view=view_out)
 
     def original():
         cur = x
@@ -276,6 +298,23 @@ def main():
     ms = time_kernel(lambda: ops.permute_flat(t_act[5], b2s_flat, b2s_perm, out=t_out))
     per_op.append({"op": "batch_to_space 4x64x32x32", "ms": ms, "GB/s": b2s_bytes / ms / 1e6,
                    "frac_hbm": b2s_bytes / ms / 1e6 / HBM_PEAK_GBS})
+    # the first and the last convolution as the timed program runs them: through the strides
+    # of the layout operator next to them
+    if folded:
+        fl = conv_flop(DIL * DIL, CHANNELS[1], hs, hs, CHANNELS[0], 3, 3)
+        ms = time_kernel(lambda: ops.conv2d(x, ws[0], 1, 1, act="relu", out=t_act[0],
+                                            x_view=view_in, x_shape=tuple(t_s2b.shape)))
+        per_op.append({"op": "conv3x3 %d->%d reading 1x%dx%dx%d through the space-to-batch "
+                             "strides" % (CHANNELS[0], CHANNELS[1], CHANNELS[0], HW, HW),
+                       "ms": ms, "TFLOP/s": fl / ms / 1e9,
+                       "frac_mfma": fl / ms / 1e9 / MFMA_FP32_PEAK_TFLOPS})
+        fl = conv_flop(DIL * DIL, CHANNELS[6], hs, hs, CHANNELS[5], 3, 3)
+        ms = time_kernel(lambda: ops.conv2d(t_act[4], ws[5], 1, 1, act="relu", out=t_out,
+                                            y_view=view_out))
+        per_op.append({"op": "conv3x3 %d->%d writing 1x%dx%dx%d through the batch-to-space "
+                             "strides" % (CHANNELS[5], CHANNELS[6], CHANNELS[6], HW, HW),
+                       "ms": ms, "TFLOP/s": fl / ms / 1e9,
+                       "frac_mfma": fl / ms / 1e9 / MFMA_FP32_PEAK_TFLOPS})
     # HBM-bound layout kernel at a size that cannot hide in cache: 1 GiB each way
     big = torch.empty((1, 4096, 256, 256), device=dev)
     big_out = torch.empty((4, 4096, 128, 128), device=dev)
@@ -586,12 +625,15 @@ def main():
         "config": {"workload": "dilated-conv block (CSRNet back-end), six 3x3 convs "
                                "512-512-512-512-256-128-64 on 1x512x64x64, PET space-to-batch "
                                "program (4x32x32 dense convs + fused ReLU, launches planned "
-                               "as the graph runtime plans them) as one HIP graph",
+                               "as the graph runtime plans them%s) as one HIP graph"
+                               % (", the two layout operators as the addressing of the first "
+                                  "and last convolution" if folded else ""),
                    "global_batch": 1},
         "value_is": "median of %d blocks of %d launches" % (REPEATS, args.steps),
         "block_ms_min": blocks[0],
         "block_ms_max": blocks[-1],
-        "planned_launches": {"accumulating_convs": [i + 1 for i in range(6) if accum[i]],
+        "planned_launches": {"layout_operators_folded": bool(folded),
+                             "accumulating_convs": [i + 1 for i in range(6) if accum[i]],
                              "batched_initialisations": len(fills)},
         "original_graph_ms": ms_org,
         "e2e_TFLOP/s": total_flop / ms_opt / 1e9,

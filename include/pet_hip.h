@@ -268,6 +268,37 @@ PET_HIP_API int pet_hip_conv3d_ex_f32(const float *x, const float *w, int w_is_p
                           int f, int kt, int r, int s, int pt, int ph, int pw, int st, int sh,
                           int sw, int dt, int dh, int dw, int groups, int act, unsigned flags,
                           pet_hip_stream_t stream);
+/* A 2-D convolution operand addressed through strides, all counted in floats: element
+ * (n, c, h, w) sits at n0 * n_stride[0] + n1 * n_stride[1] + n2 * n_stride[2] + c * c_stride +
+ * h * h_stride + w * w_stride, where the batch index is taken apart innermost first:
+ * n = (n2 * n_extent[1] + n1) * n_extent[0] + n0 (extent 1 for a factor that is not needed;
+ * the strides of factors of extent 1 are not looked at). The strides must visit every float
+ * of a dense buffer of n * c * h * w floats exactly once. */
+typedef struct pet_hip_conv_view {
+    long long c_stride, h_stride, w_stride;
+    int n_extent[2];
+    long long n_stride[3];
+} pet_hip_conv_view;
+
+/* pet_hip_conv2d_ex_f32 with x and / or y (and the residual, which is laid out like y) behind
+ * such strides; NULL for an operand in its usual layout. This is how a layout operator next
+ * to a convolution costs no launch: PET's space-to-batch Transpose in front of a convolution
+ * (src/Mutant/generator.cc, the dilated-to-dense mutation; TransposeOp::compute,
+ * src/Graph/operator.cc:2227-2245) is an x_view over the untransposed tensor, the
+ * batch-to-space Transpose behind one a y_view over its output. No counterpart upstream, where
+ * each Transpose is a kernel of its own. The sums are the ones pet_hip_conv2d_ex_f32 computes
+ * on the transposed copy, in the same order. PET_HIP_ERR_UNSUPPORTED, nothing written, for
+ * shapes outside pet_hip_conv2d_view_supported. */
+PET_HIP_API int pet_hip_conv2d_view_f32(const float *x, const pet_hip_conv_view *x_view, const float *w,
+                            const float *bias, const float *residual, float *y,
+                            const pet_hip_conv_view *y_view, int n, int c, int h, int wd, int f,
+                            int r, int s, int ph, int pw, int sh, int sw, int dh, int dw,
+                            int groups, int act, unsigned flags, pet_hip_stream_t stream);
+/* *yes = 1 when pet_hip_conv2d_view_f32 takes this shape (n, c, h, wd: the logical input):
+ * 3x3 filters over a multiple of 8 channels per group or 1x1 filters over a multiple of 32,
+ * operands below 2 GiB. */
+PET_HIP_API int pet_hip_conv2d_view_supported(int n, int c, int h, int wd, int f, int r, int s, int ph,
+                                  int pw, int sh, int sw, int dh, int dw, int groups, int *yes);
 /* *yes = 1 when a launch of this shape accumulates into y with atomics (and so starts
  * by writing bias into all of y, unless told that y is initialised). Depends on the
  * shape and on PET_HIP_DETERMINISTIC only. */

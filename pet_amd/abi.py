@@ -21,6 +21,14 @@ class Fill(ctypes.Structure):
     _fields_ = [("y", ctypes.c_void_p), ("bias", ctypes.c_void_p), ("outer", ctypes.c_size_t),
                 ("ch", ctypes.c_size_t), ("inner", ctypes.c_size_t)]
 
+class ConvView(ctypes.Structure):
+    """pet_hip_conv_view: strides, in floats, of a 2-D convolution operand; the batch index is
+    taken apart innermost first into n_extent[0], n_extent[1] and the rest."""
+    _fields_ = [("c_stride", ctypes.c_longlong), ("h_stride", ctypes.c_longlong),
+                ("w_stride", ctypes.c_longlong), ("n_extent", ctypes.c_int * 2),
+                ("n_stride", ctypes.c_longlong * 3)]
+
+
 _c_int_p = ctypes.POINTER(ctypes.c_int)
 _vp = ctypes.c_void_p
 _i = ctypes.c_int
@@ -62,6 +70,8 @@ SIGNATURES = {
     "pet_hip_conv2d_ex_f32": [_vp] * 5 + [_i] * 15 + [ctypes.c_uint, _vp],
     "pet_hip_conv3d_ex_f32": [_vp, _vp, _i, _vp, _vp, _vp] + [_i] * 20 + [ctypes.c_uint, _vp],
     "pet_hip_bmm_ex_f32": [_i] * 6 + [_vp] * 5 + [_i, ctypes.c_uint, _vp],
+    "pet_hip_conv2d_view_f32": [_vp] * 7 + [_i] * 15 + [ctypes.c_uint, _vp],
+    "pet_hip_conv2d_view_supported": [_i] * 14 + [_c_int_p],
     "pet_hip_conv2d_accumulates": [_i] * 14 + [_c_int_p],
     "pet_hip_conv3d_accumulates": [_i] * 20 + [_c_int_p],
     "pet_hip_bmm_accumulates": [_i] * 6 + [_c_int_p],

@@ -363,8 +363,12 @@ __global__ __launch_bounds__(Cfg::NT) void conv_plane_kernel(ConvParams p) {
     const int THW = p.T * p.H * p.W, HW = p.H * p.W;
     const int KRS = p.KT * RS; // weights per (f, c)
     // bases: the pad offset is folded into the image base so every voffset is >= 0
-    const int padoff = p.pt * HW + p.ph * p.W + p.pw;
-    const float *xg = p.x + (long long)g * p.cpg * THW - padoff;
+    // strides of a channel, a row and a column of x (a view brings its own; 2-D only)
+    const int xsc = p.xv.on ? (int)p.xv.sc : THW;
+    const int xsh = p.xv.on ? (int)p.xv.sh : p.W;
+    const int xsw = p.xv.on ? (int)p.xv.sw : 1;
+    const int padoff = p.pt * HW + p.ph * xsh + p.pw * xsw;
+    const float *xg = p.x + (long long)g * p.cpg * xsc - padoff;
     // floats per filter row as stored: all of K, or one kt slice of it when packed
     const int a_row = PACKED ? p.cpg * RS : p.K;
     const float *wg = p.w + (long long)g * p.M * a_row;
@@ -390,7 +394,8 @@ __global__ __launch_bounds__(Cfg::NT) void conv_plane_kernel(ConvParams p) {
             it0[pp] = (int)ot * p.st - p.pt;
             oh_[pp] = (int)oh * p.sh;
             ow_[pp] = (int)ow * p.sw;
-            pb[pp] = n * (unsigned)(p.C * THW) + ot * (unsigned)(p.st * HW) + oh_[pp] * p.W + ow_[pp];
+            pb[pp] = (p.xv.on ? view_batch_offset(p.xv, n) : n * (unsigned)(p.C * THW)) +
+                     ot * (unsigned)(p.st * HW) + oh_[pp] * xsh + ow_[pp] * xsw;
         }
         // Row i of wave w is row kl = w + NW * i of the B tile, i.e. channel kl / RS and
         // tap kl % RS: the four waves fetch neighbouring taps of one channel at the
@@ -416,7 +421,7 @@ __global__ __launch_bounds__(Cfg::NT) void conv_plane_kernel(ConvParams p) {
                 const int kl = WV + NW * i;
                 const int cl = kl / RS, t = kl % RS;
                 const int r = t / SW, s = t % SW;
-                const unsigned roff = (unsigned)(cl * THW + r * p.dh * p.W + s * p.dw);
+                const unsigned roff = (unsigned)(cl * xsc + r * p.dh * xsh + s * p.dw * xsw);
 #pragma unroll
                 for (int pp = 0; pp < PPL; ++pp)
                     voffB[i][pp] = (okr[pp][r] & okc[pp][s]) ? (pb[pp] + roff) * 4u : kOob;
@@ -498,7 +503,7 @@ __global__ __launch_bounds__(Cfg::NT) void conv_plane_kernel(ConvParams p) {
             }
         } else {
             const int row = i - NA;
-            const unsigned so = (unsigned)(pcb * CB * THW + pq * p.dt * HW) * 4u;
+            const unsigned so = (unsigned)(pcb * CB * xsc + pq * p.dt * HW) * 4u;
             const __amdgpu_buffer_rsrc_t rb = make_rsrc(xg);
 #pragma unroll
             for (int pp = 0; pp < PPL; ++pp) {
@@ -768,7 +773,15 @@ __global__ __launch_bounds__(Cfg::NT) void conv_plane_kernel(ConvParams p) {
             continue;
         unsigned n = fd_div(pix, p.fd_opix);
         unsigned rem = pix - n * p.OPIX;
-        const long long ybase = ((long long)n * p.F + (long long)g * p.M) * p.OPIX + rem;
+        // floats between two filters' outputs for this pixel, and where the first one goes
+        unsigned ysc = (unsigned)p.OPIX;
+        long long ybase = ((long long)n * p.F + (long long)g * p.M) * p.OPIX + rem;
+        if (p.yv.on) {
+            const unsigned oh = fd_div(rem, p.fd_ow);
+            ysc = p.yv.sc;
+            ybase = (long long)view_batch_offset(p.yv, n) + (long long)g * p.M * ysc +
+                    oh * p.yv.sh + (rem - oh * p.OW) * p.yv.sw;
+        }
         float *__restrict__ yb = p.y + ybase;
         const float *rb = p.res ? p.res + ybase : nullptr;
         const float *__restrict__ bias =
@@ -786,10 +799,10 @@ __global__ __launch_bounds__(Cfg::NT) void conv_plane_kernel(ConvParams p) {
                     if (f < p.M) {
                         float v = acc[tm][tn][r];
                         if (add_res) {
-                            const float rv = rb[(unsigned)f * (unsigned)p.OPIX];
+                            const float rv = rb[(unsigned)f * ysc];
                             v += p.res_relu ? fmaxf(rv, 0.f) : rv;
                         }
-                        unsafeAtomicAdd(yb + (unsigned)f * (unsigned)p.OPIX, v);
+                        unsafeAtomicAdd(yb + (unsigned)f * ysc, v);
                     }
                 }
         } else {
@@ -803,10 +816,10 @@ __global__ __launch_bounds__(Cfg::NT) void conv_plane_kernel(ConvParams p) {
                         if (bias)
                             v += bias[f];
                         if (rb) {
-                            const float rv = rb[(unsigned)f * (unsigned)p.OPIX];
+                            const float rv = rb[(unsigned)f * ysc];
                             v += p.res_relu ? fmaxf(rv, 0.f) : rv;
                         }
-                        yb[(unsigned)f * (unsigned)p.OPIX] = apply_act(v + colbias, p.act);
+                        yb[(unsigned)f * ysc] = apply_act(v + colbias, p.act);
                     }
                 }
         }
@@ -1082,7 +1095,8 @@ int launch_plane_cfg(ConvParams p, hipStream_t stream) {
     p.fd_splitk = make_fastdiv((unsigned)p.splitk);
     p.fd_mg = make_fastdiv((unsigned)p.xcd_mg);
     p.fd_band = make_fastdiv((unsigned)p.xcd_mg * grid.x);
-    p.vec_out = (p.OPIX % 4 == 0) && (((uintptr_t)p.y & 15) == 0) && (((uintptr_t)p.res & 15) == 0);
+    p.vec_out = (p.OPIX % 4 == 0) && (((uintptr_t)p.y & 15) == 0) &&
+                (((uintptr_t)p.res & 15) == 0) && !p.yv.on;
     if constexpr (has_streamk<Cfg>) {
         if (p.streamk) {
             grid = dim3(Cfg::BM * Cfg::BN >= 64 * 128 ? 256 : 512, 1, 1);
@@ -1138,13 +1152,18 @@ int try_launch_plane(const ConvParams &p, hipStream_t stream) {
     static const bool off = getenv("PET_HIP_PLANE") && atoi(getenv("PET_HIP_PLANE")) == 0;
     if (off)
         return -1;
-    const long long in_bytes = 4ll * p.N * p.C * p.T * p.H * p.W;
+    // voffsets count from the image base minus the pad offset
+    const long long in_bytes =
+        4ll * p.N * p.C * p.T * p.H * p.W +
+        (p.xv.on ? 4ll * ((long long)p.ph * p.xv.sh + (long long)p.pw * p.xv.sw) : 0);
     const long long w_bytes = 4ll * p.F * p.K;
     if (in_bytes >= (1ll << 31) || w_bytes >= (1ll << 31))
         return -1;
     if (((uintptr_t)p.w & 15) != 0 || p.w_shared || p.bias_gstride)
         return -1;
     const bool is3d = p.T > 1 || p.KT > 1 || p.pt > 0 || p.st > 1;
+    if (is3d && (p.xv.on || p.yv.on))
+        return -1;
     const int rs = p.R * p.S;
     if (rs == 9 && p.R == 3 && p.cpg % 8 == 0)
         return launch_plane<9, 8>(p, is3d, stream);
@@ -1179,6 +1198,11 @@ int launch_conv(ConvParams &p, hipStream_t stream) {
     rc = try_launch_plane(p, stream);
     if (rc >= 0)
         return rc;
+    if (p.xv.on || p.yv.on)
+        return set_error(PET_HIP_ERR_UNSUPPORTED,
+                         "strided operands are read by the kernels for 3x3 filters over a "
+                         "multiple of 8 channels and 1x1 filters over a multiple of 32 only "
+                         "(pet_hip_conv2d_view_supported would have said so)");
     if (p.wpacked)
         return set_error(PET_HIP_ERR_UNSUPPORTED,
                          "kt-major filters are only read by the plane kernel; this shape does "
@@ -1201,6 +1225,52 @@ int launch_conv(ConvParams &p, hipStream_t stream) {
     }
 }
 
+// Checks that the strides of a view visit every float of a dense buffer of n * c * h * w
+// floats once (sorted by stride, each factor starts where the ones below it end) and
+// copies them for the kernels.
+bool take_view(const pet_hip_conv_view &v, int n, int c, int h, int w, OperandView &out) {
+    const long long e0 = v.n_extent[0], e1 = v.n_extent[1];
+    if (e0 < 1 || e1 < 1 || e0 * e1 > n || n % (e0 * e1) != 0)
+        return false;
+    struct Factor {
+        long long ext, stride;
+    } fs[6] = {{e0, v.n_stride[0]}, {e1, v.n_stride[1]}, {n / (e0 * e1), v.n_stride[2]},
+               {c, v.c_stride},     {h, v.h_stride},     {w, v.w_stride}};
+    // factors that are stepped along, by stride; the others go last
+    std::sort(fs, fs + 6, [](const Factor &a, const Factor &b) {
+        return std::make_pair(a.ext == 1, a.stride) < std::make_pair(b.ext == 1, b.stride);
+    });
+    long long want = 1;
+    for (const Factor &f : fs) {
+        if (f.ext == 1)
+            continue; // never stepped along: its stride is not looked at
+        if (f.stride != want)
+            return false;
+        want *= f.ext;
+    }
+    out.on = 1;
+    out.sc = (unsigned)v.c_stride;
+    out.sh = (unsigned)v.h_stride;
+    out.sw = (unsigned)v.w_stride;
+    out.fd_ne0 = make_fastdiv((unsigned)e0);
+    out.fd_ne1 = make_fastdiv((unsigned)e1);
+    for (int i = 0; i < 3; ++i)
+        out.ns[i] = (unsigned)v.n_stride[i];
+    if (e0 == 1)
+        out.ns[0] = 0;
+    if (e1 == 1)
+        out.ns[1] = 0;
+    if (n == e0 * e1)
+        out.ns[2] = 0;
+    if (c == 1)
+        out.sc = 1; // multiplied by channel 0 only; also a divisor in the initialising launch
+    if (h == 1)
+        out.sh = 0;
+    if (w == 1)
+        out.sw = 0;
+    return true;
+}
+
 // Algorithm override (PET_HIP_CONV_ALGO, 0: the cost model decides): forced K shares per
 // tile and / or stream-K on or off.
 void apply_algo(ConvParams &p, unsigned algo) {
@@ -1213,7 +1283,9 @@ int conv_common(const float *x, const float *w, const float *bias, float *y, int
                 int h, int wd, int f, int kt, int r, int s, int pt, int ph, int pw, int st, int sh,
                 int sw, int dt, int dh, int dw, int groups, int act, hipStream_t stream,
                 bool wpacked = false, const float *res = nullptr, unsigned flags = 0,
-                int *dry = nullptr, bool static_ws = false) {
+                int *dry = nullptr, bool static_ws = false,
+                const pet_hip_conv_view *xview = nullptr,
+                const pet_hip_conv_view *yview = nullptr) {
     if (flags & ~(unsigned)(PET_HIP_CALL_Y_INITIALISED | PET_HIP_CALL_DEFER_RELU |
                             PET_HIP_CALL_X_RELU | PET_HIP_CALL_RES_RELU | 0xff00u))
         return set_error(PET_HIP_ERR_INVALID, "unknown call flags 0x%x", flags);
@@ -1295,6 +1367,17 @@ int conv_common(const float *x, const float *w, const float *bias, float *y, int
     p.defer_relu = (flags & PET_HIP_CALL_DEFER_RELU) != 0;
     p.dry_atomic = dry;
     p.static_ws = static_ws;
+    if (xview || yview) {
+        if (t != 1 || kt != 1 || pt != 0 || st != 1 || dt != 1)
+            return set_error(PET_HIP_ERR_INVALID, "strided operands are for 2-D convolutions");
+        if (xview && !take_view(*xview, n, c, h, wd, p.xv))
+            return set_error(PET_HIP_ERR_INVALID,
+                             "x_view does not address a dense [%d,%d,%d,%d] buffer", n, c, h, wd);
+        if (yview && !take_view(*yview, n, f, p.OH, p.OW, p.yv))
+            return set_error(PET_HIP_ERR_INVALID,
+                             "y_view does not address a dense [%d,%d,%d,%d] buffer", n, f, p.OH,
+                             p.OW);
+    }
     if (((flags >> 8) & 0xffu) >= PET_HIP_CONV_ALGO_COUNT)
         return set_error(PET_HIP_ERR_INVALID, "unknown convolution algorithm %u",
                          (flags >> 8) & 0xffu);
@@ -1381,7 +1464,10 @@ int launch_accumulate_init(const ConvParams &p, hipStream_t stream) {
     const size_t total = (size_t)p.NPIX * p.F;
     unsigned igrid = (unsigned)std::min<size_t>((total + 255) / 256, 4096);
     hipLaunchKernelGGL(splitk_init_kernel, dim3(igrid), dim3(256), 0, stream, p.y, p.bias, p.res,
-                       p.res_relu, p.bias_mode, (unsigned)p.F, (unsigned)p.OPIX, total);
+                       p.res_relu, p.bias_mode, (unsigned)p.F,
+                       // floats per channel run: a viewed y is a dense buffer whose channel
+                       // factor has this stride
+                       p.yv.on ? p.yv.sc : (unsigned)p.OPIX, total);
     return check_launch("splitk_init_kernel");
 }
 
@@ -1452,6 +1538,38 @@ int pet_hip_conv3d_ex_f32(const float *x, const float *w, int w_is_packed, const
     PET_REQUIRE_INIT();
     return conv_common(x, w, bias, y, n, c, t, h, wd, f, kt, r, s, pt, ph, pw, st, sh, sw, dt, dh,
                        dw, groups, act, as_stream(stream), w_is_packed != 0, residual, flags);
+}
+
+int pet_hip_conv2d_view_f32(const float *x, const pet_hip_conv_view *x_view, const float *w,
+                            const float *bias, const float *residual, float *y,
+                            const pet_hip_conv_view *y_view, int n, int c, int h, int wd, int f,
+                            int r, int s, int ph, int pw, int sh, int sw, int dh, int dw,
+                            int groups, int act, unsigned flags, pet_hip_stream_t stream) {
+    PET_REQUIRE_INIT();
+    return conv_common(x, w, bias, y, n, c, 1, h, wd, f, 1, r, s, 0, ph, pw, 1, sh, sw, 1, dh, dw,
+                       groups, act, as_stream(stream), false, residual, flags, nullptr, false,
+                       x_view, y_view);
+}
+
+int pet_hip_conv2d_view_supported(int n, int c, int h, int wd, int f, int r, int s, int ph, int pw,
+                                  int sh, int sw, int dh, int dw, int groups, int *yes) {
+    PET_REQUIRE_INIT();
+    if (!yes)
+        return set_error(PET_HIP_ERR_INVALID, "null result pointer");
+    // the shape with x in its usual layout, said as a view
+    pet_hip_conv_view plain;
+    plain.w_stride = 1;
+    plain.h_stride = wd;
+    plain.c_stride = (long long)h * wd;
+    plain.n_extent[0] = plain.n_extent[1] = 1;
+    plain.n_stride[0] = plain.n_stride[1] = 0;
+    plain.n_stride[2] = (long long)c * h * wd;
+    int accumulates = 0;
+    const int rc = conv_common(nullptr, nullptr, nullptr, nullptr, n, c, 1, h, wd, f, 1, r, s, 0, ph,
+                               pw, 1, sh, sw, 1, dh, dw, groups, PET_HIP_ACT_NONE, nullptr, false,
+                               nullptr, 0, &accumulates, false, &plain, nullptr);
+    *yes = rc == PET_HIP_OK;
+    return rc == PET_HIP_ERR_UNSUPPORTED ? PET_HIP_OK : rc;
 }
 
 int pet_hip_conv2d_accumulates(int n, int c, int h, int wd, int f, int r, int s, int ph, int pw,

@@ -6,7 +6,26 @@
 namespace pet {
 namespace mfma {
 
+// A 2-D operand read or written through strides (pet_hip_conv2d_view_f32): element
+// (n, c, h, w) sits at batch(n) + c * sc + h * sh + w * sw floats from the base, where the
+// batch index is taken apart into three factors, innermost first (extents ne0, ne1 and the
+// rest), each with a stride of its own. A layout operator next to the convolution (space to
+// batch in front, batch to space behind) becomes this addressing.
+struct OperandView {
+    int on;
+    unsigned sc, sh, sw;
+    unsigned ns[3];
+    FastDiv fd_ne0, fd_ne1;
+};
+
+__device__ __forceinline__ unsigned view_batch_offset(const OperandView &v, unsigned n) {
+    const unsigned q0 = fd_div(n, v.fd_ne0);
+    const unsigned q1 = fd_div(q0, v.fd_ne1);
+    return (n - q0 * v.fd_ne0.d) * v.ns[0] + (q0 - q1 * v.fd_ne1.d) * v.ns[1] + q1 * v.ns[2];
+}
+
 struct ConvParams {
+    OperandView xv, yv; // plane and direct kernels, 2-D only; the residual is laid out like y
     const float *x, *w, *bias;
     const float *res; // optional residual, laid out like y: y = act(conv + bias + res)
     float *y;

@@ -69,6 +69,10 @@ __global__ __launch_bounds__(Cfg::NT) void conv_direct_kernel(ConvParams p) {
     const int m0 = blockIdx.y * (32 * TM);
     const int n0 = blockIdx.x * (32 * TN);
     const int HW = p.H * p.W;
+    // strides of a channel, a row and a column of x (a view brings its own)
+    const int xsc = p.xv.on ? (int)p.xv.sc : HW;
+    const int xsh = p.xv.on ? (int)p.xv.sh : p.W;
+    const int xsw = p.xv.on ? (int)p.xv.sw : 1;
 
     // this wave's share of the K chunks: share ks * KW + wave of splitk * KW
     const int nchunks = p.cpg / CB;
@@ -87,18 +91,19 @@ __global__ __launch_bounds__(Cfg::NT) void conv_direct_kernel(ConvParams p) {
         const unsigned oh = fd_div(rem, p.fd_ow);
         const unsigned ow = rem - oh * p.OW;
         const int ih0 = (int)oh * p.sh, iw0 = (int)ow * p.sw;
-        const unsigned pb = n * (unsigned)(p.C * HW) + ih0 * p.W + iw0 + hk * (CH * HW);
+        const unsigned pb = (p.xv.on ? view_batch_offset(p.xv, n) : n * (unsigned)(p.C * HW)) +
+                            ih0 * xsh + iw0 * xsw + hk * (CH * xsc);
 #pragma unroll
         for (int r = 0; r < SR; ++r)
 #pragma unroll
             for (int s = 0; s < SW; ++s) {
                 const bool ok = (unsigned)(ih0 + r * p.dh - p.ph) < (unsigned)p.H &&
                                 (unsigned)(iw0 + s * p.dw - p.pw) < (unsigned)p.W;
-                voffB[tn][r * SW + s] = ok ? (pb + r * p.dh * p.W + s * p.dw) * 4u : kOob;
+                voffB[tn][r * SW + s] = ok ? (pb + r * p.dh * xsh + s * p.dw * xsw) * 4u : kOob;
             }
     }
-    const int padoff = p.ph * p.W + p.pw;
-    const __amdgpu_buffer_rsrc_t rb = make_rsrc(p.x + (long long)g * p.cpg * HW - padoff);
+    const int padoff = p.ph * xsh + p.pw * xsw;
+    const __amdgpu_buffer_rsrc_t rb = make_rsrc(p.x + (long long)g * p.cpg * xsc - padoff);
     // ---- and of the A tile: word i = q * 64 + lane is row i / PPR, floats 4 * (i % PPR) ..
     unsigned voffA[TM][NQ];
     int parkA[NQ]; // where that word is parked in the wave's LDS region (floats)
@@ -158,7 +163,7 @@ __global__ __launch_bounds__(Cfg::NT) void conv_direct_kernel(ConvParams p) {
     };
     auto load_b = [&](int j, int chunk) __attribute__((always_inline)) {
         const int cj = j / RS, t = j % RS; // channel inside the half-chunk, tap
-        const unsigned so = (unsigned)((chunk * CB + cj) * HW) * 4u;
+        const unsigned so = (unsigned)((chunk * CB + cj) * xsc) * 4u;
 #pragma unroll
         for (int tn = 0; tn < TN; ++tn)
             b[tn][j] = __uint_as_float(__builtin_amdgcn_raw_buffer_load_b32(rb, voffB[tn][t], so, 0));
@@ -229,7 +234,12 @@ __global__ __launch_bounds__(Cfg::NT) void conv_direct_kernel(ConvParams p) {
             continue;
         const unsigned n = fd_div(pix, p.fd_opix);
         const unsigned rem = pix - n * p.OPIX;
-        const long long yi = ((long long)n * p.F + (long long)g * p.M + f) * p.OPIX + rem;
+        long long yi = ((long long)n * p.F + (long long)g * p.M + f) * p.OPIX + rem;
+        if (p.yv.on) {
+            const unsigned oh = fd_div(rem, p.fd_ow);
+            yi = (long long)view_batch_offset(p.yv, n) + ((long long)g * p.M + f) * p.yv.sc +
+                 oh * p.yv.sh + (rem - oh * p.OW) * p.yv.sw;
+        }
         if (p.atomic_out) {
             // y was initialised (bias, residual) before this launch; activation after it
             if (p.res_first && ks == 0) {

@@ -33,11 +33,57 @@ def conv_out_dim(i, k, p, s, d):
     return (i - (k - s) * d + 2 * p) // s if (i - (k - s) * d + 2 * p) >= 0 else -1
 
 
+def interleave_view(q, c, hb, wb, d):
+    """The strides under which a [q, c, d*hb, d*wb] tensor is the batch [(i, j, q), c, hb, wb]
+    of its d*d pixel phases, entry (i*d + j)*q + image holding the pixels (d*y + i, d*x + j):
+    PET's space-to-batch Transpose when the tensor is read, batch-to-space when written."""
+    v = abi.ConvView()
+    v.c_stride, v.h_stride, v.w_stride = d * hb * d * wb, d * d * wb, d
+    v.n_extent[0], v.n_extent[1] = q, d
+    v.n_stride[0], v.n_stride[1], v.n_stride[2] = c * d * hb * d * wb, 1, d * wb
+    return v
+
+
+def conv2d_view_supported(x_shape, w_shape, ph, pw, sh=1, sw=1, dh=1, dw=1):
+    """Whether conv2d takes x_view / y_view for these (logical) shapes."""
+    abi.init(torch.cuda.current_device())
+    n, c, h, wd = x_shape
+    f, cpg, r, s = w_shape
+    yes = ctypes.c_int(0)
+    abi.call("pet_hip_conv2d_view_supported", n, c, h, wd, f, r, s, ph, pw, sh, sw, dh, dw,
+             c // cpg, ctypes.byref(yes))
+    return bool(yes.value)
+
+
 def conv2d(x, w, ph, pw, sh=1, sw=1, dh=1, dw=1, bias=None, act="none", out=None,
-           residual=None, flags=0):
+           residual=None, flags=0, x_view=None, x_shape=None, y_view=None):
     """act(conv(x, w) + bias + residual); residual has the output's shape. flags:
-    pet_hip_call_flags (abi.Y_INITIALISED, DEFER_RELU, X_RELU, RES_RELU)."""
+    pet_hip_call_flags (abi.Y_INITIALISED, DEFER_RELU, X_RELU, RES_RELU). x_view / y_view
+    (abi.ConvView): x is read, y (and the residual) written through these strides, x_shape
+    being the logical [n, c, h, w] of x and `out` a buffer of the output's size."""
     _chk(x, w, bias, out, residual)
+    if x_view is not None or y_view is not None:
+        n, c, h, wd = x_shape if x_view is not None else x.shape
+        f, cpg, r, s = w.shape
+        if cpg <= 0 or c % cpg:
+            raise abi.PetHipError(1, "input channels not divisible by weight channels")
+        oh, ow = conv_out_dim(h, r, ph, sh, dh), conv_out_dim(wd, s, pw, sw, dw)
+        if x.numel() != n * c * h * wd:
+            raise abi.PetHipError(1, "x does not hold the viewed shape")
+        if out is None:
+            if y_view is not None:
+                raise abi.PetHipError(1, "a viewed output needs its buffer")
+            out = torch.empty((n, f, max(oh, 0), max(ow, 0)), device=x.device,
+                              dtype=torch.float32)
+        if out.numel() != n * f * max(oh, 0) * max(ow, 0) or \
+                (residual is not None and residual.numel() != out.numel()):
+            raise abi.PetHipError(1, "output or residual of another size")
+        abi.call("pet_hip_conv2d_view_f32", _ptr(x),
+                 ctypes.byref(x_view) if x_view is not None else None, _ptr(w), _ptr(bias),
+                 _ptr(residual), _ptr(out), ctypes.byref(y_view) if y_view is not None else None,
+                 n, c, h, wd, f, r, s, ph, pw, sh, sw, dh, dw, c // cpg, abi.ACT[act], flags,
+                 _stream())
+        return out
     n, c, h, wd = x.shape
     f, cpg, r, s = w.shape
     if cpg <= 0 or c % cpg:
