@@ -221,6 +221,10 @@ class ConvOp : public Operator {
     int launch(pet_hip_stream_t stream) override;
     int launchFused(pet_hip_stream_t stream, const float *residual, ActType finalAct,
                     float *out, unsigned flags = 0) override;
+    // The same convolution with x read and / or y written through strides (NULL: the usual
+    // layout): a row of Transposes next to it folded into its addressing by the graph runtime.
+    int launchView(pet_hip_stream_t stream, const float *x, const pet_hip_conv_view *xView,
+                   float *y, const pet_hip_conv_view *yView, unsigned flags);
     bool accumulates() const override;
     bool canTakeResidual() const override { return act == None; }
     std::string toString() const override;

@@ -462,6 +462,225 @@ int launchChain(const std::vector<TransposeOp *> &row, pet_hip_stream_t s) {
                                prog.perms.data(), outDims, &outRank, s);
 }
 
+// ---- layout operators as the addressing of the convolution next to them ----------
+//
+// A row of Transposes without correction parameters only regroups and reorders extents: every
+// dim of its output is a run of factors, each with a stride in the row's input and one in its
+// output. When the row feeds one 2-D convolution and channel, height and width of the
+// convolution's input are single factors, the convolution reads the row's input through those
+// strides (pet_hip_conv2d_view_f32) and the row is never launched; likewise a row behind a
+// convolution, read the other way round, gives the strides the convolution writes through.
+// PET's space-to-batch / batch-to-space pair around dilated convolutions is the case in point.
+struct ViewFactor {
+    long long ext, in, out;
+    int src; // dim of the row's input the factor is cut from
+};
+
+bool chainFactors(const TransProgram &prog, std::vector<std::vector<ViewFactor>> &dims) {
+    const int rank = (int)prog.inDims.size();
+    dims.assign(rank, {});
+    long long stride = 1;
+    for (int i = rank - 1; i >= 0; --i) {
+        if (prog.inDims[i] <= 0)
+            return false;
+        dims[i].push_back({prog.inDims[i], stride, 0, i});
+        stride *= prog.inDims[i];
+    }
+    size_t pp = 0;
+    for (int o = 0; o < prog.nops; ++o) {
+        const int *op = &prog.ops[6 * o];
+        if (op[0] == 0) { // split of dim op[1] into (rest, op[2])
+            if (op[3] != 0 || op[4] != 0)
+                return false;
+            std::vector<ViewFactor> &outer = dims[op[1]], inner;
+            long long have = 1, need = op[2];
+            for (auto &f : outer)
+                have *= f.ext;
+            if (need <= 0 || have % need != 0)
+                return false;
+            while (need > 1) {
+                if (outer.empty())
+                    return false;
+                ViewFactor last = outer.back();
+                if (last.ext <= need) {
+                    if (need % last.ext != 0)
+                        return false;
+                    inner.insert(inner.begin(), last);
+                    need /= last.ext;
+                    outer.pop_back();
+                } else {
+                    if (last.ext % need != 0)
+                        return false;
+                    inner.insert(inner.begin(), {need, last.in, 0, last.src});
+                    outer.back() = {last.ext / need, last.in * need, 0, last.src};
+                    need = 1;
+                }
+            }
+            dims.insert(dims.begin() + op[1] + 1, inner);
+        } else if (op[0] == 1) {
+            std::vector<std::vector<ViewFactor>> moved(dims.size());
+            for (size_t i = 0; i < dims.size(); ++i)
+                moved[i] = dims[prog.perms[pp + i]];
+            pp += dims.size();
+            dims.swap(moved);
+        } else {
+            if (op[2] != 0 || op[3] != 0 || op[1] + 1 >= (int)dims.size())
+                return false;
+            std::vector<ViewFactor> &head = dims[op[1]], &tail = dims[op[1] + 1];
+            head.insert(head.end(), tail.begin(), tail.end());
+            dims.erase(dims.begin() + op[1] + 1);
+        }
+    }
+    stride = 1;
+    for (int i = (int)dims.size() - 1; i >= 0; --i)
+        for (int j = (int)dims[i].size() - 1; j >= 0; --j) {
+            dims[i][j].out = stride;
+            stride *= dims[i][j].ext;
+        }
+    for (auto &d : dims) // factors of extent 1 are never stepped along
+        d.erase(std::remove_if(d.begin(), d.end(), [](const ViewFactor &f) { return f.ext == 1; }),
+                d.end());
+    return true;
+}
+
+// (batch factors outermost first, channel, height, width) -> the C structure; `use_out`
+// picks the strides in the row's output instead of its input
+bool makeView(const std::vector<ViewFactor> &n, const std::vector<ViewFactor> &c,
+              const std::vector<ViewFactor> &h, const std::vector<ViewFactor> &w, bool use_out,
+              pet_hip_conv_view &v) {
+    if (n.size() > 3 || c.size() > 1 || h.size() > 1 || w.size() > 1)
+        return false;
+    auto st = [&](const ViewFactor &f) { return use_out ? f.out : f.in; };
+    v.c_stride = c.empty() ? 0 : st(c[0]);
+    v.h_stride = h.empty() ? 0 : st(h[0]);
+    v.w_stride = w.empty() ? 0 : st(w[0]);
+    v.n_extent[0] = v.n_extent[1] = 1;
+    v.n_stride[0] = v.n_stride[1] = v.n_stride[2] = 0;
+    // innermost first; the outermost factor takes the third place, whose extent is implied
+    std::vector<ViewFactor> in(n.rbegin(), n.rend());
+    if (!in.empty()) {
+        v.n_stride[2] = st(in.back());
+        in.pop_back();
+    }
+    for (size_t i = 0; i < in.size(); ++i) {
+        v.n_extent[i] = (int)in[i].ext;
+        v.n_stride[i] = st(in[i]);
+    }
+    return true;
+}
+
+struct ConvView {
+    bool hasX = false, hasY = false;
+    pet_hip_conv_view x, y;
+    Tensor *src = nullptr; // what the convolution reads instead of its input
+    Tensor *dst = nullptr; // what it writes instead of its output
+};
+
+struct ConvViews {
+    std::map<const Operator *, ConvView> byConv;
+    std::set<const Operator *> folded;    // Transposes that never launch
+    std::set<const Tensor *> notThere;    // tensors that are never written
+};
+
+ConvViews planConvViews(const OpVec &order, const TensorVec &graphOutputs,
+                        const std::set<const Operator *> &skipped, const TransposeChains &rows,
+                        const std::set<const Operator *> &taken) {
+    ConvViews plan;
+    static const bool off = getenv("PET_HOST_NO_CONV_VIEWS") != nullptr ||
+                            getenv("PET_HOST_NO_LAUNCH_FUSION") != nullptr;
+    if (off)
+        return plan;
+    std::set<const Tensor *> outs(graphOutputs.begin(), graphOutputs.end());
+    auto supported = [](ConvOp *conv) {
+        auto d = conv->getInputs()[0]->getDims(), w = conv->getInputs()[1]->getDims();
+        int yes = 0;
+        if (w[1] <= 0 || d[1] % w[1] != 0)
+            return false;
+        return pet_hip_conv2d_view_supported(d[0], d[1], d[2], d[3], w[0], w[2], w[3],
+                                             conv->getPh(), conv->getPw(), conv->getSh(),
+                                             conv->getSw(), conv->getDh(), conv->getDw(),
+                                             d[1] / w[1], &yes) == PET_HIP_OK &&
+               yes != 0;
+    };
+    for (auto op : order) {
+        auto last = dynamic_cast<TransposeOp *>(op);
+        if (!last || skipped.count(op) || rows.folded.count(op) || taken.count(op) || weightOnly(op))
+            continue;
+        std::vector<TransposeOp *> row = {last};
+        if (rows.chains.count(op))
+            row = rows.chains.at(op);
+        bool free = true;
+        for (auto tr : row)
+            free = free && !taken.count(tr) && !plan.folded.count(tr);
+        TransProgram prog;
+        std::vector<std::vector<ViewFactor>> dims;
+        if (!free || !lowerChain(row, prog) || !chainFactors(prog, dims))
+            continue;
+        Tensor *in = row.front()->getInputs()[0], *out = last->getOutputs()[0];
+        // in front of a convolution: the row's output is that convolution's input and nothing else
+        const OpVec &users = out->getInputOf();
+        auto reader = users.size() == 1 ? dynamic_cast<ConvOp *>(users[0]) : nullptr;
+        if (reader && !outs.count(out) && reader->getInputs()[0] == out &&
+            reader->getInputs()[1] != out && !skipped.count(reader) && !taken.count(reader) &&
+            !plan.byConv[reader].hasX && dims.size() == 4 && supported(reader)) {
+            ConvView &cv = plan.byConv[reader];
+            if (makeView(dims[0], dims[1], dims[2], dims[3], false, cv.x)) {
+                cv.hasX = true;
+                cv.src = in;
+                for (auto tr : row) {
+                    plan.folded.insert(tr);
+                    plan.notThere.insert(tr->getOutputs()[0]);
+                }
+                continue;
+            }
+        }
+        // behind a convolution: the row's input is that convolution's output, read by the row only
+        auto writer = dynamic_cast<ConvOp *>(in->getOutputOf());
+        if (writer && !outs.count(in) && in->getInputOf().size() == 1 && !skipped.count(writer) &&
+            !taken.count(writer) && !plan.byConv[writer].hasY && prog.inDims.size() == 4 &&
+            supported(writer)) {
+            std::vector<std::vector<ViewFactor>> bySrc(4);
+            for (auto &d : dims)
+                for (auto &f : d)
+                    bySrc[f.src].push_back(f);
+            for (auto &d : bySrc)
+                std::sort(d.begin(), d.end(),
+                          [](const ViewFactor &a, const ViewFactor &b) { return a.in > b.in; });
+            ConvView &cv = plan.byConv[writer];
+            if (makeView(bySrc[0], bySrc[1], bySrc[2], bySrc[3], true, cv.y)) {
+                cv.hasY = true;
+                cv.dst = out;
+                plan.notThere.insert(in);
+                for (auto tr : row) {
+                    plan.folded.insert(tr);
+                    if (tr != last)
+                        plan.notThere.insert(tr->getOutputs()[0]);
+                }
+            }
+        }
+    }
+    for (auto it = plan.byConv.begin(); it != plan.byConv.end();)
+        it = (it->second.hasX || it->second.hasY) ? std::next(it) : plan.byConv.erase(it);
+    return plan;
+}
+
+// A fill planned for the output of a convolution that writes through strides moves to the
+// buffer it writes: dense, with the channel factor's stride as the run per channel.
+void retargetFills(LaunchPlan &lp, const ConvViews &views) {
+    for (auto &cvp : views.byConv) {
+        const ConvView &cv = cvp.second;
+        if (!cv.hasY)
+            continue;
+        Tensor *own = const_cast<Operator *>(cvp.first)->getOutputs()[0];
+        for (auto &f : lp.fills)
+            if (f.out == own) {
+                f.out = cv.dst;
+                f.inner = cv.y.c_stride > 0 ? (size_t)cv.y.c_stride : 1;
+                f.outer = cv.dst->size() / (f.ch * f.inner);
+            }
+    }
+}
+
 } // namespace
 
 // A Matmul whose lhs is one [1, m, k] tensor stacked b times on dim 0 (an Extend, or a Concat
@@ -690,6 +909,14 @@ std::unique_ptr<GraphExec> CodeEngine::instantiate(std::shared_ptr<SubGraph> &gr
                                     [](const Tensor *) { return true; });
     for (auto &f : relus.flags)
         lp.flags[f.first] |= f.second;
+    // what another plan already runs its own way
+    std::set<const Operator *> taken(att.absorbed.begin(), att.absorbed.end());
+    taken.insert(relus.folded.begin(), relus.folded.end());
+    taken.insert(tails.absorbed.begin(), tails.absorbed.end());
+    for (auto &t : tails.atAdd)
+        taken.insert(t.second.contraction);
+    ConvViews views = planConvViews(order, graph->getOutputs(), plan.skipped, rows, taken);
+    retargetFills(lp, views);
     auto flagsOf = [&](const Operator *op) {
         auto it = lp.flags.find(op);
         return it == lp.flags.end() ? 0u : it->second;
@@ -698,6 +925,14 @@ std::unique_ptr<GraphExec> CodeEngine::instantiate(std::shared_ptr<SubGraph> &gr
         auto fa = att.atMerge.find(op);
         if (fa != att.atMerge.end())
             return launchAttention(fa->second, st);
+        auto cv = views.byConv.find(op);
+        if (cv != views.byConv.end()) {
+            const ConvView &v = cv->second;
+            return static_cast<ConvOp *>(op)->launchView(
+                st, (v.hasX ? v.src : op->getInputs()[0])->devicePtr(), v.hasX ? &v.x : nullptr,
+                (v.hasY ? v.dst : op->getOutputs()[0])->devicePtr(), v.hasY ? &v.y : nullptr,
+                flagsOf(op));
+        }
         auto tail = tails.atAdd.find(op);
         if (tail != tails.atAdd.end()) {
             const FusedTail &f = tail->second;
@@ -752,7 +987,7 @@ std::unique_ptr<GraphExec> CodeEngine::instantiate(std::shared_ptr<SubGraph> &gr
         if (weightOnly(op))
             continue;
         if (rows.folded.count(op) || tails.absorbed.count(op) || att.absorbed.count(op) ||
-            relus.folded.count(op)) {
+            relus.folded.count(op) || views.folded.count(op)) {
             exec->nFoldedOps++;
             continue;
         }
@@ -780,7 +1015,7 @@ std::unique_ptr<GraphExec> CodeEngine::instantiate(std::shared_ptr<SubGraph> &gr
             if (tail != tails.atAdd.end() && tail->second.out != t)
                 inside = true;
             if (inside || lp.preAct.count(t) || att.absorbed.count(prod) || stacked.count(prod) ||
-                relus.folded.count(prod))
+                relus.folded.count(prod) || views.notThere.count(t))
                 continue; // not there, or there without its ReLU
             t->deviceWritten();
             t->setComputed();
@@ -949,9 +1184,22 @@ std::string CodeEngine::genCode(std::shared_ptr<SubGraph> &graph) {
                                     [](const Tensor *) { return true; });
     for (auto &f : relus.flags)
         lp.flags[f.first] |= f.second;
+    std::set<const Operator *> taken(att.absorbed.begin(), att.absorbed.end()); // as instantiate()
+    taken.insert(tails.absorbed.begin(), tails.absorbed.end());
+    for (auto &t : tails.atAdd)
+        taken.insert(t.second.contraction);
+    ConvViews views = planConvViews(order, graph->getOutputs(), skipped, rows, taken);
+    retargetFills(lp, views);
     auto flagsOf = [&](const Operator *op) {
         auto it = lp.flags.find(op);
         return it == lp.flags.end() ? 0u : it->second;
+    };
+    auto viewText = [](const pet_hip_conv_view &v) {
+        std::ostringstream t;
+        t << "{" << v.c_stride << ", " << v.h_stride << ", " << v.w_stride << ", {"
+          << v.n_extent[0] << ", " << v.n_extent[1] << "}, {" << v.n_stride[0] << ", "
+          << v.n_stride[1] << ", " << v.n_stride[2] << "}}";
+        return t.str();
     };
     // set while a contraction is emitted in place of the Add that follows it
     const FusedTail *tail = nullptr;
@@ -977,6 +1225,26 @@ std::string CodeEngine::genCode(std::shared_ptr<SubGraph> &graph) {
               << e.name(f.v) << ", " << e.name(f.out) << ", 1, " << f.heads << ", " << f.seq << ", "
               << f.dh << ", " << ld << ", " << ld << ", " << ld << ", " << ld
               << ", 0, 0, 0, 0, 1.0f, " << nullable(e, f.scale) << ", s)";
+        } else if (views.byConv.count(op)) {
+            // the Transposes next to this convolution are its addressing
+            auto conv = static_cast<ConvOp *>(op);
+            const ConvView &v = views.byConv.at(op);
+            auto d = op->getInputs()[0]->getDims(), w = op->getInputs()[1]->getDims();
+            const std::string id = std::to_string(op->getGuid());
+            if (v.hasX)
+                e.line("    static const pet_hip_conv_view xv" + id + " = " + viewText(v.x) + ";");
+            if (v.hasY)
+                e.line("    static const pet_hip_conv_view yv" + id + " = " + viewText(v.y) + ";");
+            c << "pet_hip_conv2d_view_f32(" << (v.hasX ? e.name(v.src) : in(0)) << ", "
+              << (v.hasX ? "&xv" + id : std::string("nullptr")) << ", " << in(1) << ", "
+              << nullable(e, conv->getBias()) << ", nullptr, "
+              << (v.hasY ? e.name(v.dst) : out(0)) << ", "
+              << (v.hasY ? "&yv" + id : std::string("nullptr")) << ", " << d[0] << ", " << d[1]
+              << ", " << d[2] << ", " << d[3] << ", " << w[0] << ", " << w[2] << ", " << w[3] << ", "
+              << conv->getPh() << ", " << conv->getPw() << ", " << conv->getSh() << ", "
+              << conv->getSw() << ", " << conv->getDh() << ", " << conv->getDw() << ", "
+              << d[1] / w[1] << ", " << (int)conv->getAct() << ", "
+              << (flagsOf(op) | PET_HIP_CONV_ALGO(conv->getAlgo())) << "u, s)";
         } else if (auto conv = dynamic_cast<ConvOp *>(op)) {
             auto d = op->getInputs()[0]->getDims(), w = op->getInputs()[1]->getDims();
             const unsigned fl = flagsOf(op) | PET_HIP_CONV_ALGO(conv->getAlgo());
@@ -1244,7 +1512,8 @@ std::string CodeEngine::genCode(std::shared_ptr<SubGraph> &graph) {
     }
     for (auto op : order)
         if (!weightOnly(op) && !skipped.count(op) && !rows.folded.count(op) &&
-            !tails.absorbed.count(op) && !att.absorbed.count(op) && !emitOp(op))
+            !tails.absorbed.count(op) && !att.absorbed.count(op) && !views.folded.count(op) &&
+            !emitOp(op))
             return "";
     e.line("    pet_hip_graph_t g; CHECK(pet_hip_graph_end_capture(s, &g));");
     e.line("    pet_hip_event_t st, ed; CHECK(pet_hip_event_create(&st)); "

@@ -342,6 +342,18 @@ int ConvOp::launchFused(pet_hip_stream_t stream, const float *residual, ActType 
                                  (int)finalAct, flags | PET_HIP_CONV_ALGO(algo), stream);
 }
 
+int ConvOp::launchView(pet_hip_stream_t stream, const float *x, const pet_hip_conv_view *xView,
+                       float *y, const pet_hip_conv_view *yView, unsigned flags) {
+    auto in = inputs[0]->getDims(), wt = inputs[1]->getDims();
+    int groups = in[1] / wt[1];
+    if (groups <= 0 || wt[0] % groups != 0)
+        return PET_HIP_ERR_INVALID;
+    return pet_hip_conv2d_view_f32(x, xView, inputs[1]->devicePtr(),
+                                   bias ? bias->devicePtr() : nullptr, nullptr, y, yView, in[0],
+                                   in[1], in[2], in[3], wt[0], wt[2], wt[3], ph, pw, sh, sw, dh, dw,
+                                   groups, (int)act, flags | PET_HIP_CONV_ALGO(algo), stream);
+}
+
 bool ConvOp::accumulates() const {
     auto in = inputs[0]->getDims(), wt = inputs[1]->getDims();
     int groups = wt[1] > 0 ? in[1] / wt[1] : 0, yes = 0;
